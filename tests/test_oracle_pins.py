@@ -1,0 +1,395 @@
+"""Pins the CPU oracle against things that do not share its code: library routines,
+closed forms, brute force on tiny inputs and invariants.  The reference ships no
+tests, golden vectors or fixtures for this path, so these checks are what anchors
+the oracle; each one is chosen so that a plausible slip (dropped weight, wrong
+sign, swapped sin/cos, transposed index) fails it."""
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import llsa_oracle as O
+
+torch.manual_seed(0)
+
+
+# ----------------------------------------------------------------------------- Z-order
+def _zorder_recursive(side):
+    if side == 1:
+        return [[0]]
+    h = side // 2
+    sub = _zorder_recursive(h)
+    out = [[0] * side for _ in range(side)]
+    for qr in range(2):
+        for qc in range(2):
+            base = (qr * 2 + qc) * h * h            # quadrants in order TL, TR, BL, BR
+            for r in range(h):
+                for c in range(h):
+                    out[qr * h + r][qc * h + c] = base + sub[r][c]
+    return out
+
+
+@pytest.mark.parametrize("side", [2, 4, 8, 16, 32, 64])
+def test_zorder_matches_quadrant_recursion(side):
+    perm, inv = O.zorder_perm(side)
+    ref = torch.tensor(_zorder_recursive(side)).flatten()
+    assert torch.equal(perm, ref)
+    assert torch.equal(perm[inv], torch.arange(side * side))
+    assert torch.equal(inv[perm], torch.arange(side * side))
+
+
+def test_zorder_base_case_and_patches():
+    perm, inv = O.zorder_perm(2)
+    assert perm.tolist() == [0, 1, 2, 3]
+    perm, inv = O.zorder_perm(16)
+    # 16 consecutive Z-ordered tokens form a 4x4 pixel patch, 256 a 16x16 patch
+    for blk in range(16):
+        ras = inv[blk * 16:(blk + 1) * 16]
+        r, c = ras // 16, ras % 16
+        assert r.max() - r.min() == 3 and c.max() - c.min() == 3
+        assert r.min() % 4 == 0 and c.min() % 4 == 0
+    # second token of the order is the right neighbour, third is the pixel below
+    assert inv[1] == 1 and inv[2] == 16
+
+
+# ----------------------------------------------------------------------------- RoPE
+def test_rope_table_closed_form_entries():
+    side = 8
+    tab = O.rope_table(side, (32, 32), 10000.0, torch.float64, zorder=False)
+    assert tab.shape == (64, 64)
+    for (r, c, j) in [(0, 0, 0), (3, 5, 0), (7, 1, 4), (2, 6, 15)]:
+        w = 10000.0 ** (-2.0 * j / 32)
+        row = tab[r * side + c]
+        assert row[2 * j].item() == pytest.approx(math.sin(r * w), abs=1e-12)
+        assert row[2 * j + 1].item() == pytest.approx(math.cos(r * w), abs=1e-12)
+        assert row[32 + 2 * j].item() == pytest.approx(math.sin(c * w), abs=1e-12)
+        assert row[32 + 2 * j + 1].item() == pytest.approx(math.cos(c * w), abs=1e-12)
+    # Z-ordered table is the raster table indexed by inv_perm
+    _, inv = O.zorder_perm(side)
+    assert torch.equal(O.rope_table(side, dtype=torch.float64), tab[inv])
+
+
+def test_rope_apply_is_complex_multiplication():
+    side = 8
+    tab = O.rope_table(side, dtype=torch.float64)
+    x = torch.randn(2, 3, 64, 64, dtype=torch.float64)
+    y = O.rope_apply(x, tab)
+    xc = torch.view_as_complex(x.reshape(2, 3, 64, 32, 2).contiguous())
+    rot = torch.complex(tab[:, 1::2], tab[:, 0::2])          # cos + i sin
+    yc = torch.view_as_real(xc * rot).reshape(2, 3, 64, 64)
+    assert torch.allclose(y, yc, atol=1e-12)
+    # orthogonal: norms kept, backward is the inverse
+    assert torch.allclose(y.norm(dim=-1), x.norm(dim=-1), atol=1e-10)
+    assert torch.allclose(O.rope_apply_bwd(y, tab), x, atol=1e-10)
+    # backward is the transpose of forward: <R x, g> == <x, R^T g>
+    g = torch.randn_like(x)
+    assert torch.allclose((y * g).sum(), (x * O.rope_apply_bwd(g, tab)).sum(), atol=1e-8)
+
+
+def test_rope_relative_position_property():
+    side = 16
+    tab = O.rope_table(side, dtype=torch.float64, zorder=False).reshape(side, side, 64)
+    q = torch.randn(64, dtype=torch.float64)
+    k = torch.randn(64, dtype=torch.float64)
+
+    def dot(pq, pk):
+        a = O.rope_apply(q.view(1, 1, 1, 64), tab[pq[0], pq[1]].view(1, 64))
+        b = O.rope_apply(k.view(1, 1, 1, 64), tab[pk[0], pk[1]].view(1, 64))
+        return (a * b).sum().item()
+
+    assert dot((3, 4), (1, 9)) == pytest.approx(dot((5, 6), (3, 11)), abs=1e-9)
+    assert dot((3, 4), (1, 9)) != pytest.approx(dot((3, 4), (2, 9)), abs=1e-6)
+
+
+def test_rope_bf16_rounds_every_op():
+    tab = O.rope_table(4, dtype=torch.bfloat16)
+    x = torch.randn(1, 1, 16, 64).bfloat16()
+    y = O.rope_apply(x, tab)
+    # scalar re-computation of a few entries with explicit roundings
+    for (s, p) in [(0, 0), (5, 3), (15, 31), (9, 17)]:
+        sin, cos = tab[s, 2 * p], tab[s, 2 * p + 1]
+        xe, xo = x[0, 0, s, 2 * p], x[0, 0, s, 2 * p + 1]
+        ye = ((cos.float() * xe.float()).bfloat16().float() - (sin.float() * xo.float()).bfloat16().float()).bfloat16()
+        yo = ((sin.float() * xe.float()).bfloat16().float() + (cos.float() * xo.float()).bfloat16().float()).bfloat16()
+        assert y[0, 0, s, 2 * p] == ye and y[0, 0, s, 2 * p + 1] == yo
+
+
+# ----------------------------------------------------------------------------- pooling
+def test_pool_fp32_is_avg_pool1d():
+    x = torch.randn(2, 3, 64, 8)
+    y = O.mean_pool(x, 16)
+    ref = F.avg_pool1d(x.reshape(6, 64, 8).transpose(1, 2), 16).transpose(1, 2).reshape(2, 3, 4, 8)
+    assert torch.allclose(y, ref, atol=1e-6)
+
+
+def test_pool_bf16_sequential_rounding_bruteforce():
+    x = (torch.randn(1, 1, 32, 4) * 3).bfloat16()
+    y = O.mean_pool(x, 16)
+    for s in range(2):
+        for c in range(4):
+            acc = torch.tensor(0.0).bfloat16()
+            for t in range(16):
+                acc = (acc.float() + x[0, 0, s * 16 + t, c].float()).bfloat16()
+            assert y[0, 0, s, c] == (acc.float() / 16).bfloat16()
+    # and it really differs from a one-shot fp32 mean somewhere on a larger input
+    xl = (torch.randn(1, 1, 16 * 64, 64) * 3).bfloat16()
+    assert not torch.equal(O.mean_pool(xl, 16), xl.float().reshape(1, 1, 64, 16, 64).mean(3).bfloat16())
+
+
+def test_pool_bwd_is_autograd_of_avg_pool():
+    x = torch.randn(1, 2, 32, 4, requires_grad=True)
+    dy = torch.randn(1, 2, 2, 4)
+    F.avg_pool1d(x.reshape(2, 32, 4).transpose(1, 2), 16).transpose(1, 2).reshape(1, 2, 2, 4).backward(dy)
+    assert torch.allclose(O.mean_pool_bwd(dy, 16), x.grad, atol=1e-7)
+
+
+# ----------------------------------------------------------------------------- selection
+def test_dense_selection_matches_bruteforce_fp32():
+    pq, pk = torch.randn(1, 2, 32, 16), torch.randn(1, 2, 32, 16)
+    idx = O.gen_sparse_indices(pq, pk, 4)
+    assert idx.dtype == torch.int64 and idx.shape == (1, 2, 32, 4)
+    for h in range(2):
+        for m in range(32):
+            sc = [(float(pq[0, h, m] @ pk[0, h, n]), n) for n in range(32)]
+            sc.sort(key=lambda t: -t[0])
+            assert idx[0, h, m].tolist() == [n for _, n in sc[:4]]
+    # scores are NOT scaled by 1/sqrt(D) and use pq . pk (not pk . pk): permuting pk rows permutes indices
+    perm = torch.randperm(32)
+    idx_p = O.gen_sparse_indices(pq, pk[:, :, perm], 4)
+    assert torch.equal(perm[idx_p], idx)
+    # k larger than the row length is clamped (topk.py:8)
+    assert O.gen_sparse_indices(pq, pk, 64).shape[-1] == 32
+
+
+def test_topk_lowest_index_tie_rule():
+    s = torch.tensor([[1.0, 3.0, 3.0, 2.0, 3.0, 0.0]])
+    assert O.topk_lowest_index(s, 4).tolist() == [[1, 2, 4, 3]]
+    gi = torch.tensor([[50, 40, 30, 20, 10, 0]])
+    assert O.topk_lowest_index(s, 4, gi).tolist() == [[10, 30, 40, 20]]
+
+
+def test_topk_sparse_bruteforce_with_ties():
+    B, H, N1, D, T, T2, bs = 1, 2, 64, 8, 4, 2, 16
+    pq = torch.randn(B, H, N1, D).bfloat16()
+    pk = torch.randn(B, H, N1, D).bfloat16()
+    pk[0, 0, 5] = pk[0, 0, 37]                          # forced exact ties
+    pk[0, 1, 20] = pk[0, 1, 21]
+    N2 = N1 // bs
+    p_idx = torch.stack([torch.stack([torch.randperm(N2)[:T2] for _ in range(N2)]) for _ in range(H)])[None]
+    out = O.topk_sparse(pq, pk, p_idx, T, bs)
+    assert out.dtype == torch.int32 and out.shape == (B, H, N1, T)
+    for h in range(H):
+        for g in range(N1):
+            G = g // bs
+            cands = [int(p_idx[0, h, G, a]) * bs + b for a in range(T2) for b in range(bs)]
+            sc = [(-float((pq[0, h, g].float() * pk[0, h, c].float()).sum()), c) for c in cands]
+            sc.sort()                                    # descending score, then ascending index
+            assert out[0, h, g].tolist() == [c for _, c in sc[:T]]
+
+
+# ----------------------------------------------------------------------------- transpose
+def test_transpose_indices_bruteforce():
+    B, H, Mb, T = 2, 2, 32, 4
+    idx = torch.stack([torch.randperm(Mb)[:T] for _ in range(B * H * Mb)]).reshape(B, H, Mb, T)
+    off, flat = O.transpose_indices(idx)
+    assert off.shape == (B, H, Mb + 1) and flat.shape == (B, H, Mb * T)
+    assert (off[..., 0] == 0).all() and (off[..., -1] == Mb * T).all()
+    for b in range(B):
+        for h in range(H):
+            for n in range(Mb):
+                want = sorted(g for g in range(Mb) if n in idx[b, h, g].tolist())
+                assert flat[b, h, off[b, h, n]:off[b, h, n + 1]].tolist() == want
+    # rectangular: key-block count different from query-block count
+    idx2 = torch.randint(0, 8, (1, 1, 16, 1))
+    off2, flat2 = O.transpose_indices(idx2, 8)
+    assert off2.shape == (1, 1, 9)
+    for n in range(8):
+        assert flat2[0, 0, off2[0, 0, n]:off2[0, 0, n + 1]].tolist() == [g for g in range(16) if idx2[0, 0, g, 0] == n]
+
+
+# ----------------------------------------------------------------------------- forward
+def _rand_problem(B, H, N, D, T, dtype, T2=None, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    q, k, v = (torch.randn(B, H, N, D, generator=g).to(dtype) for _ in range(3))
+    pk, pv = O.mean_pool(k), O.mean_pool(v)
+    N1 = N // 16
+    if T2 is None:
+        idx = torch.stack([torch.randperm(N1, generator=g)[:T] for _ in range(B * H * N1)]).reshape(B, H, N1, T)
+        return q, k, v, pk, pv, idx
+    pk2, pv2 = O.mean_pool(pk), O.mean_pool(pv)
+    N2 = N1 // 16
+    pidx = torch.stack([torch.randperm(N2, generator=g)[:T2] for _ in range(B * H * N2)]).reshape(B, H, N2, T2)
+    idx = O.topk_sparse(O.mean_pool(q), pk, pidx, T)
+    return q, k, v, pk, pv, pk2, pv2, idx, pidx
+
+
+def test_forward_l1_matches_closed_form_fp32():
+    q, k, v, pk, pv, idx = _rand_problem(1, 2, 1024, 32, 8, torch.float32)
+    o, lse = O.attn_fwd_l1(q, k, v, pk, pv, idx, 16)
+    oc, lc = O.closed_form_l1(q.double(), k.double(), v.double(), pk.double(), pv.double(), idx, 16)
+    assert torch.allclose(o.double(), oc, atol=2e-5)
+    assert torch.allclose(lse.double(), lc, atol=2e-5)
+    # the weight matters: a wrong weight is far outside that tolerance
+    ow, _ = O.closed_form_l1(q.double(), k.double(), v.double(), pk.double(), pv.double(), idx, 1)
+    assert (ow - oc).abs().max() > 1e-2
+
+
+def test_forward_l1_explicit_formula_one_query():
+    """L_i = sum_fine e^s + w sum_coarse e^s, O_i = (sum_fine e^s v + w sum_coarse e^s pv) / L_i, by hand."""
+    q, k, v, pk, pv, idx = _rand_problem(1, 1, 1024, 16, 4, torch.float64, seed=3)
+    o, lse = O.attn_fwd_l1(q.float(), k.float(), v.float(), pk.float(), pv.float(), idx, 16)
+    i = 333
+    g = i // 16
+    toks = [int(b) * 16 + u for b in idx[0, 0, g] for u in range(16)]
+    es = torch.exp((k[0, 0, toks] @ q[0, 0, i]) / 4.0)
+    ec = torch.exp((pk[0, 0] @ q[0, 0, i]) / 4.0)
+    L = es.sum() + 16 * ec.sum()
+    oi = (es @ v[0, 0, toks] + 16 * (ec @ pv[0, 0])) / L
+    assert torch.allclose(o[0, 0, i].double(), oi, atol=1e-5)
+    assert lse[0, 0, i].item() == pytest.approx(math.log(L.item()), abs=1e-5)
+
+
+def test_forward_reduces_to_sdpa_when_all_blocks_selected_and_weight_zero():
+    B, H, N, D = 1, 2, 1024, 32
+    q, k, v = (torch.randn(B, H, N, D) for _ in range(3))
+    N1 = N // 16
+    idx = torch.stack([torch.randperm(N1) for _ in range(B * H * N1)]).reshape(B, H, N1, N1)
+    o, lse = O.attn_fwd_l1(q, k, v, O.mean_pool(k), O.mean_pool(v), idx, token_weight=0)
+    ref = F.scaled_dot_product_attention(q, k, v)
+    assert torch.allclose(o, ref, atol=2e-5)
+    assert torch.allclose(lse, torch.logsumexp(q @ k.transpose(-1, -2) / math.sqrt(D), -1), atol=2e-5)
+
+
+def test_forward_constant_v_and_equal_k():
+    q, k, v, pk, pv, pk2, pv2, idx, pidx = _rand_problem(1, 1, 4096 * 4, 16, 4, torch.float32, T2=4, seed=1)
+    vc = torch.ones_like(v) * 0.75
+    o, _ = O.attn_fwd_l2(q, k, vc, pk, O.mean_pool(vc), pk2, O.mean_pool(O.mean_pool(vc)), idx, pidx)
+    assert torch.allclose(o, vc, atol=1e-5)
+    # all keys equal: every logit equal, O = weighted mean with weights {1, 16, 256}
+    ke = torch.zeros_like(k)
+    pke, pk2e = O.mean_pool(ke), O.mean_pool(O.mean_pool(ke))
+    o, lse = O.attn_fwd_l2(q, ke, v, pke, pv, pk2e, pv2, idx, pidx)
+    g = 100
+    G = g // 16
+    fine = torch.cat([v[0, 0, int(b) * 16:int(b) * 16 + 16] for b in idx[0, 0, g]])
+    lvl1 = torch.cat([pv[0, 0, int(b) * 16:int(b) * 16 + 16] for b in pidx[0, 0, G]])
+    num = fine.sum(0) + 16 * lvl1.sum(0) + 256 * pv2[0, 0].sum(0)
+    den = fine.shape[0] + 16 * lvl1.shape[0] + 256 * pv2.shape[2]
+    assert torch.allclose(o[0, 0, g * 16 + 3], num / den, atol=1e-5)
+    assert lse[0, 0, g * 16 + 3].item() == pytest.approx(math.log(den), abs=1e-5)
+
+
+def test_forward_l2_matches_closed_form_and_is_index_order_invariant():
+    q, k, v, pk, pv, pk2, pv2, idx, pidx = _rand_problem(1, 1, 16384, 16, 8, torch.float32, T2=4, seed=2)
+    o, lse = O.attn_fwd_l2(q, k, v, pk, pv, pk2, pv2, idx, pidx)
+    args = [t.double() for t in (q, k, v, pk, pv, pk2, pv2)]
+    oc, lc = O.closed_form_l2(*args, idx, pidx)
+    assert torch.allclose(o.double(), oc, atol=2e-5) and torch.allclose(lse.double(), lc, atol=2e-5)
+    o2, _ = O.attn_fwd_l2(q, k, v, pk, pv, pk2, pv2, idx.flip(-1), pidx.flip(-1))
+    assert torch.allclose(o, o2, atol=2e-5)
+
+
+def test_forward_bf16_within_stated_tolerance_of_closed_form():
+    q, k, v, pk, pv, idx = _rand_problem(1, 2, 1024, 64, 8, torch.bfloat16)
+    o, lse = O.attn_fwd_l1(q, k, v, pk, pv, idx, 16)
+    assert o.dtype == torch.bfloat16 and lse.dtype == torch.float32
+    oc, lc = O.closed_form_l1(*[t.double() for t in (q, k, v, pk, pv)], idx, 16)
+    rel = (o.double() - oc).norm() / oc.norm()
+    assert rel < 1e-2 and (o.double() - oc).abs().max() < 2e-2
+    assert (lse.double() - lc).abs().max() < 1e-3
+
+
+# ----------------------------------------------------------------------------- backward
+def _autograd_grads(fn, leaves, do):
+    leaves = [t.double().requires_grad_(True) for t in leaves]
+    o, _ = fn(*leaves)
+    return torch.autograd.grad(o, leaves, do.double())
+
+
+def test_backward_l1_matches_autograd_of_closed_form_with_quirk():
+    q, k, v, pk, pv, idx = _rand_problem(1, 2, 1024, 32, 8, torch.float32, seed=5)
+    do = torch.randn_like(q)
+    o, lse = O.attn_fwd_l1(q, k, v, pk, pv, idx, 16)
+    dq, dk, dv, dpk, dpv = O.attn_bwd_l1(do, q, k, v, pk, pv, o, lse, idx, 16)
+    gq, gk, gv, gpk, gpv = _autograd_grads(lambda *a: O.closed_form_l1(*a, idx, 16), (q, k, v, pk, pv), do)
+    for a, b in ((dq, gq), (dk, gk), (dv, gv)):
+        assert (a.double() - b).norm() / b.norm() < 1e-5
+    # the reference's dpk/dpv are the true gradient divided by token_weight
+    assert (dpk.double() - gpk / 16).norm() / (gpk / 16).norm() < 1e-5
+    assert (dpv.double() - gpv / 16).norm() / (gpv / 16).norm() < 1e-5
+    # and with the quirk switched off they are the true gradient
+    *_, tpk, tpv = O.attn_bwd_l1(do, q, k, v, pk, pv, o, lse, idx, 16, coarse_grad_weight=None)
+    assert (tpk.double() - gpk).norm() / gpk.norm() < 1e-5 and (tpv.double() - gpv).norm() / gpv.norm() < 1e-5
+
+
+def test_backward_l2_matches_autograd_of_closed_form():
+    prob = _rand_problem(1, 1, 16384, 16, 8, torch.float32, T2=4, seed=6)
+    q, k, v, pk, pv, pk2, pv2, idx, pidx = prob
+    do = torch.randn_like(q)
+    o, lse = O.attn_fwd_l2(q, k, v, pk, pv, pk2, pv2, idx, pidx)
+    got = O.attn_bwd_l2(do, q, k, v, pk, pv, pk2, pv2, o, lse, idx, pidx)
+    want = _autograd_grads(lambda *a: O.closed_form_l2(*a, idx, pidx), (q, k, v, pk, pv, pk2, pv2), do)
+    for a, b in zip(got, want):
+        assert (a.double() - b).norm() / b.norm() < 2e-5
+
+
+def test_delta_variants():
+    o = torch.randn(1, 1, 8, 64).bfloat16()
+    do = torch.randn(1, 1, 8, 64).bfloat16()
+    d32 = O.attn_delta(o, do)
+    assert torch.allclose(d32, (o.double() * do.double()).sum(-1).float(), atol=1e-5)
+    dbf = O.attn_delta(o, do, in_dtype=True)
+    assert (dbf - d32).abs().max() < 0.25 and not torch.equal(dbf, d32)
+
+
+def test_whole_op_l1_backward_composition():
+    """llsa_l1_bwd = op grads + pool-backward of the pooled grads, against autograd through
+    k -> avg_pool -> pk in fp64 with the quirk applied to the pooled branch."""
+    B, H, N, D, T = 1, 1, 1024, 32, 8
+    q, k, v = (torch.randn(B, H, N, D) for _ in range(3))
+    do = torch.randn(B, H, N, D)
+    o, ctx = O.llsa_l1_fwd(q, k, v, T)
+    dq, dk, dv, _ = O.llsa_l1_bwd(do, ctx)
+    idx = ctx["indices"]
+
+    def pool64(x):
+        return x.reshape(B, H, N // 16, 16, D).mean(3)
+
+    class Quirk(torch.autograd.Function):       # identity whose gradient is divided by token_weight
+        @staticmethod
+        def forward(ctx_, x):
+            return x.clone()
+
+        @staticmethod
+        def backward(ctx_, g):
+            return g / 16
+
+    ql, kl, vl = (t.double().requires_grad_(True) for t in (q, k, v))
+    oc, _ = O.closed_form_l1(ql, kl, vl, Quirk.apply(pool64(kl)), Quirk.apply(pool64(vl)), idx, 16)
+    gq, gk, gv = torch.autograd.grad(oc, (ql, kl, vl), do.double())
+    assert torch.allclose(o.double(), oc, atol=2e-5)
+    for a, b in ((dq, gq), (dk, gk), (dv, gv)):
+        assert (a.double() - b).norm() / b.norm() < 1e-5
+
+
+def test_whole_op_l2_backward_composition():
+    B, H, N, D = 1, 1, 16384, 16
+    q, k, v = (torch.randn(B, H, N, D) for _ in range(3))
+    do = torch.randn(B, H, N, D)
+    o, ctx = O.llsa_l2_fwd(q, k, v, 4, 4)
+    dq, dk, dv, _ = O.llsa_l2_bwd(do, ctx)
+
+    def pool64(x):
+        return x.reshape(B, H, x.shape[2] // 16, 16, D).mean(3)
+
+    ql, kl, vl = (t.double().requires_grad_(True) for t in (q, k, v))
+    pk, pv = pool64(kl), pool64(vl)
+    oc, _ = O.closed_form_l2(ql, kl, vl, pk, pv, pool64(pk), pool64(pv), ctx["indices"], ctx["p_indices"])
+    gq, gk, gv = torch.autograd.grad(oc, (ql, kl, vl), do.double())
+    assert torch.allclose(o.double(), oc, atol=2e-5)
+    for a, b in ((dq, gq), (dk, gk), (dv, gv)):
+        assert (a.double() - b).norm() / b.norm() < 2e-5
+    # selection is hierarchical: every fine index lies inside a coarse block its parent selected
+    par = ctx["p_indices"].repeat_interleave(16, dim=2)
+    assert ((ctx["indices"].long()[..., None] // 16) == par[:, :, :, None, :]).any(-1).all()
