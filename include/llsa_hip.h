@@ -1,0 +1,176 @@
+/*
+ * libllsa_hip.so -- C ABI of the MI355X (gfx950) implementation of the llsa_l1 / llsa_l2
+ * hot path of SingleZombie/LLSA (log-linear sparse attention on Z-ordered tokens).
+ *
+ * The reference has no FFI: its boundary is a Python operator API whose launchers take
+ * torch tensors and start Triton kernels (the modules of src/llsa/kernel/torch_op calling
+ * those of src/llsa/kernel/triton).  Each entry point below replaces one of those launchers;
+ * the comment on it names the launcher (file:line in the reference checkout).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller; nothing is allocated here
+ *   - tensors are bf16 (the MFMA kernels) unless a `dtype` argument says otherwise
+ *   - strides are in ELEMENTS; the innermost (channel) stride is always 1 and every row
+ *     start must be 16-byte aligned
+ *   - the head dimension D is 64 and the block size is 16 in every attention/selection
+ *     kernel (the only values the reference's configs use); llsa_mean_pool_* are general
+ *   - indices are int32 block ids
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*); no host sync
+ *   - return value: 0 on success, negative on a rejected argument or a launch error;
+ *     llsa_last_error_string() describes the last failure on the calling thread
+ *
+ * Block-transposed layout ("xt" below): a (B,H,n,64) tensor viewed as blocks of 16 rows,
+ * each block stored channel-major: xt[b][h][blk][d][t] = x[b][h][16*blk + t][d].  The
+ * MFMA kernels read one operand of every product whose contraction runs over tokens
+ * (P.V, dS.K, P^T.dO, dS^T.Q) from this layout with plain 8-byte loads.
+ */
+#ifndef LLSA_HIP_H
+#define LLSA_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LLSA_DTYPE_BF16 0
+#define LLSA_DTYPE_F32 1
+
+int llsa_version(void);
+const char* llsa_last_error_string(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Pooling pyramid.  Replaces the 3 (l1) / 6 (l2) launches of mean_pool1d
+ * (kernel/triton/mean_pool.py:129-148, called from torch_op/flash_sparse_attention_res_1.py:42-44
+ * and ..._res_2.py:49-55) and, when `freq` is given, my_rope_fn on the same tensor
+ * (kernel/triton/rope.py:100-127) in one pass over the input.  One launch serves up to 4
+ * tensors.  Rounding follows the reference: the accumulator has the tensor dtype, summed in
+ * token order.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct llsa_pool_item {
+    const void* x;          /* (B,H,n,64) bf16, strides below                                   */
+    int64_t sxb, sxh, sxn;
+    int32_t n;              /* rows of this item, multiple of 16                                */
+    int32_t rope;           /* rotate x with `freq` first (needs xrot)                          */
+    void* y1;               /* (B,H,n/16,64)   mean over 16 rows, contiguous, or NULL           */
+    void* y2;               /* (B,H,n/256,64)  mean over 16 rows of y1, or NULL (n % 256 == 0)  */
+    void* xt;               /* (B,H,n/16,64,16) block-transposed (rotated) x, or NULL           */
+    void* y1t;              /* (B,H,n/256,64,16) block-transposed y1, or NULL (n % 256 == 0)    */
+    void* xrot;             /* (B,H,n,64) contiguous rotated x, or NULL                         */
+} llsa_pool_item;
+
+int llsa_pool_pyramid_fwd(const llsa_pool_item* items, int n_items, const void* freq /* (n,64) bf16 or NULL */,
+                          int B, int H, void* stream);
+
+/* General mean_pool1d forward / backward, layout 'bhsc' (mean_pool.py:6-58,129-165); the
+ * 'bsc' layout (mean_pool.py:61-110,168-206) is the same call with H = 1.  Any K dividing S,
+ * any C, bf16 or fp32, arbitrary strides (4 element strides each). */
+int llsa_mean_pool_fwd(const void* x, const int64_t* sx, void* y, const int64_t* sy,
+                       int B, int H, int S, int C, int K, int dtype, void* stream);
+int llsa_mean_pool_bwd(const void* dy, const int64_t* sdy, void* dx, const int64_t* sdx,
+                       int B, int H, int S_out, int C, int K, int dtype, void* stream);
+
+/* What autograd does after the operator's backward: out = rn(dx + rn(g1 / 16)) per token with
+ * g1 = dy1 (l1) or rn(dy1 + rn(dy2 / 16)) (l2), i.e. mean_pool backward (mean_pool.py:150-165)
+ * plus the gradient accumulation into k / v, in one pass; with `freq` the result is then
+ * rotated back (rope.py:130-145).  out may alias dx. */
+int llsa_pool_bwd_accum(const void* dx, const int64_t* sdx /*3*/, const void* dy1, const void* dy2 /* or NULL */,
+                        void* out, const int64_t* sout /*3*/, const void* freq /* or NULL */,
+                        int B, int H, int N, void* stream);
+
+/* 2-D RoPE rotation, forward and backward (rope.py:6-97,100-145).  freq is (S,64) with
+ * [sin, cos] interleaved; arithmetic is rounded to bf16 after every operation. */
+int llsa_rope_fwd(const void* x, const int64_t* sx /*3*/, const void* freq, void* y, const int64_t* sy /*3*/,
+                  int B, int H, int S, void* stream);
+int llsa_rope_bwd(const void* dy, const int64_t* sdy /*3*/, const void* freq, void* dx, const int64_t* sdx /*3*/,
+                  int B, int H, int S, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Selection.
+ * llsa_topk_dense replaces gen_sparse_indices (kernel/triton/topk.py:6-9): scores pq.pk^T are
+ * rounded to bf16 when round_scores != 0 (the reference's matmul returns the input dtype),
+ * top-T per row, descending, equal scores -> smaller index (torch.topk leaves that order
+ * unspecified; this library fixes it).  pq, pk (B,H,n,64) contiguous, out (B,H,n,T) int32.
+ * llsa_topk_sparse replaces compute_topk_indices_sparse (topk.py:172-197): the candidates of
+ * the 16 rows of parent block G are the level-1 key blocks parent_idx[G][a]*16 + b; fp32
+ * scores; descending, ties -> smaller index (topk.py:155-164).
+ * ---------------------------------------------------------------------------------------- */
+int llsa_topk_dense(const void* pq, const void* pk, int32_t* out_idx, int B, int H, int n, int T,
+                    int round_scores, void* stream);
+int llsa_topk_sparse(const void* pq, const void* pk, const int32_t* parent_idx, int32_t* out_idx,
+                     int B, int H, int N1, int T, int T2, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Forward.  Replaces sparse_indices_attn_res_fwd (sparse_attention_res_1.py:123-150) when
+ * levels == 1 and sparse_indices_attn_res_2_2_fwd (sparse_attention_res_2.py:166-199) when
+ * levels == 2.
+ * ---------------------------------------------------------------------------------------- */
+typedef struct llsa_attn_fwd_args {
+    const void* q;  int64_t sqb, sqh, sqn;     /* (B,H,N,64)                                      */
+    const void* k;  int64_t skb, skh, skn;     /* (B,H,N,64)                                      */
+    const void* vt;                            /* (B,H,N/16,64,16)  block-transposed v            */
+    const void* pk;                            /* (B,H,N/16,64)     level-1 pooled k, contiguous  */
+    const void* pvt;                           /* (B,H,N/256,64,16) block-transposed pooled v     */
+    const void* pk2;                           /* (B,H,N/256,64)    level-2 pooled k (levels==2)  */
+    const void* pv2t;                          /* (B,H,N/4096,64,16)                              */
+    const int32_t* idx;                        /* (B,H,N/16,T)   selected fine blocks             */
+    const int32_t* pidx;                       /* (B,H,N/256,T2) selected coarse blocks (l2)      */
+    void* o;        int64_t sob, soh, son;     /* (B,H,N,64) out                                  */
+    float* lse;                                /* (B,H,N) out, m + log(l)                          */
+    int32_t B, H, N, T, T2, levels;
+    float w1, w2;                              /* token_weight, token_weight_2                    */
+} llsa_attn_fwd_args;
+
+int llsa_attn_fwd(const llsa_attn_fwd_args* a, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Index transpose.  Replaces transpose_indices (kernel/triton/indices_transpose.py:104-109):
+ * idx (B,H,Mb,T) -> offsets (B,H,Kb+1) with offsets[0] = 0 and flat (B,H,Mb*T); segment n of
+ * flat lists the query blocks that selected key block n in ASCENDING order (the reference's
+ * order is whatever its atomics produce).  Rows of idx must hold distinct values.
+ * ---------------------------------------------------------------------------------------- */
+int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, int B, int H, int Mb, int Kb,
+                           int T, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Backward.  Replaces sparse_indices_attn_res_scatter_bwd_v2 (sparse_attention_res_1.py:403-471)
+ * and sparse_indices_attn_res_scatter_2_2_bwd_v2 (sparse_attention_res_2.py:578-681): the
+ * delta pre-pass, dQ, dK/dV over the transposed index, the sparse level-1 pooled gradients
+ * and the dense coarsest pooled gradients.  The k*scale temporaries of the reference
+ * (:420-422) do not exist here.  cgw1 is the factor used on the dpk/dpv path of the level-1
+ * pooled tokens: the reference uses 1 for l1 (sparse_attention_res_1.py:388-389) and w1 for
+ * l2 (sparse_attention_res_2.py:564).
+ * ---------------------------------------------------------------------------------------- */
+typedef struct llsa_attn_bwd_args {
+    const void* dout; int64_t sdob, sdoh, sdon;  /* (B,H,N,64) upstream gradient                 */
+    const void* q;    int64_t sqb, sqh, sqn;
+    const void* k;    int64_t skb, skh, skn;
+    const void* v;    int64_t svb, svh, svn;
+    const void* o;    int64_t sob, soh, son;
+    const float* lse;                            /* (B,H,N)                                       */
+    const void* pk;  const void* pv;             /* (B,H,N/16,64) contiguous                      */
+    const void* pk2; const void* pv2;            /* (B,H,N/256,64) contiguous (levels == 2)       */
+    const void* qt;  const void* kt;             /* block-transposed q, k   (B,H,N/16,64,16)      */
+    const void* pkt;                             /* block-transposed pk     (B,H,N/256,64,16)     */
+    const void* pk2t;                            /* block-transposed pk2    (B,H,N/4096,64,16)    */
+    const int32_t* idx;  const int32_t* pidx;
+    const int32_t* off;  const int32_t* flat;    /* transposed idx  (Kb = N/16)                   */
+    const int32_t* poff; const int32_t* pflat;   /* transposed pidx (Kb = N/256), levels == 2     */
+    void* dq; int64_t sdqb, sdqh, sdqn;
+    void* dk; int64_t sdkb, sdkh, sdkn;
+    void* dv; int64_t sdvb, sdvh, sdvn;
+    void* dpk;  void* dpv;                       /* (B,H,N/16,64) contiguous out                  */
+    void* dpk2; void* dpv2;                      /* (B,H,N/256,64) contiguous out (levels == 2)   */
+    void* workspace; int64_t workspace_bytes;    /* see llsa_attn_bwd_workspace_bytes             */
+    const void* freq_dq;                         /* (N,64) or NULL: rotate dq back (fused rope)   */
+    int32_t B, H, N, T, T2, levels;
+    float w1, w2, cgw1;
+} llsa_attn_bwd_args;
+
+int64_t llsa_attn_bwd_workspace_bytes(int B, int H, int N, int levels);
+int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LLSA_HIP_H */

@@ -1,0 +1,503 @@
+// Backward of the block-sparse attention: delta pre-pass, dQ per query block, and the
+// K-side gradients (dK/dV of the fine tokens through the transposed index, the sparse
+// level-1 pooled gradients of llsa_l2, and the dense coarsest pooled gradients).
+//
+// MFMA orientations (bf16 16x16x32, see llsa_device.h for the register layout):
+//   dQ pass, per key block (keys on M, queries on N, like the forward):
+//       S^T  = K . Q^T          dP^T = V . dO^T          dS^T = P^T o (dP^T - delta)
+//       dQ^T (64 ch x 16 q) += K_blk^T (64 x 32 keys) . dS^T      A = block-transposed K
+//   K-side pass, per key block and per pair of query blocks (queries on M, keys on N):
+//       S    = Q . K^T          dP   = dO . V^T          dS   = P o (dP - delta)
+//       dV^T (64 ch x 16 keys) += dO_blk^T (64 x 32 q) . P        A = block-transposed dO
+//       dK^T (64 ch x 16 keys) += Q_blk^T  (64 x 32 q) . dS       A = block-transposed Q
+// In both passes the score tile leaves the MFMA in exactly the operand layout the next
+// product needs, so P and dS go from registers to registers.
+#include "llsa_device.h"
+#include "llsa_host.h"
+#include "../../include/llsa_hip.h"
+
+namespace llsa {
+
+// ---------------------------------------------------------------------------------------
+// delta = rowsum(O * dO) in fp32, and the block-transposed copy of dO.
+// Same thread mapping as the pooling kernel: 16 blocks x 8 channel chunks per workgroup.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(128) void bwd_pre_kernel(llsa_attn_bwd_args a, float* __restrict__ delta,
+                                                      bf16* __restrict__ dot) {
+    const int N1 = a.N / kBlk;
+    const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+    const int t = threadIdx.x, c = t & 7, r = t >> 3;
+    const int blk = blockIdx.x * 16 + r;
+    if (blk >= N1) return;                      // no barrier below
+    const bf16* op = (const bf16*)a.o + b * a.sob + h * a.soh + (int64_t)blk * kBlk * a.son + c * 8;
+    const bf16* gp = (const bf16*)a.dout + b * a.sdob + h * a.sdoh + (int64_t)blk * kBlk * a.sdon + c * 8;
+    bf16x8 gv[16];
+    float part[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        gv[i] = ld16(gp + i * a.sdon);
+        const bf16x8 ov = ld16(op + i * a.son);
+        float s = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) s += (float)ov[e] * (float)gv[i][e];
+        part[i] = s;
+    }
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        float s = part[i];
+        s += __shfl_xor(s, 1);
+        s += __shfl_xor(s, 2);
+        s += __shfl_xor(s, 4);
+        part[i] = s;
+    }
+    if (c == 0) {
+        float* dp = delta + (int64_t)bh * a.N + blk * kBlk;
+#pragma unroll
+        for (int i = 0; i < 16; i++) dp[i] = part[i];
+    }
+    bf16* xt = dot + (((int64_t)bh * N1 + blk) * kD + c * 8) * kBlk;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        bf16x8 lo, hi;
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            lo[i] = gv[i][e];
+            hi[i] = gv[8 + i][e];
+        }
+        st16(xt + e * kBlk, lo);
+        st16(xt + e * kBlk + 8, hi);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// dQ: one wave per query block, key blocks taken two at a time (32 keys = one MFMA K step)
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ void dq_pair(f32x4 dq[4], const bf16x8 bq[2], const bf16x8 bdo[2], float lse2, float delta,
+                                        float w, const bf16* const kb[2], int64_t ks, const bf16* const vb[2], int64_t vs,
+                                        const bf16* const ktb[2], int lane) {
+    const int r = lane & 15, quad = lane >> 4;
+    bf16x8 bds;
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const bf16* kp = kb[j] + r * ks + quad * 8;
+        const bf16* vp = vb[j] + r * vs + quad * 8;
+        f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
+        s = mfma_bf16(ld16(kp), bq[0], s);
+        s = mfma_bf16(ld16(kp + 32), bq[1], s);
+        dp = mfma_bf16(ld16(vp), bdo[0], dp);
+        dp = mfma_bf16(ld16(vp + 32), bdo[1], dp);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const float p = exp2_fast(fmaf(s[e], kScaleLog2e, -lse2)) * w;
+            bds[j * 4 + e] = (bf16)(p * (dp[e] - delta));
+        }
+    }
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++) {
+        const int off = (dt * 16 + r) * kBlk + quad * 4;
+        dq[dt] = mfma_bf16(cat(ld8(ktb[0] + off), ld8(ktb[1] + off)), bds, dq[dt]);
+    }
+}
+
+__global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, const float* __restrict__ delta) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int N1 = a.N / kBlk, N2 = N1 / kBlk;
+    const int g = blockIdx.x * 4 + wave;
+    if (g >= N1) return;
+    const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+    const int r = lane & 15, quad = lane >> 4;
+    const int tok = g * kBlk + r;
+
+    bf16x8 bq[2], bdo[2];
+    {
+        const bf16* qp = (const bf16*)a.q + b * a.sqb + h * a.sqh + (int64_t)tok * a.sqn + quad * 8;
+        const bf16* gp = (const bf16*)a.dout + b * a.sdob + h * a.sdoh + (int64_t)tok * a.sdon + quad * 8;
+        bq[0] = ld16(qp);
+        bq[1] = ld16(qp + 32);
+        bdo[0] = ld16(gp);
+        bdo[1] = ld16(gp + 32);
+    }
+    const float lse2 = a.lse[(int64_t)bh * a.N + tok] * kLog2e;
+    const float dl = delta[(int64_t)bh * a.N + tok];
+    f32x4 dq[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++) dq[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const bf16* kbase = (const bf16*)a.k + b * a.skb + h * a.skh;
+    const bf16* vbase = (const bf16*)a.v + b * a.svb + h * a.svh;
+    const bf16* kt = (const bf16*)a.kt + (int64_t)bh * N1 * (kD * kBlk);
+    const bf16* pk = (const bf16*)a.pk + (int64_t)bh * N1 * kD;
+    const bf16* pv = (const bf16*)a.pv + (int64_t)bh * N1 * kD;
+    const bf16* pkt = (const bf16*)a.pkt + (int64_t)bh * N2 * (kD * kBlk);
+    const bf16 *kb[2], *vb[2], *ktb[2];
+
+    const int* ip = a.idx + ((int64_t)bh * N1 + g) * a.T;
+    for (int t = 0; t < a.T / 2; t++) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int blk = clampi(ip[2 * t + j], 0, N1 - 1);
+            kb[j] = kbase + (int64_t)blk * kBlk * a.skn;
+            vb[j] = vbase + (int64_t)blk * kBlk * a.svn;
+            ktb[j] = kt + (int64_t)blk * (kD * kBlk);
+        }
+        dq_pair(dq, bq, bdo, lse2, dl, 1.f, kb, a.skn, vb, a.svn, ktb, lane);
+    }
+    if (a.levels == 2) {
+        const int* pip = a.pidx + ((int64_t)bh * N2 + g / kBlk) * a.T2;
+        for (int t = 0; t < a.T2 / 2; t++) {
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const int blk = clampi(pip[2 * t + j], 0, N2 - 1);
+                kb[j] = pk + (int64_t)blk * kBlk * kD;
+                vb[j] = pv + (int64_t)blk * kBlk * kD;
+                ktb[j] = pkt + (int64_t)blk * (kD * kBlk);
+            }
+            dq_pair(dq, bq, bdo, lse2, dl, a.w1, kb, kD, vb, kD, ktb, lane);
+        }
+        const bf16* pk2 = (const bf16*)a.pk2 + (int64_t)bh * N2 * kD;
+        const bf16* pv2 = (const bf16*)a.pv2 + (int64_t)bh * N2 * kD;
+        const bf16* pk2t = (const bf16*)a.pk2t + (int64_t)bh * (N2 / kBlk) * (kD * kBlk);
+        for (int t = 0; t < N2 / 32; t++) {
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                kb[j] = pk2 + (int64_t)(2 * t + j) * kBlk * kD;
+                vb[j] = pv2 + (int64_t)(2 * t + j) * kBlk * kD;
+                ktb[j] = pk2t + (int64_t)(2 * t + j) * (kD * kBlk);
+            }
+            dq_pair(dq, bq, bdo, lse2, dl, a.w2, kb, kD, vb, kD, ktb, lane);
+        }
+    } else {
+        for (int t = 0; t < N1 / 32; t++) {
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                kb[j] = pk + (int64_t)(2 * t + j) * kBlk * kD;
+                vb[j] = pv + (int64_t)(2 * t + j) * kBlk * kD;
+                ktb[j] = pkt + (int64_t)(2 * t + j) * (kD * kBlk);
+            }
+            dq_pair(dq, bq, bdo, lse2, dl, a.w1, kb, kD, vb, kD, ktb, lane);
+        }
+    }
+
+    bf16* op = (bf16*)a.dq + b * a.sdqb + h * a.sdqh + (int64_t)tok * a.sdqn + quad * 4;
+    const bf16* fq = a.freq_dq ? (const bf16*)a.freq_dq + (int64_t)tok * kD + quad * 4 : nullptr;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++) {
+        bf16x4 o = cvt4(dq[dt] * kScale);
+        if (fq != nullptr) {                    // rotate the gradient back: [sin, cos] pairs
+            const bf16x4 f = ld8(fq + dt * 16);
+            bf16x4 y;
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const float s = (float)f[2 * j], c = (float)f[2 * j + 1];
+                const float ge = (float)o[2 * j], go = (float)o[2 * j + 1];
+                y[2 * j] = (bf16)(rn_bf16(c * ge) + rn_bf16(s * go));
+                y[2 * j + 1] = (bf16)(rn_bf16(-s * ge) + rn_bf16(c * go));
+            }
+            o = y;
+        }
+        st8(op + dt * 16, o);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// K-side gradients.  A "unit" is 16 key rows (a fine K block, 16 level-1 pooled tokens of one
+// coarse block, or 16 tokens of the dense coarsest level) together with a list of query
+// blocks; the unit's waves walk the list two query blocks at a time.
+// ---------------------------------------------------------------------------------------
+enum { MODE_FINE = 0, MODE_SPARSE1 = 1, MODE_DENSE = 2 };
+
+struct KSideParams {
+    const bf16* q;   int64_t sqb, sqh, sqn;
+    const bf16* dout; int64_t sdob, sdoh, sdon;
+    const bf16* qt;  const bf16* dot;             // block-transposed q and dO, (BH, N1, 64, 16)
+    const float* lse; const float* delta;         // (BH, N)
+    const bf16* kk;  int64_t skb, skh, skn;       // the unit's key rows come from here
+    const bf16* vv;  int64_t svb, svh, svn;
+    const int* off;  const int* flat;             // CSR of the list (FINE: per K block, SPARSE1: per coarse block)
+    bf16* dk; int64_t sdkb, sdkh, sdkn;           // bf16 outputs (FINE, SPARSE1)
+    bf16* dv; int64_t sdvb, sdvh, sdvn;
+    float* part_k; float* part_v;                 // fp32 partial outputs (DENSE): (chunks, BH, n_units*16, 64)
+    int H, N, n_units, chunk_len;
+    int64_t flat_stride;                          // entries of `flat` per (b,h)
+    float w;
+};
+
+__device__ __forceinline__ void kside_pair(f32x4 dk[4], f32x4 dv[4], const bf16x8 bk[2], const bf16x8 bv[2], float w,
+                                           int g0, int g1, const KSideParams& p, const bf16* qb, const bf16* gb,
+                                           const bf16* qtb, const bf16* dotb, const float* lseb, const float* dlb,
+                                           int lane) {
+    const int r = lane & 15, quad = lane >> 4;
+    bf16x8 bp, bds;
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const bool valid = (u == 0) || (g1 >= 0);
+        const int g = (u == 0 || g1 < 0) ? g0 : g1;
+        const bf16* qp = qb + (int64_t)(g * kBlk + r) * p.sqn + quad * 8;
+        const bf16* gp = gb + (int64_t)(g * kBlk + r) * p.sdon + quad * 8;
+        f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
+        s = mfma_bf16(ld16(qp), bk[0], s);
+        s = mfma_bf16(ld16(qp + 32), bk[1], s);
+        dp = mfma_bf16(ld16(gp), bv[0], dp);
+        dp = mfma_bf16(ld16(gp + 32), bv[1], dp);
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(lseb + g * kBlk + quad * 4);
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(dlb + g * kBlk + quad * 4);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            float pe = exp2_fast(fmaf(s[e], kScaleLog2e, -l4[e] * kLog2e)) * w;
+            if (!valid) pe = 0.f;
+            bp[u * 4 + e] = (bf16)pe;
+            bds[u * 4 + e] = (bf16)(pe * (dp[e] - d4[e]));
+        }
+    }
+    const int ga = g0, gb2 = (g1 < 0) ? g0 : g1;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++) {
+        const int off = (dt * 16 + r) * kBlk + quad * 4;
+        dv[dt] = mfma_bf16(cat(ld8(dotb + (int64_t)ga * (kD * kBlk) + off), ld8(dotb + (int64_t)gb2 * (kD * kBlk) + off)), bp, dv[dt]);
+        dk[dt] = mfma_bf16(cat(ld8(qtb + (int64_t)ga * (kD * kBlk) + off), ld8(qtb + (int64_t)gb2 * (kD * kBlk) + off)), bds, dk[dt]);
+    }
+}
+
+template <int MODE>
+__global__ __launch_bounds__(256) void attn_kside_kernel(KSideParams p) {
+    constexpr int W = (MODE == MODE_FINE) ? 1 : 4;            // waves per unit
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int N1 = p.N / kBlk;
+    const int bh = blockIdx.y, b = bh / p.H, h = bh % p.H;
+    const int r = lane & 15, quad = lane >> 4;
+    const int unit = (MODE == MODE_FINE) ? blockIdx.x * 4 + wave : blockIdx.x;
+    const int sub = (MODE == MODE_FINE) ? 0 : wave;
+    const int chunk = (MODE == MODE_DENSE) ? blockIdx.z : 0;
+    const bool active = unit < p.n_units;
+
+    f32x4 dk[4], dv[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++) {
+        dk[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        dv[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    if (active) {
+        bf16x8 bk[2], bv[2];
+        {
+            const bf16* kp = p.kk + b * p.skb + h * p.skh + (int64_t)(unit * kBlk + r) * p.skn + quad * 8;
+            const bf16* vp = p.vv + b * p.svb + h * p.svh + (int64_t)(unit * kBlk + r) * p.svn + quad * 8;
+            bk[0] = ld16(kp);
+            bk[1] = ld16(kp + 32);
+            bv[0] = ld16(vp);
+            bv[1] = ld16(vp + 32);
+        }
+        int start = 0, cnt = 0;
+        if (MODE == MODE_FINE) {
+            const int* o = p.off + (int64_t)bh * (p.n_units + 1) + unit;
+            start = o[0];
+            cnt = o[1] - o[0];
+        } else if (MODE == MODE_SPARSE1) {
+            const int* o = p.off + (int64_t)bh * (p.n_units + 1) + unit;
+            start = o[0];
+            cnt = (o[1] - o[0]) * kBlk;
+        } else {
+            start = chunk * p.chunk_len;
+            cnt = min(p.chunk_len, N1 - start);
+        }
+        const int* fl = (MODE == MODE_DENSE) ? nullptr : p.flat + (int64_t)bh * p.flat_stride;
+        auto entry = [&](int i) -> int {          // i-th query block of this unit's list
+            if (MODE == MODE_FINE) return clampi(fl[start + i], 0, N1 - 1);
+            if (MODE == MODE_SPARSE1) return clampi(fl[start + i / kBlk], 0, N1 / kBlk - 1) * kBlk + (i % kBlk);
+            return start + i;
+        };
+        const bf16* qb = p.q + b * p.sqb + h * p.sqh;
+        const bf16* gb = p.dout + b * p.sdob + h * p.sdoh;
+        const bf16* qtb = p.qt + (int64_t)bh * N1 * (kD * kBlk);
+        const bf16* dotb = p.dot + (int64_t)bh * N1 * (kD * kBlk);
+        const float* lseb = p.lse + (int64_t)bh * p.N;
+        const float* dlb = p.delta + (int64_t)bh * p.N;
+        for (int i = 2 * sub; i < cnt; i += 2 * W) {
+            const int g0 = entry(i);
+            const int g1 = (i + 1 < cnt) ? entry(i + 1) : -1;
+            kside_pair(dk, dv, bk, bv, p.w, g0, g1, p, qb, gb, qtb, dotb, lseb, dlb, lane);
+        }
+    }
+
+    if (MODE == MODE_FINE) {
+        if (!active) return;
+        bf16* kp = p.dk + b * p.sdkb + h * p.sdkh + (int64_t)(unit * kBlk + r) * p.sdkn + quad * 4;
+        bf16* vp = p.dv + b * p.sdvb + h * p.sdvh + (int64_t)(unit * kBlk + r) * p.sdvn + quad * 4;
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+            st8(kp + dt * 16, cvt4(dk[dt] * kScale));
+            st8(vp + dt * 16, cvt4(dv[dt]));
+        }
+        return;
+    }
+    // four waves per unit: reduce through LDS, wave w finishes channel tile w
+    __shared__ f32x4 red[4][8][kWave];
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++) {
+        red[wave][dt][lane] = dk[dt];
+        red[wave][4 + dt][lane] = dv[dt];
+    }
+    __syncthreads();
+    const int dt = wave;
+    f32x4 sk = red[0][dt][lane], sv = red[0][4 + dt][lane];
+#pragma unroll
+    for (int w = 1; w < 4; w++) {
+        sk += red[w][dt][lane];
+        sv += red[w][4 + dt][lane];
+    }
+    if (MODE == MODE_SPARSE1) {
+        bf16* kp = p.dk + b * p.sdkb + h * p.sdkh + (int64_t)(unit * kBlk + r) * p.sdkn + quad * 4 + dt * 16;
+        bf16* vp = p.dv + b * p.sdvb + h * p.sdvh + (int64_t)(unit * kBlk + r) * p.sdvn + quad * 4 + dt * 16;
+        st8(kp, cvt4(sk * kScale));
+        st8(vp, cvt4(sv));
+    } else {
+        const int64_t row = ((int64_t)chunk * gridDim.y + bh) * ((int64_t)p.n_units * kBlk) + unit * kBlk + r;
+        *reinterpret_cast<f32x4*>(p.part_k + row * kD + dt * 16 + quad * 4) = sk;
+        *reinterpret_cast<f32x4*>(p.part_v + row * kD + dt * 16 + quad * 4) = sv;
+    }
+}
+
+// sums the per-chunk fp32 partials of the dense pass in chunk order and rounds to bf16
+__global__ __launch_bounds__(256) void dense_reduce_kernel(const float* __restrict__ part_k, const float* __restrict__ part_v,
+                                                           bf16* __restrict__ dpk, bf16* __restrict__ dpv, int64_t n_elem4,
+                                                           int chunks) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n_elem4) return;
+    f32x4 sk = {0.f, 0.f, 0.f, 0.f}, sv = {0.f, 0.f, 0.f, 0.f};
+    for (int c = 0; c < chunks; c++) {
+        sk += reinterpret_cast<const f32x4*>(part_k)[c * n_elem4 + i];
+        sv += reinterpret_cast<const f32x4*>(part_v)[c * n_elem4 + i];
+    }
+    st8(dpk + i * 4, cvt4(sk * kScale));
+    st8(dpv + i * 4, cvt4(sv));
+}
+
+struct DensePlan {
+    int n_tok;       // tokens of the dense coarsest level per (b,h)
+    int chunks;      // query range split
+    int chunk_len;   // query blocks per chunk (even)
+};
+
+static DensePlan dense_plan(int B, int H, int N, int levels) {
+    const int N1 = N / 16;
+    DensePlan d;
+    d.n_tok = (levels == 2) ? N1 / 16 : N1;
+    const int units = (d.n_tok / 16) * B * H;
+    int chunks = (1024 + units - 1) / units;
+    if (chunks > N1 / 16) chunks = N1 / 16;
+    if (chunks < 1) chunks = 1;
+    int len = (N1 + chunks - 1) / chunks;
+    len += len & 1;
+    d.chunk_len = len;
+    d.chunks = (N1 + len - 1) / len;
+    return d;
+}
+
+static int64_t align256(int64_t x) { return (x + 255) & ~(int64_t)255; }
+
+}  // namespace llsa
+
+using namespace llsa;
+
+extern "C" int64_t llsa_attn_bwd_workspace_bytes(int B, int H, int N, int levels) {
+    if (B <= 0 || H <= 0 || N <= 0 || N % 16 != 0 || (levels != 1 && levels != 2)) return -1;
+    const DensePlan d = dense_plan(B, H, N, levels);
+    const int64_t BH = (int64_t)B * H;
+    int64_t bytes = align256(BH * N * 4);                       // delta
+    bytes += align256(BH * N * 64 * 2);                         // block-transposed dO
+    bytes += 2 * align256((int64_t)d.chunks * BH * d.n_tok * 64 * 4);   // dense partials (k, v)
+    return bytes;
+}
+
+extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
+    LLSA_REQUIRE(a != nullptr, "attn_bwd: null args");
+    LLSA_REQUIRE(a->levels == 1 || a->levels == 2, "attn_bwd: levels must be 1 or 2");
+    LLSA_REQUIRE(a->B > 0 && a->H > 0 && a->N > 0, "attn_bwd: bad B/H/N");
+    LLSA_REQUIRE(a->dout && a->q && a->k && a->v && a->o && a->lse && a->pk && a->pv && a->qt && a->kt && a->pkt && a->idx &&
+                     a->off && a->flat && a->dq && a->dk && a->dv && a->dpk && a->dpv && a->workspace,
+                 "attn_bwd: null tensor");
+    LLSA_REQUIRE(a->T >= 4 && a->T % 4 == 0 && a->T <= a->N / 16, "attn_bwd: topk=%d must be a multiple of 4 and <= N/16", a->T);
+    LLSA_REQUIRE(a->w1 > 0.f && a->cgw1 > 0.f, "attn_bwd: weights must be > 0");
+    if (a->levels == 1) {
+        LLSA_REQUIRE(a->N % 1024 == 0, "attn_bwd: llsa_l1 needs N %% 1024 == 0 (N=%d)", a->N);
+    } else {
+        LLSA_REQUIRE(a->N % 16384 == 0, "attn_bwd: llsa_l2 needs N %% 16384 == 0 (N=%d)", a->N);
+        LLSA_REQUIRE(a->pk2 && a->pv2 && a->pk2t && a->pidx && a->poff && a->pflat && a->dpk2 && a->dpv2, "attn_bwd: level-2 tensors missing");
+        LLSA_REQUIRE(a->T2 >= 4 && a->T2 % 4 == 0 && a->T2 <= a->N / 256, "attn_bwd: topk2=%d must be a multiple of 4 and <= N/256", a->T2);
+        LLSA_REQUIRE(a->w2 > 0.f, "attn_bwd: token_weight_2 must be > 0");
+    }
+    const void* al[] = {a->dout, a->q, a->k, a->v, a->o, a->pk, a->pv, a->pk2, a->pv2, a->qt, a->kt, a->pkt, a->pk2t,
+                        a->dq, a->dk, a->dv, a->dpk, a->dpv, a->dpk2, a->dpv2, a->workspace, a->freq_dq, a->lse};
+    for (const void* p : al) LLSA_REQUIRE(aligned16(p), "attn_bwd: tensors must be 16-byte aligned");
+    const int64_t st[] = {a->sdob, a->sdoh, a->sdon, a->sqb, a->sqh, a->sqn, a->skb, a->skh, a->skn, a->svb, a->svh, a->svn,
+                          a->sob, a->soh, a->son};
+    for (int64_t s : st) LLSA_REQUIRE(stride_ok(s), "attn_bwd: input row strides must keep rows 16-byte aligned");
+    const int64_t so[] = {a->sdqb, a->sdqh, a->sdqn, a->sdkb, a->sdkh, a->sdkn, a->sdvb, a->sdvh, a->sdvn};
+    for (int64_t s : so) LLSA_REQUIRE(s % 4 == 0, "attn_bwd: output row strides must keep rows 8-byte aligned");
+    const int64_t need = llsa_attn_bwd_workspace_bytes(a->B, a->H, a->N, a->levels);
+    LLSA_REQUIRE(a->workspace_bytes >= need, "attn_bwd: workspace too small (%lld < %lld)", (long long)a->workspace_bytes, (long long)need);
+
+    hipStream_t s = (hipStream_t)stream;
+    const int B = a->B, H = a->H, N = a->N, N1 = N / 16, N2 = N1 / 16, BH = B * H;
+    const DensePlan d = dense_plan(B, H, N, a->levels);
+    char* ws = (char*)a->workspace;
+    float* delta = (float*)ws;
+    ws += align256((int64_t)BH * N * 4);
+    bf16* dot = (bf16*)ws;
+    ws += align256((int64_t)BH * N * 64 * 2);
+    float* part_k = (float*)ws;
+    ws += align256((int64_t)d.chunks * BH * d.n_tok * 64 * 4);
+    float* part_v = (float*)ws;
+
+    hipLaunchKernelGGL(bwd_pre_kernel, dim3((N1 + 15) / 16, BH), dim3(128), 0, s, *a, delta, dot);
+    hipLaunchKernelGGL(attn_dq_kernel, dim3((N1 + 3) / 4, BH), dim3(256), 0, s, *a, (const float*)delta);
+
+    KSideParams p;
+    p.q = (const bf16*)a->q; p.sqb = a->sqb; p.sqh = a->sqh; p.sqn = a->sqn;
+    p.dout = (const bf16*)a->dout; p.sdob = a->sdob; p.sdoh = a->sdoh; p.sdon = a->sdon;
+    p.qt = (const bf16*)a->qt; p.dot = dot; p.lse = a->lse; p.delta = delta;
+    p.H = H; p.N = N; p.part_k = nullptr; p.part_v = nullptr; p.chunk_len = 0;
+
+    // fine K/V blocks
+    p.kk = (const bf16*)a->k; p.skb = a->skb; p.skh = a->skh; p.skn = a->skn;
+    p.vv = (const bf16*)a->v; p.svb = a->svb; p.svh = a->svh; p.svn = a->svn;
+    p.off = a->off; p.flat = a->flat; p.flat_stride = (int64_t)N1 * a->T;
+    p.dk = (bf16*)a->dk; p.sdkb = a->sdkb; p.sdkh = a->sdkh; p.sdkn = a->sdkn;
+    p.dv = (bf16*)a->dv; p.sdvb = a->sdvb; p.sdvh = a->sdvh; p.sdvn = a->sdvn;
+    p.n_units = N1; p.w = 1.f;
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_FINE>), dim3((N1 + 3) / 4, BH), dim3(256), 0, s, p);
+
+    const int64_t s1b = (int64_t)H * N1 * 64, s1h = (int64_t)N1 * 64;
+    const int64_t s2b = (int64_t)H * N2 * 64, s2h = (int64_t)N2 * 64;
+    if (a->levels == 2) {
+        // level-1 pooled tokens, through the transposed coarse index
+        p.kk = (const bf16*)a->pk; p.skb = s1b; p.skh = s1h; p.skn = 64;
+        p.vv = (const bf16*)a->pv; p.svb = s1b; p.svh = s1h; p.svn = 64;
+        p.off = a->poff; p.flat = a->pflat; p.flat_stride = (int64_t)N2 * a->T2;
+        p.dk = (bf16*)a->dpk; p.sdkb = s1b; p.sdkh = s1h; p.sdkn = 64;
+        p.dv = (bf16*)a->dpv; p.sdvb = s1b; p.sdvh = s1h; p.sdvn = 64;
+        p.n_units = N2; p.w = a->cgw1;
+        hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_SPARSE1>), dim3(N2, BH), dim3(256), 0, s, p);
+    }
+    // dense coarsest level
+    if (a->levels == 2) {
+        p.kk = (const bf16*)a->pk2; p.skb = s2b; p.skh = s2h; p.skn = 64;
+        p.vv = (const bf16*)a->pv2; p.svb = s2b; p.svh = s2h; p.svn = 64;
+        p.w = a->w2;
+    } else {
+        p.kk = (const bf16*)a->pk; p.skb = s1b; p.skh = s1h; p.skn = 64;
+        p.vv = (const bf16*)a->pv; p.svb = s1b; p.svh = s1h; p.svn = 64;
+        p.w = a->cgw1;
+    }
+    p.off = nullptr; p.flat = nullptr; p.flat_stride = 0; p.dk = nullptr; p.dv = nullptr;
+    p.part_k = part_k; p.part_v = part_v;
+    p.n_units = d.n_tok / 16; p.chunk_len = d.chunk_len;
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_DENSE>), dim3(p.n_units, BH, d.chunks), dim3(256), 0, s, p);
+    const int64_t n4 = (int64_t)BH * d.n_tok * 64 / 4;
+    bf16* odk = (bf16*)(a->levels == 2 ? a->dpk2 : a->dpk);
+    bf16* odv = (bf16*)(a->levels == 2 ? a->dpv2 : a->dpv);
+    hipLaunchKernelGGL(dense_reduce_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, (const float*)part_k,
+                       (const float*)part_v, odk, odv, n4, d.chunks);
+    return launch_status("attn_bwd");
+}

@@ -1,0 +1,304 @@
+// Bandwidth-bound kernels around the attention: the pooling pyramid (with optional fused
+// RoPE and the block-transposed copies the MFMA kernels read), the general mean pool,
+// the pooled-gradient accumulation of the backward pass, and the stand-alone RoPE.
+#include "llsa_device.h"
+#include "llsa_host.h"
+#include "../../include/llsa_hip.h"
+
+namespace llsa {
+
+// ---------------------------------------------------------------------------------------
+// rotation of one 8-channel chunk (4 interleaved pairs) with bf16 rounding after every
+// multiply and add, the arithmetic the reference performs in the tensor dtype
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ bf16x8 rope_chunk_fwd(bf16x8 x, bf16x8 f) {
+    bf16x8 y;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        float s = (float)f[2 * j], c = (float)f[2 * j + 1];
+        float xe = (float)x[2 * j], xo = (float)x[2 * j + 1];
+        y[2 * j] = (bf16)(rn_bf16(c * xe) - rn_bf16(s * xo));
+        y[2 * j + 1] = (bf16)(rn_bf16(s * xe) + rn_bf16(c * xo));
+    }
+    return y;
+}
+__device__ __forceinline__ bf16x8 rope_chunk_bwd(bf16x8 g, bf16x8 f) {
+    bf16x8 y;
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        float s = (float)f[2 * j], c = (float)f[2 * j + 1];
+        float ge = (float)g[2 * j], go = (float)g[2 * j + 1];
+        y[2 * j] = (bf16)(rn_bf16(c * ge) + rn_bf16(s * go));
+        y[2 * j + 1] = (bf16)(rn_bf16(-s * ge) + rn_bf16(c * go));
+    }
+    return y;
+}
+
+// ---------------------------------------------------------------------------------------
+// pooling pyramid: one workgroup = 256 consecutive tokens (16 blocks of 16) of one (b,h) of
+// one item.  Thread t owns block r = t/8 and the 8-channel chunk c = t%8: it streams the 16
+// rows of its block with 16-byte loads (8 neighbouring lanes cover one 128-byte row), keeps
+// them in registers, and emits everything that derives from them.
+// ---------------------------------------------------------------------------------------
+struct PoolParams {
+    llsa_pool_item it[4];
+    const bf16* freq;
+    int H;
+};
+
+__global__ __launch_bounds__(128) void pool_pyramid_kernel(PoolParams p) {
+    const llsa_pool_item& it = p.it[blockIdx.z];
+    const int n1 = it.n / kBlk;
+    if ((int)blockIdx.x * 16 >= n1) return;
+    const int bh = blockIdx.y, b = bh / p.H, h = bh % p.H;
+    const int t = threadIdx.x, c = t & 7, r = t >> 3;
+    const int blk = blockIdx.x * 16 + r;
+    const bool valid = blk < n1;
+
+    bf16x8 xv[16];
+    bf16x8 y = zero8();
+    if (valid) {
+        const bf16* x = (const bf16*)it.x + b * it.sxb + h * it.sxh + (int64_t)blk * kBlk * it.sxn + c * 8;
+#pragma unroll
+        for (int i = 0; i < 16; i++) xv[i] = ld16(x + i * it.sxn);
+        if (it.rope) {
+            const bf16* f = p.freq + ((int64_t)blk * kBlk) * kD + c * 8;
+            bf16* xr = (bf16*)it.xrot + ((int64_t)bh * it.n + (int64_t)blk * kBlk) * kD + c * 8;
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                xv[i] = rope_chunk_fwd(xv[i], ld16(f + i * kD));
+                st16(xr + i * kD, xv[i]);
+            }
+        }
+        if (it.y1 != nullptr || it.y2 != nullptr || it.y1t != nullptr) {
+            float acc[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc[e] = 0.f;
+#pragma unroll
+            for (int i = 0; i < 16; i++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) acc[e] = rn_bf16(acc[e] + (float)xv[i][e]);
+#pragma unroll
+            for (int e = 0; e < 8; e++) y[e] = (bf16)(acc[e] * 0.0625f);
+            if (it.y1 != nullptr) st16((bf16*)it.y1 + ((int64_t)bh * n1 + blk) * kD + c * 8, y);
+        }
+        if (it.xt != nullptr) {
+            bf16* xt = (bf16*)it.xt + (((int64_t)bh * n1 + blk) * kD + c * 8) * kBlk;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                bf16x8 lo, hi;
+#pragma unroll
+                for (int i = 0; i < 8; i++) {
+                    lo[i] = xv[i][e];
+                    hi[i] = xv[8 + i][e];
+                }
+                st16(xt + e * kBlk, lo);
+                st16(xt + e * kBlk + 8, hi);
+            }
+        }
+    }
+    if (it.y2 == nullptr && it.y1t == nullptr) return;      // uniform over the workgroup
+
+    __shared__ bf16 sm[16][kD];
+    st16(&sm[r][c * 8], y);
+    __syncthreads();
+    const int n2 = it.n / (kBlk * kBlk);
+    if (it.y2 != nullptr && t < 8) {
+        float acc[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc[e] = 0.f;
+        for (int i = 0; i < 16; i++) {
+            bf16x8 v = ld16(&sm[i][t * 8]);
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc[e] = rn_bf16(acc[e] + (float)v[e]);
+        }
+        bf16x8 y2;
+#pragma unroll
+        for (int e = 0; e < 8; e++) y2[e] = (bf16)(acc[e] * 0.0625f);
+        st16((bf16*)it.y2 + ((int64_t)bh * n2 + blockIdx.x) * kD + t * 8, y2);
+    }
+    if (it.y1t != nullptr) {
+        const int d = t & 63, half = t >> 6;
+        bf16x8 v;
+#pragma unroll
+        for (int i = 0; i < 8; i++) v[i] = sm[half * 8 + i][d];
+        st16((bf16*)it.y1t + (((int64_t)bh * n2 + blockIdx.x) * kD + d) * kBlk + half * 8, v);
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// general mean pool (any K, C, strides), one thread per output element
+// ---------------------------------------------------------------------------------------
+struct Strides4 {
+    int64_t s[4];
+};
+
+template <typename T>
+__global__ void mean_pool_fwd_kernel(const T* x, Strides4 sx, T* y, Strides4 sy, int H, int C, int K) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    const int s = blockIdx.y, bh = blockIdx.z, b = bh / H, h = bh % H;
+    const T* xp = x + b * sx.s[0] + h * sx.s[1] + (int64_t)s * K * sx.s[2] + c * sx.s[3];
+    float acc = 0.f;
+    for (int i = 0; i < K; i++) acc = (float)(T)(acc + (float)xp[i * sx.s[2]]);
+    y[b * sy.s[0] + h * sy.s[1] + s * sy.s[2] + c * sy.s[3]] = (T)(acc / (float)K);
+}
+
+template <typename T>
+__global__ void mean_pool_bwd_kernel(const T* dy, Strides4 sdy, T* dx, Strides4 sdx, int H, int C, int K) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    const int s = blockIdx.y, bh = blockIdx.z, b = bh / H, h = bh % H;
+    const T g = (T)((float)dy[b * sdy.s[0] + h * sdy.s[1] + s * sdy.s[2] + c * sdy.s[3]] / (float)K);
+    T* xp = dx + b * sdx.s[0] + h * sdx.s[1] + (int64_t)s * K * sdx.s[2] + c * sdx.s[3];
+    for (int i = 0; i < K; i++) xp[i * sdx.s[2]] = g;
+}
+
+// ---------------------------------------------------------------------------------------
+// pooled-gradient accumulation: out = rn(dx + rn(g1/16)), g1 = dy1 or rn(dy1 + rn(dy2/16)),
+// optionally rotated back.  One thread per (token, 8-channel chunk).
+// ---------------------------------------------------------------------------------------
+struct Strides3 {
+    int64_t b, h, n;
+};
+
+__global__ __launch_bounds__(256) void pool_bwd_accum_kernel(const bf16* dx, Strides3 sdx, const bf16* dy1,
+                                                             const bf16* dy2, bf16* out, Strides3 so,
+                                                             const bf16* freq, int H, int N) {
+    const int tok = blockIdx.x * 32 + (threadIdx.x >> 3), c = threadIdx.x & 7;
+    if (tok >= N) return;
+    const int bh = blockIdx.y, b = bh / H, h = bh % H;
+    const int n1 = N / kBlk, n2 = n1 / kBlk;
+    bf16x8 g1 = ld16(dy1 + ((int64_t)bh * n1 + tok / kBlk) * kD + c * 8);
+    if (dy2 != nullptr) {
+        bf16x8 g2 = ld16(dy2 + ((int64_t)bh * n2 + tok / (kBlk * kBlk)) * kD + c * 8);
+#pragma unroll
+        for (int e = 0; e < 8; e++) g1[e] = (bf16)((float)g1[e] + rn_bf16((float)g2[e] * 0.0625f));
+    }
+    bf16x8 x = ld16(dx + b * sdx.b + h * sdx.h + (int64_t)tok * sdx.n + c * 8);
+#pragma unroll
+    for (int e = 0; e < 8; e++) x[e] = (bf16)((float)x[e] + rn_bf16((float)g1[e] * 0.0625f));
+    if (freq != nullptr) x = rope_chunk_bwd(x, ld16(freq + (int64_t)tok * kD + c * 8));
+    st16(out + b * so.b + h * so.h + (int64_t)tok * so.n + c * 8, x);
+}
+
+// ---------------------------------------------------------------------------------------
+// stand-alone RoPE: one thread per (token, 8-channel chunk), 32 tokens per workgroup
+// ---------------------------------------------------------------------------------------
+template <bool BWD>
+__global__ __launch_bounds__(256) void rope_kernel(const bf16* x, Strides3 sx, const bf16* freq, bf16* y,
+                                                   Strides3 sy, int H, int S) {
+    const int tok = blockIdx.x * 32 + (threadIdx.x >> 3), c = threadIdx.x & 7;
+    if (tok >= S) return;
+    const int bh = blockIdx.y, b = bh / H, h = bh % H;
+    bf16x8 v = ld16(x + b * sx.b + h * sx.h + (int64_t)tok * sx.n + c * 8);
+    bf16x8 f = ld16(freq + (int64_t)tok * kD + c * 8);
+    v = BWD ? rope_chunk_bwd(v, f) : rope_chunk_fwd(v, f);
+    st16(y + b * sy.b + h * sy.h + (int64_t)tok * sy.n + c * 8, v);
+}
+
+}  // namespace llsa
+
+using namespace llsa;
+
+extern "C" int llsa_pool_pyramid_fwd(const llsa_pool_item* items, int n_items, const void* freq, int B, int H,
+                                     void* stream) {
+    LLSA_REQUIRE(items != nullptr && n_items >= 1 && n_items <= 4, "pool_pyramid: 1..4 items, got %d", n_items);
+    LLSA_REQUIRE(B > 0 && H > 0, "pool_pyramid: bad B/H");
+    PoolParams p;
+    p.freq = (const bf16*)freq;
+    p.H = H;
+    int max_n = 0;
+    for (int i = 0; i < n_items; i++) {
+        const llsa_pool_item& it = items[i];
+        LLSA_REQUIRE(it.x != nullptr && it.n > 0 && it.n % 16 == 0, "pool_pyramid: item %d: n=%d must be a positive multiple of 16", i, it.n);
+        LLSA_REQUIRE(aligned16(it.x) && stride_ok(it.sxb) && stride_ok(it.sxh) && stride_ok(it.sxn),
+                     "pool_pyramid: item %d: rows must be 16-byte aligned", i);
+        LLSA_REQUIRE((it.y2 == nullptr && it.y1t == nullptr) || it.n % 256 == 0,
+                     "pool_pyramid: item %d: level-2 outputs need n %% 256 == 0 (n=%d)", i, it.n);
+        LLSA_REQUIRE(!it.rope || (freq != nullptr && it.xrot != nullptr), "pool_pyramid: item %d: rope needs freq and xrot", i);
+        LLSA_REQUIRE(aligned16(it.y1) && aligned16(it.y2) && aligned16(it.xt) && aligned16(it.y1t) && aligned16(it.xrot),
+                     "pool_pyramid: item %d: outputs must be 16-byte aligned", i);
+        p.it[i] = it;
+        if (it.n > max_n) max_n = it.n;
+    }
+    for (int i = n_items; i < 4; i++) p.it[i] = items[0];
+    dim3 grid((max_n + 255) / 256, B * H, n_items);
+    hipLaunchKernelGGL(pool_pyramid_kernel, grid, dim3(128), 0, (hipStream_t)stream, p);
+    return launch_status("pool_pyramid");
+}
+
+template <typename T>
+static int mean_pool_launch(bool bwd, const void* a, const int64_t* sa, void* o, const int64_t* so, int B, int H,
+                            int S_out, int C, int K, hipStream_t st) {
+    Strides4 s1, s2;
+    for (int i = 0; i < 4; i++) {
+        s1.s[i] = sa[i];
+        s2.s[i] = so[i];
+    }
+    dim3 grid((C + 63) / 64, S_out, B * H);
+    if (!bwd)
+        hipLaunchKernelGGL(HIP_KERNEL_NAME(mean_pool_fwd_kernel<T>), grid, dim3(64), 0, st, (const T*)a, s1, (T*)o, s2, H, C, K);
+    else
+        hipLaunchKernelGGL(HIP_KERNEL_NAME(mean_pool_bwd_kernel<T>), grid, dim3(64), 0, st, (const T*)a, s1, (T*)o, s2, H, C, K);
+    return launch_status("mean_pool");
+}
+
+extern "C" int llsa_mean_pool_fwd(const void* x, const int64_t* sx, void* y, const int64_t* sy, int B, int H, int S,
+                                  int C, int K, int dtype, void* stream) {
+    LLSA_REQUIRE(x && y && sx && sy, "mean_pool_fwd: null argument");
+    LLSA_REQUIRE(B > 0 && H > 0 && C > 0 && K > 0 && S > 0 && S % K == 0, "mean_pool_fwd: S=%d must be a positive multiple of K=%d", S, K);
+    LLSA_REQUIRE(S / K <= 65535 && B * H <= 65535, "mean_pool_fwd: grid too large");
+    if (dtype == LLSA_DTYPE_BF16) return mean_pool_launch<bf16>(false, x, sx, y, sy, B, H, S / K, C, K, (hipStream_t)stream);
+    if (dtype == LLSA_DTYPE_F32) return mean_pool_launch<float>(false, x, sx, y, sy, B, H, S / K, C, K, (hipStream_t)stream);
+    return fail(-2, "mean_pool_fwd: unsupported dtype %d", dtype);
+}
+
+extern "C" int llsa_mean_pool_bwd(const void* dy, const int64_t* sdy, void* dx, const int64_t* sdx, int B, int H,
+                                  int S_out, int C, int K, int dtype, void* stream) {
+    LLSA_REQUIRE(dy && dx && sdy && sdx, "mean_pool_bwd: null argument");
+    LLSA_REQUIRE(B > 0 && H > 0 && C > 0 && K > 0 && S_out > 0, "mean_pool_bwd: bad shape");
+    LLSA_REQUIRE(S_out <= 65535 && B * H <= 65535, "mean_pool_bwd: grid too large");
+    if (dtype == LLSA_DTYPE_BF16) return mean_pool_launch<bf16>(true, dy, sdy, dx, sdx, B, H, S_out, C, K, (hipStream_t)stream);
+    if (dtype == LLSA_DTYPE_F32) return mean_pool_launch<float>(true, dy, sdy, dx, sdx, B, H, S_out, C, K, (hipStream_t)stream);
+    return fail(-2, "mean_pool_bwd: unsupported dtype %d", dtype);
+}
+
+static bool s3_ok(const int64_t* s) { return stride_ok(s[0]) && stride_ok(s[1]) && stride_ok(s[2]); }
+
+extern "C" int llsa_pool_bwd_accum(const void* dx, const int64_t* sdx, const void* dy1, const void* dy2, void* out,
+                                   const int64_t* sout, const void* freq, int B, int H, int N, void* stream) {
+    LLSA_REQUIRE(dx && dy1 && out && sdx && sout, "pool_bwd_accum: null argument");
+    LLSA_REQUIRE(N > 0 && N % 16 == 0 && (dy2 == nullptr || N % 256 == 0), "pool_bwd_accum: bad N=%d", N);
+    LLSA_REQUIRE(aligned16(dx) && aligned16(dy1) && aligned16(dy2) && aligned16(out) && aligned16(freq) && s3_ok(sdx) && s3_ok(sout),
+                 "pool_bwd_accum: rows must be 16-byte aligned");
+    Strides3 a{sdx[0], sdx[1], sdx[2]}, o{sout[0], sout[1], sout[2]};
+    hipLaunchKernelGGL(pool_bwd_accum_kernel, dim3((N + 31) / 32, B * H), dim3(256), 0, (hipStream_t)stream, (const bf16*)dx, a,
+                       (const bf16*)dy1, (const bf16*)dy2, (bf16*)out, o, (const bf16*)freq, H, N);
+    return launch_status("pool_bwd_accum");
+}
+
+static int rope_launch(bool bwd, const void* x, const int64_t* sx, const void* freq, void* y, const int64_t* sy, int B,
+                       int H, int S, void* stream) {
+    LLSA_REQUIRE(x && y && freq && sx && sy, "rope: null argument");
+    LLSA_REQUIRE(B > 0 && H > 0 && S > 0, "rope: bad shape");
+    LLSA_REQUIRE(aligned16(x) && aligned16(y) && aligned16(freq) && s3_ok(sx) && s3_ok(sy), "rope: rows must be 16-byte aligned");
+    Strides3 a{sx[0], sx[1], sx[2]}, o{sy[0], sy[1], sy[2]};
+    dim3 grid((S + 31) / 32, B * H);
+    if (bwd)
+        hipLaunchKernelGGL(HIP_KERNEL_NAME(rope_kernel<true>), grid, dim3(256), 0, (hipStream_t)stream, (const bf16*)x, a,
+                           (const bf16*)freq, (bf16*)y, o, H, S);
+    else
+        hipLaunchKernelGGL(HIP_KERNEL_NAME(rope_kernel<false>), grid, dim3(256), 0, (hipStream_t)stream, (const bf16*)x, a,
+                           (const bf16*)freq, (bf16*)y, o, H, S);
+    return launch_status("rope");
+}
+
+extern "C" int llsa_rope_fwd(const void* x, const int64_t* sx, const void* freq, void* y, const int64_t* sy, int B, int H,
+                             int S, void* stream) {
+    return rope_launch(false, x, sx, freq, y, sy, B, H, S, stream);
+}
+extern "C" int llsa_rope_bwd(const void* dy, const int64_t* sdy, const void* freq, void* dx, const int64_t* sdx, int B,
+                             int H, int S, void* stream) {
+    return rope_launch(true, dy, sdy, freq, dx, sdx, B, H, S, stream);
+}

@@ -1,0 +1,176 @@
+// Block selection: dense coarsest-level top-k and parent-guided fine top-k.
+//
+// Both kernels score one tile of 16 pooled queries against 16-key tiles with the bf16
+// MFMA, park the scores of the 16 rows in LDS and then let each wave pull the T best
+// entries out of "its" rows by repeated wave-wide arg-max.  The order is total --
+// higher score first, equal scores by smaller key index -- so the result does not
+// depend on how the work is split.
+#include "llsa_device.h"
+#include "llsa_host.h"
+#include "../../include/llsa_hip.h"
+
+namespace llsa {
+
+constexpr int kMaxT = 64;        // largest supported top-k
+constexpr int kChunk = 512;      // keys scored per pass of the dense kernel
+constexpr int kMaxCand = 512;    // candidates per parent in the sparse kernel (T2 * 16)
+constexpr int kNoIdx = 0x7fffffff;
+
+// Removes the T best entries of `row[0..npos)` (a wave's private LDS row) one by one.
+// Lane `lane` only ever touches positions congruent to it mod 64, so no barrier is
+// needed between iterations.  Taken entries are overwritten with NaN, which never
+// compares greater or equal.  Winners are written by lane 0.
+template <typename IdxFn>
+__device__ __forceinline__ void wave_topk_row(float* row, int npos, int T, IdxFn gidx_of, float* win_val,
+                                              int* win_idx) {
+    const int lane = threadIdx.x & (kWave - 1);
+    for (int t = 0; t < T; t++) {
+        float bv = -INFINITY;
+        int bi = kNoIdx, bp = -1;
+        for (int pos = lane; pos < npos; pos += kWave) {
+            const float v = row[pos];
+            const int gi = gidx_of(pos);
+            if (v > bv || (v == bv && gi < bi)) {
+                bv = v;
+                bi = gi;
+                bp = pos;
+            }
+        }
+        float wv = bv;
+        int wi = bi;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            const float ov = __shfl_xor(wv, off);
+            const int oi = __shfl_xor(wi, off);
+            if (ov > wv || (ov == wv && oi < wi)) {
+                wv = ov;
+                wi = oi;
+            }
+        }
+        if (bp >= 0 && bi == wi && bv == wv) row[bp] = __builtin_nanf("");
+        if (lane == 0) {
+            win_val[t] = (wi == kNoIdx) ? __builtin_nanf("") : wv;
+            win_idx[t] = wi;
+        }
+    }
+}
+
+// S^T tile: rows = 16 keys starting at krow, columns = the wave's 16 queries (bq).
+// Lane l gets the scores of query l%16 against keys 4*(l/16) .. +3 of the tile.
+__device__ __forceinline__ f32x4 score_tile(const bf16* krow, const bf16x8 bq[2]) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const bf16* p = krow + (lane & 15) * kD + (lane >> 4) * 8;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    acc = mfma_bf16(ld16(p), bq[0], acc);
+    acc = mfma_bf16(ld16(p + 32), bq[1], acc);
+    return acc;
+}
+
+__global__ __launch_bounds__(256) void topk_dense_kernel(const bf16* __restrict__ pq, const bf16* __restrict__ pk,
+                                                         int* __restrict__ out, int n, int T, int round_scores) {
+    __shared__ float sc[16][kMaxT + kChunk + 1];
+    __shared__ int carry_idx[16][kMaxT];
+    __shared__ float win_val[16][kMaxT];
+    __shared__ int win_idx[16][kMaxT];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int bh = blockIdx.y, q0 = blockIdx.x * 16;
+    const bf16* pqb = pq + ((int64_t)bh * n + q0) * kD;
+    const bf16* pkb = pk + (int64_t)bh * n * kD;
+
+    bf16x8 bq[2];
+    bq[0] = ld16(pqb + (lane & 15) * kD + (lane >> 4) * 8);
+    bq[1] = ld16(pqb + (lane & 15) * kD + (lane >> 4) * 8 + 32);
+
+    for (int i = tid; i < 16 * T; i += 256) {
+        sc[i / T][i % T] = __builtin_nanf("");
+        carry_idx[i / T][i % T] = kNoIdx;
+    }
+    __syncthreads();
+
+    for (int base = 0; base < n; base += kChunk) {
+        const int len = min(kChunk, n - base);
+        for (int tile = wave; tile < len / 16; tile += 4) {
+            f32x4 s = score_tile(pkb + (int64_t)(base + tile * 16) * kD, bq);
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                sc[lane & 15][T + tile * 16 + 4 * (lane >> 4) + e] = round_scores ? rn_bf16(s[e]) : s[e];
+        }
+        __syncthreads();
+        for (int row = wave; row < 16; row += 4) {
+            const int* ci = carry_idx[row];
+            wave_topk_row(
+                sc[row], T + len, T, [=](int pos) { return pos < T ? ci[pos] : base + pos - T; }, win_val[row],
+                win_idx[row]);
+        }
+        __syncthreads();
+        for (int i = tid; i < 16 * T; i += 256) {
+            sc[i / T][i % T] = win_val[i / T][i % T];
+            carry_idx[i / T][i % T] = win_idx[i / T][i % T];
+        }
+        __syncthreads();
+    }
+    for (int i = tid; i < 16 * T; i += 256) out[((int64_t)bh * n + q0 + i / T) * T + i % T] = win_idx[i / T][i % T];
+}
+
+__global__ __launch_bounds__(256) void topk_sparse_kernel(const bf16* __restrict__ pq, const bf16* __restrict__ pk,
+                                                          const int* __restrict__ pidx, int* __restrict__ out, int N1,
+                                                          int T, int T2) {
+    __shared__ float sc[16][kMaxCand + 1];
+    __shared__ int cand[kMaxCand];
+    __shared__ float win_val[16][kMaxT];
+    __shared__ int win_idx[16][kMaxT];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int bh = blockIdx.y, G = blockIdx.x;
+    const int N2 = N1 / kBlk, C = T2 * kBlk;
+    const bf16* pqb = pq + ((int64_t)bh * N1 + G * kBlk) * kD;
+    const bf16* pkb = pk + (int64_t)bh * N1 * kD;
+
+    for (int i = tid; i < C; i += 256)
+        cand[i] = clampi(pidx[((int64_t)bh * N2 + G) * T2 + i / kBlk], 0, N2 - 1) * kBlk + (i % kBlk);
+    bf16x8 bq[2];
+    bq[0] = ld16(pqb + (lane & 15) * kD + (lane >> 4) * 8);
+    bq[1] = ld16(pqb + (lane & 15) * kD + (lane >> 4) * 8 + 32);
+    __syncthreads();
+
+    for (int a = wave; a < T2; a += 4) {
+        f32x4 s = score_tile(pkb + (int64_t)cand[a * kBlk] * kD, bq);
+#pragma unroll
+        for (int e = 0; e < 4; e++) sc[lane & 15][a * kBlk + 4 * (lane >> 4) + e] = s[e];
+    }
+    __syncthreads();
+    for (int row = wave; row < 16; row += 4)
+        wave_topk_row(
+            sc[row], C, T, [&](int pos) { return cand[pos]; }, win_val[row], win_idx[row]);
+    __syncthreads();
+    for (int i = tid; i < 16 * T; i += 256)
+        out[((int64_t)bh * N1 + G * kBlk + i / T) * T + i % T] = win_idx[i / T][i % T];
+}
+
+}  // namespace llsa
+
+using namespace llsa;
+
+extern "C" int llsa_topk_dense(const void* pq, const void* pk, int32_t* out_idx, int B, int H, int n, int T,
+                               int round_scores, void* stream) {
+    LLSA_REQUIRE(pq && pk && out_idx, "topk_dense: null argument");
+    LLSA_REQUIRE(B > 0 && H > 0 && n > 0 && n % 16 == 0, "topk_dense: n=%d must be a positive multiple of 16", n);
+    LLSA_REQUIRE(T >= 1 && T <= kMaxT && T <= n, "topk_dense: need 1 <= T <= min(%d, n=%d), got %d", kMaxT, n, T);
+    LLSA_REQUIRE(aligned16(pq) && aligned16(pk), "topk_dense: inputs must be 16-byte aligned");
+    hipLaunchKernelGGL(topk_dense_kernel, dim3(n / 16, B * H), dim3(256), 0, (hipStream_t)stream, (const bf16*)pq,
+                       (const bf16*)pk, out_idx, n, T, round_scores);
+    return launch_status("topk_dense");
+}
+
+extern "C" int llsa_topk_sparse(const void* pq, const void* pk, const int32_t* parent_idx, int32_t* out_idx, int B, int H,
+                                int N1, int T, int T2, void* stream) {
+    LLSA_REQUIRE(pq && pk && parent_idx && out_idx, "topk_sparse: null argument");
+    LLSA_REQUIRE(B > 0 && H > 0 && N1 > 0 && N1 % 16 == 0, "topk_sparse: N1=%d must be a positive multiple of 16", N1);
+    LLSA_REQUIRE(T2 >= 1 && T2 * 16 <= kMaxCand && T2 <= N1 / 16, "topk_sparse: need 1 <= T2 <= min(%d, N1/16), got %d", kMaxCand / 16, T2);
+    LLSA_REQUIRE(T >= 1 && T <= kMaxT && T <= T2 * 16, "topk_sparse: need 1 <= T <= min(%d, 16*T2), got %d", kMaxT, T);
+    LLSA_REQUIRE(aligned16(pq) && aligned16(pk), "topk_sparse: inputs must be 16-byte aligned");
+    hipLaunchKernelGGL(topk_sparse_kernel, dim3(N1 / 16, B * H), dim3(256), 0, (hipStream_t)stream, (const bf16*)pq,
+                       (const bf16*)pk, parent_idx, out_idx, N1, T, T2);
+    return launch_status("topk_sparse");
+}

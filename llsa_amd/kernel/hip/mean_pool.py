@@ -1,0 +1,157 @@
+"""Mean pooling over consecutive tokens.  Mirrors the reference module
+kernel/triton/mean_pool.py: `mean_pool1d(x, k, format)` is an autograd function with the
+same rounding (accumulator in the tensor dtype, token order).  `pool_pyramid` is the fused
+launcher the operators use: several tensors, two levels, optional RoPE and the
+block-transposed copies in one pass."""
+from __future__ import annotations
+
+from typing import Optional, Sequence
+
+import torch
+
+from ..._lib import PoolItem
+from ._common import BLOCK, HEAD_DIM, as_rows, i64x, lib_for, ptr, require_bf16, stream_of
+
+_DTYPES = {torch.bfloat16: 0, torch.float32: 1}
+
+
+def _pool_launch(lib, bwd, a, o, B, H, S_out, C, K):
+    if a.dtype not in _DTYPES:
+        raise NotImplementedError(f"mean_pool1d supports bf16 and fp32 (got {a.dtype})")
+    fn = lib.mean_pool_bwd if bwd else lib.mean_pool_fwd
+    n = S_out if bwd else S_out * K
+    lib.check(fn(ptr(a), i64x(a.stride()), ptr(o), i64x(o.stride()), B, H, n, C, K, _DTYPES[a.dtype],
+                 stream_of(lib, a)), "mean_pool1d")
+
+
+class MeanPool1dFunction_BHSC(torch.autograd.Function):
+    """mean_pool.py:129-165."""
+
+    @staticmethod
+    def forward(ctx, x, kernel_size: int):
+        B, H, S, C = x.shape
+        assert S % kernel_size == 0
+        lib = lib_for(x)
+        y = torch.empty((B, H, S // kernel_size, C), device=x.device, dtype=x.dtype)
+        _pool_launch(lib, False, x, y, B, H, S // kernel_size, C, kernel_size)
+        ctx.kernel_size = kernel_size
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        K = ctx.kernel_size
+        B, H, S_out, C = dy.shape
+        lib = lib_for(dy)
+        dx = torch.empty((B, H, S_out * K, C), device=dy.device, dtype=dy.dtype)
+        _pool_launch(lib, True, dy, dx, B, H, S_out, C, K)
+        return dx, None
+
+
+class MeanPool1dFunction_BSC(torch.autograd.Function):
+    """mean_pool.py:168-206: the (B,S,C) layout is the (B,1,S,C) case of the same kernel."""
+
+    @staticmethod
+    def forward(ctx, x, kernel_size: int):
+        B, S, C = x.shape
+        assert S % kernel_size == 0
+        lib = lib_for(x)
+        y = torch.empty((B, S // kernel_size, C), device=x.device, dtype=x.dtype)
+        _pool_launch(lib, False, x.unsqueeze(1), y.unsqueeze(1), B, 1, S // kernel_size, C, kernel_size)
+        ctx.kernel_size = kernel_size
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        K = ctx.kernel_size
+        B, S_out, C = dy.shape
+        lib = lib_for(dy)
+        dx = torch.empty((B, S_out * K, C), device=dy.device, dtype=dy.dtype)
+        _pool_launch(lib, True, dy.unsqueeze(1), dx.unsqueeze(1), B, 1, S_out, C, K)
+        return dx, None
+
+
+def mean_pool1d(x: torch.Tensor, k: int, format='bhsc'):
+    """mean_pool.py:209-216."""
+    if format == 'bhsc':
+        return MeanPool1dFunction_BHSC.apply(x, k)
+    elif format == 'bsc':
+        return MeanPool1dFunction_BSC.apply(x, k)
+    else:
+        raise NotImplementedError(f'Format {format} is not implemented for mean_pool1d')
+
+
+class PoolSpec:
+    """What to produce from one (B,H,n,64) bf16 tensor in a pool_pyramid launch."""
+
+    def __init__(self, x, y1=False, y2=False, xt=False, y1t=False, rope=False):
+        self.x, self.y1, self.y2, self.xt, self.y1t, self.rope = x, y1, y2, xt, y1t, rope
+
+
+def pool_pyramid(specs: Sequence[PoolSpec], freq: Optional[torch.Tensor] = None):
+    """One launch of llsa_pool_pyramid_fwd.  Returns, per spec, a dict with the requested
+    outputs: y1 (B,H,n/16,64), y2 (B,H,n/256,64), xt (B,H,n/16,64,16), y1t (B,H,n/256,64,16),
+    xrot (B,H,n,64)."""
+    assert 1 <= len(specs) <= 4
+    x0 = specs[0].x
+    lib = lib_for(*[s.x for s in specs], freq)
+    B, H = x0.shape[0], x0.shape[1]
+    items, outs, keep = [], [], []
+    for s in specs:
+        x = s.x
+        require_bf16(x)
+        if x.shape[-1] != HEAD_DIM or x.shape[0] != B or x.shape[1] != H:
+            raise ValueError("pool_pyramid: all tensors must be (B,H,n,64)")
+        x = as_rows(x)
+        keep.append(x)
+        n = x.shape[2]
+        if n % BLOCK != 0:
+            raise ValueError(f"token count {n} is not a multiple of {BLOCK}")
+        if (s.y2 or s.y1t) and n % (BLOCK * BLOCK) != 0:
+            raise ValueError(f"token count {n} is not a multiple of {BLOCK * BLOCK}")
+        e = lambda *shape: torch.empty(shape, device=x.device, dtype=x.dtype)
+        o = {}
+        if s.y1:
+            o["y1"] = e(B, H, n // 16, 64)
+        if s.y2:
+            o["y2"] = e(B, H, n // 256, 64)
+        if s.xt:
+            o["xt"] = e(B, H, n // 16, 64, 16)
+        if s.y1t:
+            o["y1t"] = e(B, H, n // 256, 64, 16)
+        if s.rope:
+            if freq is None:
+                raise ValueError("rope requested without a table")
+            o["xrot"] = e(B, H, n, 64)
+        outs.append(o)
+        items.append(PoolItem(x.data_ptr(), x.stride(0), x.stride(1), x.stride(2), n, 1 if s.rope else 0,
+                              *(o[k].data_ptr() if k in o else None for k in ("y1", "y2", "xt", "y1t", "xrot"))))
+    if freq is not None:
+        require_bf16(freq)
+        freq = freq.contiguous()
+        if any(s.rope and freq.shape != (s.x.shape[2], HEAD_DIM) for s in specs):
+            raise ValueError("rope table must be (n, 64)")
+    arr = (PoolItem * len(items))(*items)
+    lib.check(lib.pool_pyramid_fwd(arr, len(items), ptr(freq), B, H, stream_of(lib, x0)), "pool_pyramid")
+    return outs
+
+
+def block_transpose(*tensors):
+    """(B,H,n,64) -> (B,H,n/16,64,16) for up to 4 tensors in one launch."""
+    outs = pool_pyramid([PoolSpec(t, xt=True) for t in tensors])
+    return [o["xt"] for o in outs]
+
+
+def pool_bwd_accum(dx, dy1, dy2=None, freq=None, out=None):
+    """out = rn(dx + rn(g1/16)) per token, g1 = dy1 or rn(dy1 + rn(dy2/16)); with freq the result is
+    rotated back.  The fused equivalent of mean_pool backward + autograd's accumulation."""
+    lib = lib_for(dx, dy1, dy2, freq)
+    require_bf16(dx, dy1, dy2, freq)
+    B, H, N, D = dx.shape
+    dxr = as_rows(dx)
+    if out is None:
+        out = torch.empty_like(dxr)
+    s = lambda t: i64x((t.stride(0), t.stride(1), t.stride(2)))
+    lib.check(lib.pool_bwd_accum(ptr(dxr), s(dxr), ptr(dy1.contiguous()), ptr(None if dy2 is None else dy2.contiguous()),
+                                 ptr(out), s(out), ptr(None if freq is None else freq.contiguous()), B, H, N,
+                                 stream_of(lib, dx)), "pool_bwd_accum")
+    return out

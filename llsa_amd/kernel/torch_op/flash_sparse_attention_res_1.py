@@ -1,0 +1,93 @@
+"""llsa_l1: one pooled level.  Mirrors torch_op/flash_sparse_attention_res_1.py of the
+reference: `FlashSparseResidualAttentionL1`, `flash_sparse_residual_attention_l1_op`,
+`llsa_l1(q, k, v, topk=8, block_size=16)` with the same positional arguments.
+
+`llsa_l1` additionally accepts `rope=freq` (an (N, 64) table of interleaved sin/cos): then
+q and k are rotated inside the pooling pass and the gradients are rotated back inside the
+backward kernels, which is the same function as
+`llsa_l1(my_rope_fn(q, freq), my_rope_fn(k, freq), v, ...)`.
+"""
+from __future__ import annotations
+
+import torch
+from torch.autograd import Function
+
+from ..hip.mean_pool import PoolSpec, mean_pool1d, pool_bwd_accum, pool_pyramid
+from ..hip.sparse_attention_res_1 import sparse_indices_attn_res_fwd, sparse_indices_attn_res_scatter_bwd_v2
+from ..hip.topk import gen_sparse_indices
+
+
+class FlashSparseResidualAttentionL1(Function):
+    """flash_sparse_attention_res_1.py:10-35."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, pq, pk, pv, topk, token_weight=1, block_size=16):
+        indices = gen_sparse_indices(pq, pk, topk)
+        output, m = sparse_indices_attn_res_fwd(q, k, v, pk, pv, indices, indices.shape[-1], token_weight,
+                                                int(block_size ** 0.5))
+        ctx.save_for_backward(q, k, v, pk, pv, output, m, indices)
+        ctx.topk = indices.shape[-1]
+        ctx.block_size = block_size
+        ctx.token_weight = token_weight
+        return output
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, pk, pv, o, m, indices = ctx.saved_tensors
+        return *sparse_indices_attn_res_scatter_bwd_v2(do, q, k, v, pk, pv, o, m, indices, ctx.topk,
+                                                       ctx.block_size, ctx.token_weight), None, None, None
+
+
+flash_sparse_residual_attention_l1_op = FlashSparseResidualAttentionL1.apply
+
+
+class _LlsaL1Fused(Function):
+    """llsa_l1 as one autograd node: pooling pyramid (+RoPE, + the block-transposed copies the
+    kernels read) in one pass, selection, attention; the backward folds the pooled gradients
+    into dk / dv (what mean_pool's backward and autograd's accumulation do in the reference)
+    and rotates dq / dk back."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, topk, block_size, freq):
+        if block_size != 16:
+            raise NotImplementedError("block_size must be 16")
+        need_grad = any(ctx.needs_input_grad[:3])
+        rope = freq is not None
+        oq, ok, ov = pool_pyramid([PoolSpec(q, y1=True, xt=need_grad, rope=rope),
+                                   PoolSpec(k, y1=True, xt=need_grad, y1t=need_grad, rope=rope),
+                                   PoolSpec(v, y1=True, xt=True, y1t=True)], freq)
+        if rope:
+            q, k = oq["xrot"], ok["xrot"]
+        pq, pk, pv = oq["y1"], ok["y1"], ov["y1"]
+        indices = gen_sparse_indices(pq, pk, topk)
+        o, m = sparse_indices_attn_res_fwd(q, k, v, pk, pv, indices, indices.shape[-1], block_size, 4,
+                                           vt=ov["xt"], pvt=ov["y1t"])
+        if need_grad:
+            ctx.save_for_backward(q, k, v, pk, pv, o, m, indices, oq["xt"], ok["xt"], ok["y1t"], freq)
+        ctx.block_size = block_size
+        ctx.indices = indices
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, pk, pv, o, m, indices, qt, kt, pkt, freq = ctx.saved_tensors
+        bs = ctx.block_size
+        dq, dk, dv, _, dpk, dpv = sparse_indices_attn_res_scatter_bwd_v2(
+            do, q, k, v, pk, pv, o, m, indices, indices.shape[-1], bs, bs, qt=qt, kt=kt, pkt=pkt, freq_dq=freq)
+        dk = pool_bwd_accum(dk, dpk, None, freq, out=dk)
+        dv = pool_bwd_accum(dv, dpv, None, None, out=dv)
+        return dq, dk, dv, None, None, None
+
+
+def llsa_l1(q, k, v, topk=8, block_size=16, rope=None):
+    """flash_sparse_attention_res_1.py:41-47."""
+    return _LlsaL1Fused.apply(q, k, v, topk, block_size, rope)
+
+
+def llsa_l1_unfused(q, k, v, topk=8, block_size=16):
+    """The reference's own composition, kernel for kernel: three mean_pool1d calls, then the op
+    (gradients reach k and v through mean_pool1d's backward and autograd's accumulation)."""
+    pq = mean_pool1d(q, block_size)
+    pk = mean_pool1d(k, block_size)
+    pv = mean_pool1d(v, block_size)
+    return flash_sparse_residual_attention_l1_op(q, k, v, pq, pk, pv, topk, block_size, block_size)

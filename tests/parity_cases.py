@@ -1,0 +1,346 @@
+"""Parity checks of the HIP kernels against the CPU oracle, written once and run twice:
+on the GPU through libllsa_hip.so (tests/test_gpu_parity.py, `-m gpu`) and, at tiny sizes,
+on the CPU through the x86 emulation build of the same sources (tests/test_emu_parity.py).
+
+Tolerances (bf16): outputs and gradients must satisfy
+    rel-L2 error      <= 1e-2
+    max-abs error     <= 2e-2 * max(1, max|reference|)
+(the max-abs bound is scaled because one bf16 ulp is already 3e-2 for values in [4, 8)).
+Integer results (pool bit patterns, indices on tie-free rows, CSR) must be identical.
+"""
+import math
+
+import torch
+
+from oracle import llsa_oracle as O
+
+REL_L2 = 1e-2
+MAX_ABS = 2e-2
+
+
+def close(name, got, ref, rel=REL_L2, mabs=MAX_ABS):
+    g, r = got.detach().double().cpu(), ref.detach().double().cpu()
+    assert g.shape == r.shape, f"{name}: shape {tuple(g.shape)} vs {tuple(r.shape)}"
+    assert torch.isfinite(g).all(), f"{name}: non-finite values"
+    e_rel = ((g - r).norm() / r.norm().clamp_min(1e-30)).item()
+    e_abs = (g - r).abs().max().item()
+    bound = mabs * max(1.0, r.abs().max().item())
+    assert e_rel <= rel and e_abs <= bound, f"{name}: rel-L2 {e_rel:.3e} (<= {rel}), max-abs {e_abs:.3e} (<= {bound:.3e})"
+    return e_rel, e_abs
+
+
+def smooth_inputs(B, H, N, D, dev, seeds=(1, 2, 3, 4)):
+    from llsa_amd.utils.synth import smooth_field
+    q = smooth_field(seeds[0], B, H, N, D)
+    k = smooth_field(seeds[1], B, H, N, D)
+    v = smooth_field(seeds[2], B, H, N, D)
+    do = torch.randn(B, H, N, D, generator=torch.Generator().manual_seed(seeds[3])).bfloat16()
+    return tuple(t.to(dev) for t in (q, k, v, do))
+
+
+def randn_inputs(B, H, N, D, dev, seed=0, strided=False):
+    g = torch.Generator().manual_seed(seed)
+    if strided:      # physical layout (B,N,H,D) viewed as (B,H,N,D), what the DiT attention processor passes
+        mk = lambda: torch.randn(B, N, H, D, generator=g).bfloat16().to(dev).transpose(1, 2)
+    else:
+        mk = lambda: torch.randn(B, H, N, D, generator=g).bfloat16().to(dev)
+    return mk(), mk(), mk(), mk()
+
+
+# ------------------------------------------------------------------------------------------
+def check_pool_pyramid(dev, B=1, H=2, N=512, strided=True, rope=True):
+    from llsa_amd.kernel.hip.mean_pool import PoolSpec, pool_pyramid
+    x, *_ = randn_inputs(B, H, N, 64, dev, seed=5, strided=strided)
+    x = x * 2
+    freq = torch.randn(N, 64, generator=torch.Generator().manual_seed(6)).bfloat16().to(dev) if rope else None
+    out, = pool_pyramid([PoolSpec(x, y1=True, y2=True, xt=True, y1t=True, rope=rope)], freq)
+    xc = x.cpu()
+    xr = O.rope_apply(xc, freq.cpu()) if rope else xc
+    p1 = O.mean_pool(xr)
+    p2 = O.mean_pool(p1)
+    if rope:
+        assert torch.equal(out["xrot"].cpu(), xr), "rotated copy differs"
+    assert torch.equal(out["y1"].cpu(), p1), "level-1 pool differs"
+    assert torch.equal(out["y2"].cpu(), p2), "level-2 pool differs"
+    assert torch.equal(out["xt"].cpu(), xr.reshape(B, H, N // 16, 16, 64).transpose(-1, -2)), "xt differs"
+    assert torch.equal(out["y1t"].cpu(), p1.reshape(B, H, N // 256, 16, 64).transpose(-1, -2)), "y1t differs"
+
+
+def check_mean_pool1d(dev, dtype=torch.bfloat16, K=16, C=64, S=128, fmt='bhsc'):
+    from llsa_amd.kernel.hip.mean_pool import mean_pool1d
+    g = torch.Generator().manual_seed(7)
+    shape = (2, 3, S, C) if fmt == 'bhsc' else (2, S, C)
+    x = (torch.randn(*shape, generator=g) * 3).to(dtype).to(dev).requires_grad_(True)
+    y = mean_pool1d(x, K, fmt)
+    dy = torch.randn(*y.shape, generator=g).to(dtype).to(dev)
+    y.backward(dy)
+    xc = x.detach().cpu()
+    x4 = xc if fmt == 'bhsc' else xc.unsqueeze(1)
+    ref = O.mean_pool(x4, K)
+    dref = O.mean_pool_bwd(dy.cpu() if fmt == 'bhsc' else dy.cpu().unsqueeze(1), K)
+    if fmt == 'bsc':
+        ref, dref = ref.squeeze(1), dref.squeeze(1)
+    assert torch.equal(y.detach().cpu(), ref), "mean_pool1d forward differs"
+    assert torch.equal(x.grad.cpu(), dref), "mean_pool1d backward differs"
+
+
+def check_rope(dev, B=1, H=2, side=8, strided=True):
+    from llsa_amd.kernel.hip.rope import my_rope_fn
+    from llsa_amd.utils.rope_table import rope_table
+    N = side * side
+    x, dy, *_ = randn_inputs(B, H, N, 64, dev, seed=8, strided=strided)
+    freq = rope_table(side, dtype=torch.bfloat16).to(dev)
+    assert torch.equal(freq.cpu(), O.rope_table(side, dtype=torch.bfloat16)), "rope table differs"
+    x = x.detach().requires_grad_(True)
+    y = my_rope_fn(x, freq)
+    y.backward(dy)
+    assert torch.equal(y.detach().cpu(), O.rope_apply(x.detach().cpu(), freq.cpu())), "rope forward differs"
+    assert torch.equal(x.grad.cpu(), O.rope_apply_bwd(dy.cpu(), freq.cpu())), "rope backward differs"
+
+
+def _safe_rows(score, T, eps_rel):
+    """Rows whose T-th / (T+1)-th scores (and, for the ordered check, all adjacent pairs among
+    the best T+1) are separated by more than eps_rel * max(1, |score|)."""
+    s, _ = torch.sort(score, dim=-1, descending=True)
+    top = s[..., :T + 1] if s.shape[-1] > T else s
+    gaps = top[..., :-1] - top[..., 1:]
+    tol = eps_rel * top[..., :-1].abs().clamp_min(1.0)
+    boundary_ok = (gaps[..., T - 1] > tol[..., T - 1]) if s.shape[-1] > T else torch.ones_like(gaps[..., 0], dtype=torch.bool)
+    ordered_ok = (gaps > tol).all(-1)
+    return boundary_ok, ordered_ok
+
+
+def check_topk_dense(dev, B=1, H=2, n=64, T=8, round_scores=True, min_safe=0.3):
+    from llsa_amd.kernel.hip.topk import gen_sparse_indices
+    g = torch.Generator().manual_seed(9)
+    pq = torch.randn(B, H, n, 64, generator=g).bfloat16()
+    pk = torch.randn(B, H, n, 64, generator=g).bfloat16()
+    idx = gen_sparse_indices(pq.to(dev), pk.to(dev), T, round_scores=round_scores).cpu().long()
+    assert idx.shape == (B, H, n, T) and idx.min() >= 0 and idx.max() < n
+    assert (idx.sort(-1).values.diff(dim=-1) > 0).all(), "duplicate index in a row"
+    exact = O.dense_scores(pq, pk, round_to_input=False)
+    ref = O.topk_lowest_index(O.dense_scores(pq, pk, round_to_input=round_scores), T)
+    # one bf16 ulp is 2^-8 relative: demand 2^-6 of separation on the unrounded scores
+    b_ok, o_ok = _safe_rows(exact, T, 2.0 ** -6 if round_scores else 1e-4)
+    assert b_ok.float().mean() >= min_safe, f"test input has too few tie-free rows ({b_ok.float().mean():.2f})"
+    same_set = (idx.sort(-1).values == ref.sort(-1).values).all(-1)
+    assert same_set[b_ok].all(), "selected set differs on tie-free rows"
+    assert (idx == ref).all(-1)[o_ok].all(), "order differs on rows with well separated scores"
+    # descending by the rounded score everywhere
+    sc = torch.gather(O.dense_scores(pq, pk, round_to_input=round_scores), -1, idx)
+    tol = (2.0 ** -6 if round_scores else 1e-4) * sc.abs().clamp_min(1.0)
+    assert (sc[..., :-1] - sc[..., 1:] >= -tol[..., 1:]).all(), "not descending"
+    return idx
+
+
+def check_topk_dense_ties(dev):
+    """Exact ties (duplicated key rows): the smaller index must come first."""
+    from llsa_amd.kernel.hip.topk import gen_sparse_indices
+    g = torch.Generator().manual_seed(10)
+    pq = torch.randn(1, 1, 32, 64, generator=g).bfloat16()
+    pk = torch.randn(1, 1, 32, 64, generator=g).bfloat16()
+    pk[0, 0, 20] = pk[0, 0, 3]
+    pk[0, 0, 9] = pk[0, 0, 3]
+    idx = gen_sparse_indices(pq.to(dev), pk.to(dev), 32).cpu().long()      # full ranking
+    for row in idx[0, 0]:
+        pos = {int(v): i for i, v in enumerate(row)}
+        assert pos[3] + 1 == pos[9] and pos[9] + 1 == pos[20], "equal scores must be ordered by index"
+
+
+def check_topk_sparse(dev, B=1, H=2, N1=256, T=8, T2=4):
+    from llsa_amd.kernel.hip.topk import compute_topk_indices_sparse
+    g = torch.Generator().manual_seed(11)
+    pq = torch.randn(B, H, N1, 64, generator=g).bfloat16()
+    pk = torch.randn(B, H, N1, 64, generator=g).bfloat16()
+    N2 = N1 // 16
+    pidx = torch.stack([torch.randperm(N2, generator=g)[:T2] for _ in range(B * H * N2)]).reshape(B, H, N2, T2).int()
+    idx = compute_topk_indices_sparse(pq.to(dev), pk.to(dev), pidx.to(dev), T, T2).cpu()
+    assert idx.dtype == torch.int32 and idx.shape == (B, H, N1, T)
+    ref, score, gidx = O.topk_sparse(pq, pk, pidx.long(), T, return_scores=True)
+    par = pidx.long().repeat_interleave(16, dim=2)
+    assert ((idx.long()[..., None] // 16) == par[:, :, :, None, :]).any(-1).all(), "index outside the parent's blocks"
+    assert (idx.long().sort(-1).values.diff(dim=-1) > 0).all(), "duplicate index in a row"
+    b_ok, o_ok = _safe_rows(score, T, 1e-4)
+    assert b_ok.float().mean() > 0.9
+    assert (idx.sort(-1).values == ref.sort(-1).values).all(-1)[b_ok].all(), "selected set differs on tie-free rows"
+    assert (idx == ref).all(-1)[o_ok].all(), "order differs on rows with well separated scores"
+
+
+def check_transpose(dev, B=2, H=2, Mb=64, T=8, Kb=None):
+    from llsa_amd.kernel.hip.indices_transpose import transpose_indices
+    g = torch.Generator().manual_seed(12)
+    kb = Kb or Mb
+    idx = torch.stack([torch.randperm(kb, generator=g)[:T] for _ in range(B * H * Mb)]).reshape(B, H, Mb, T).int()
+    off, flat = transpose_indices(idx.to(dev), Kb)
+    ro, rf = O.transpose_indices(idx.long(), Kb)
+    assert torch.equal(off.cpu().long(), ro), "offsets differ"
+    assert torch.equal(flat.cpu().long(), rf), "flat list differs"
+
+
+def check_transpose_hot_block(dev):
+    """Every query block selects key block 5 (a segment as long as the query axis) plus others."""
+    from llsa_amd.kernel.hip.indices_transpose import transpose_indices
+    B, H, Mb, T = 1, 1, 256, 4
+    g = torch.Generator().manual_seed(13)
+    rest = torch.stack([(torch.randperm(Mb - 1, generator=g)[:T - 1] + 6) % Mb for _ in range(Mb)])
+    rest[rest == 5] = 4
+    idx = torch.cat([torch.full((Mb, 1), 5), rest], 1).reshape(B, H, Mb, T).int()
+    # make rows distinct where the remap collided
+    for r in range(Mb):
+        while len(set(idx[0, 0, r].tolist())) < T:
+            idx[0, 0, r, 1:] = (torch.randperm(Mb - 8, generator=g)[:T - 1] + 8).int()
+    off, flat = transpose_indices(idx.to(dev))
+    ro, rf = O.transpose_indices(idx.long())
+    assert torch.equal(off.cpu().long(), ro) and torch.equal(flat.cpu().long(), rf)
+
+
+# ------------------------------------------------------------------------------------------
+def _selection_l1(q, k, T):
+    pq, pk = O.mean_pool(q.cpu()), O.mean_pool(k.cpu())
+    return O.topk_lowest_index(O.dense_scores(pq, pk), T)
+
+
+def check_attn_l1(dev, B=1, H=2, N=1024, T=8, strided=False, smooth=False, weight=16.0):
+    """Forward and backward kernels with oracle-chosen indices."""
+    from llsa_amd.kernel.hip._attention import attn_bwd, attn_fwd
+    q, k, v, do = smooth_inputs(B, H, N, 64, dev) if smooth else randn_inputs(B, H, N, 64, dev, seed=14, strided=strided)
+    qc, kc, vc, doc = (t.cpu() for t in (q, k, v, do))
+    pk, pv = O.mean_pool(kc), O.mean_pool(vc)
+    idx = _selection_l1(qc, kc, T)
+    o, lse = attn_fwd(q, k, v, pk.to(dev), pv.to(dev), idx.int().to(dev), weight)
+    ro, rl = O.attn_fwd_l1(qc, kc, vc, pk, pv, idx, weight)
+    assert o.stride() == q.stride(), "o must have q's strides"
+    close("o", o, ro)
+    assert (lse.cpu() - rl).abs().max() < 2e-3, f"lse differs by {(lse.cpu() - rl).abs().max():.3e}"
+    got = attn_bwd(do, q, k, v, pk.to(dev), pv.to(dev), o, lse, idx.int().to(dev), weight, 1.0)
+    ref = O.attn_bwd_l1(doc, qc, kc, vc, pk, pv, o.cpu(), lse.cpu(), idx, weight)
+    for name, a, b in zip(("dq", "dk", "dv", "dpk", "dpv"), got, ref):
+        close(name, a, b)
+
+
+def check_attn_l2(dev, B=1, H=1, N=16384, T=8, T2=4, smooth=False):
+    from llsa_amd.kernel.hip._attention import attn_bwd, attn_fwd
+    q, k, v, do = smooth_inputs(B, H, N, 64, dev) if smooth else randn_inputs(B, H, N, 64, dev, seed=15)
+    qc, kc, vc, doc = (t.cpu() for t in (q, k, v, do))
+    pq, pk, pv = O.mean_pool(qc), O.mean_pool(kc), O.mean_pool(vc)
+    pq2, pk2, pv2 = O.mean_pool(pq), O.mean_pool(pk), O.mean_pool(pv)
+    pidx = O.topk_lowest_index(O.dense_scores(pq2, pk2), T2)
+    idx = O.topk_sparse(pq, pk, pidx, T)
+    d = lambda t: t.to(dev)
+    o, lse = attn_fwd(q, k, v, d(pk), d(pv), d(idx), 16.0, pk2=d(pk2), pv2=d(pv2), p_indices=d(pidx.int()),
+                      token_weight_2=256.0)
+    ro, rl = O.attn_fwd_l2(qc, kc, vc, pk, pv, pk2, pv2, idx, pidx)
+    close("o", o, ro)
+    assert (lse.cpu() - rl).abs().max() < 2e-3
+    got = attn_bwd(do, q, k, v, d(pk), d(pv), o, lse, d(idx), 16.0, 16.0, pk2=d(pk2), pv2=d(pv2),
+                   p_indices=d(pidx.int()), token_weight_2=256.0)
+    ref = O.attn_bwd_l2(doc, qc, kc, vc, pk, pv, pk2, pv2, o.cpu(), lse.cpu(), idx, pidx)
+    for name, a, b in zip(("dq", "dk", "dv", "dpk", "dpv", "dpk2", "dpv2"), got, ref):
+        close(name, a, b)
+
+
+def check_attn_reduces_to_sdpa(dev, B=1, H=2, N=1024):
+    """All blocks selected and a vanishing pooled weight: the kernel must equal dense attention."""
+    import torch.nn.functional as F
+    from llsa_amd.kernel.hip._attention import attn_fwd
+    q, k, v, _ = randn_inputs(B, H, N, 64, dev, seed=16)
+    N1 = N // 16
+    g = torch.Generator().manual_seed(17)
+    idx = torch.stack([torch.randperm(N1, generator=g) for _ in range(B * H * N1)]).reshape(B, H, N1, N1).int()
+    pk, pv = O.mean_pool(k.cpu()).to(dev), O.mean_pool(v.cpu()).to(dev)
+    o, lse = attn_fwd(q, k, v, pk, pv, idx.to(dev), 2.0 ** -60)
+    ref = F.scaled_dot_product_attention(q.cpu().float(), k.cpu().float(), v.cpu().float())
+    close("o vs sdpa", o, ref)
+    rl = torch.logsumexp(q.cpu().float() @ k.cpu().float().transpose(-1, -2) / 8.0, -1)
+    assert (lse.cpu() - rl).abs().max() < 2e-3
+
+
+def check_constant_v(dev, N=1024):
+    from llsa_amd.kernel.hip._attention import attn_fwd
+    q, k, _, _ = randn_inputs(1, 1, N, 64, dev, seed=18)
+    v = torch.full((1, 1, N, 64), 0.75, dtype=torch.bfloat16, device=dev)
+    idx = _selection_l1(q, k, 4)
+    o, _ = attn_fwd(q, k, v, O.mean_pool(k.cpu()).to(dev), O.mean_pool(v.cpu()).to(dev), idx.int().to(dev), 16.0)
+    assert (o.float() - 0.75).abs().max() < 4e-3
+
+
+# ------------------------------------------------------------------------------------------
+def _grads(fn, q, k, v, do):
+    q, k, v = (t.detach().requires_grad_(True) for t in (q, k, v))
+    o = fn(q, k, v)
+    o.backward(do)
+    return o.detach(), q.grad, k.grad, v.grad
+
+
+def check_op_l1(dev, B=1, H=2, N=1024, T=8, fused=True, rope=False, strided=False, smooth=False):
+    """The whole operator through autograd, against the oracle's composition fed with the
+    indices the device selected (selection itself is checked separately)."""
+    from llsa_amd.kernel.hip.rope import my_rope_fn
+    from llsa_amd.kernel.torch_op import flash_sparse_attention_res_1 as M
+    from llsa_amd.utils.rope_table import rope_table
+    q, k, v, do = smooth_inputs(B, H, N, 64, dev) if smooth else randn_inputs(B, H, N, 64, dev, seed=19, strided=strided)
+    freq = rope_table(int(math.isqrt(N)), dtype=torch.bfloat16).to(dev) if rope else None
+    captured = {}
+
+    def run(q_, k_, v_):
+        if fused:
+            out = M.llsa_l1(q_, k_, v_, T, 16, rope=freq)
+            captured["idx"] = out.grad_fn.indices
+            return out
+        if rope:
+            q_, k_ = my_rope_fn(q_, freq), my_rope_fn(k_, freq)
+        out = M.llsa_l1_unfused(q_, k_, v_, T, 16)
+        captured["idx"] = out.grad_fn.saved_tensors[7]
+        return out
+
+    o, dq, dk, dv = _grads(run, q, k, v, do)
+    qc, kc, vc, doc = (t.cpu() for t in (q, k, v, do))
+    fc = freq.cpu() if rope else None
+    qr, kr = (O.rope_apply(qc, fc), O.rope_apply(kc, fc)) if rope else (qc, kc)
+    idx = captured["idx"].cpu().long()
+    ro, ctx = O.llsa_l1_fwd(qr, kr, vc, T, 16, indices=idx)
+    rq, rk, rv, _ = O.llsa_l1_bwd(doc, ctx)
+    if rope:
+        rq, rk = O.rope_apply_bwd(rq, fc), O.rope_apply_bwd(rk, fc)
+    close("o", o, ro)
+    close("dq", dq, rq)
+    close("dk", dk, rk)
+    close("dv", dv, rv)
+    # and the device's selection is a legal top-k of the oracle's scores
+    sc = O.dense_scores(ctx["pq"], ctx["pk"])
+    kth = torch.sort(sc, -1, descending=True).values[..., T - 1:T]
+    picked = torch.gather(sc, -1, idx)
+    assert (picked >= kth - 2.0 ** -6 * kth.abs().clamp_min(1.0)).all(), "selected a block below the top-k threshold"
+
+
+def check_op_l2(dev, B=1, H=1, N=16384, T=8, T2=4, fused=True, rope=False, smooth=False):
+    from llsa_amd.kernel.hip.rope import my_rope_fn
+    from llsa_amd.kernel.torch_op import flash_sparse_attention_res_2 as M
+    from llsa_amd.utils.rope_table import rope_table
+    q, k, v, do = smooth_inputs(B, H, N, 64, dev) if smooth else randn_inputs(B, H, N, 64, dev, seed=20)
+    freq = rope_table(int(math.isqrt(N)), dtype=torch.bfloat16).to(dev) if rope else None
+    captured = {}
+
+    def run(q_, k_, v_):
+        if fused:
+            out = M.llsa_l2(q_, k_, v_, T, T2, 16, rope=freq)
+            captured["idx"], captured["pidx"] = out.grad_fn.indices, out.grad_fn.p_indices
+            return out
+        if rope:
+            q_, k_ = my_rope_fn(q_, freq), my_rope_fn(k_, freq)
+        out = M.llsa_l2_unfused(q_, k_, v_, T, T2, 16)
+        captured["idx"], captured["pidx"] = out.grad_fn.saved_tensors[9], out.grad_fn.saved_tensors[10]
+        return out
+
+    o, dq, dk, dv = _grads(run, q, k, v, do)
+    qc, kc, vc, doc = (t.cpu() for t in (q, k, v, do))
+    fc = freq.cpu() if rope else None
+    qr, kr = (O.rope_apply(qc, fc), O.rope_apply(kc, fc)) if rope else (qc, kc)
+    ro, ctx = O.llsa_l2_fwd(qr, kr, vc, T, T2, 16, indices=captured["idx"].cpu(), p_indices=captured["pidx"].cpu().long())
+    rq, rk, rv, _ = O.llsa_l2_bwd(doc, ctx)
+    if rope:
+        rq, rk = O.rope_apply_bwd(rq, fc), O.rope_apply_bwd(rk, fc)
+    close("o", o, ro)
+    close("dq", dq, rq)
+    close("dk", dk, rk)
+    close("dv", dv, rv)

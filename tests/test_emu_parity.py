@@ -1,0 +1,75 @@
+"""The parity cases of tests/parity_cases.py at tiny sizes on the CPU, through the x86
+emulation build of the HIP sources (tests/cpu_emu).  This checks index arithmetic, operand
+layouts and the Python/autograd glue without a GPU; the GPU run of the same cases is
+tests/test_gpu_parity.py."""
+import pytest
+import torch
+
+import parity_cases as P
+from emu_util import emu_lib
+from llsa_amd._lib import override_library_for_tests
+
+DEV = torch.device("cpu")
+
+
+@pytest.fixture(autouse=True)
+def _emu():
+    with override_library_for_tests(emu_lib()):
+        yield
+
+
+def test_pool_pyramid():
+    P.check_pool_pyramid(DEV, N=512, strided=True, rope=True)
+    P.check_pool_pyramid(DEV, N=256, strided=False, rope=False)
+
+
+def test_mean_pool1d():
+    P.check_mean_pool1d(DEV, torch.bfloat16, 16, 64, 64, 'bhsc')
+    P.check_mean_pool1d(DEV, torch.float32, 4, 24, 32, 'bhsc')
+    P.check_mean_pool1d(DEV, torch.bfloat16, 8, 100, 32, 'bsc')
+
+
+def test_rope():
+    P.check_rope(DEV, side=8, strided=True)
+
+
+def test_topk_dense():
+    P.check_topk_dense(DEV, n=64, T=8, round_scores=True)
+    P.check_topk_dense(DEV, n=64, T=8, round_scores=False, min_safe=0.9)
+    P.check_topk_dense_ties(DEV)
+
+
+def test_topk_dense_multi_chunk():
+    P.check_topk_dense(DEV, B=1, H=1, n=1088, T=16, round_scores=False, min_safe=0.9)
+
+
+def test_topk_sparse():
+    P.check_topk_sparse(DEV, N1=256, T=8, T2=4)
+
+
+def test_transpose():
+    P.check_transpose(DEV, Mb=64, T=8)
+    P.check_transpose(DEV, B=1, H=1, Mb=64, T=4, Kb=16)
+    P.check_transpose_hot_block(DEV)
+
+
+def test_attn_l1():
+    P.check_attn_l1(DEV, B=1, H=2, N=1024, T=8, strided=True)
+
+
+def test_attn_special_cases():
+    P.check_attn_reduces_to_sdpa(DEV, B=1, H=1, N=1024)
+    P.check_constant_v(DEV)
+
+
+@pytest.mark.parametrize("fused,rope", [(True, False), (True, True), (False, False)])
+def test_op_l1(fused, rope):
+    P.check_op_l1(DEV, B=1, H=1, N=1024, T=8, fused=fused, rope=rope, strided=True)
+
+
+def test_attn_l2():
+    P.check_attn_l2(DEV, B=1, H=1, N=16384, T=4, T2=4)
+
+
+def test_op_l2_fused_rope():
+    P.check_op_l2(DEV, B=1, H=1, N=16384, T=4, T2=4, fused=True, rope=True)

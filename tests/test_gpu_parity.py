@@ -1,0 +1,99 @@
+"""GPU parity: the HIP kernels (through libllsa_hip.so and the Python operator API) against
+the CPU oracle on the same seeded inputs.  Run with `pytest -m gpu` on an MI355X."""
+import pytest
+import torch
+
+import parity_cases as P
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available()
+    from llsa_amd._lib import get_lib
+    get_lib()                       # fails loudly if the HIP library is not built
+    return torch.device("cuda:0")
+
+
+def test_library_loaded(dev):
+    from llsa_amd._lib import EXPORTS, get_lib
+    lib = get_lib()
+    assert lib.device_library and lib.version() >= 100
+    for name in EXPORTS:
+        assert hasattr(lib.cdll, name)
+
+
+def test_cpu_tensors_are_rejected(dev):
+    import llsa_amd
+    x = torch.randn(1, 1, 1024, 64).bfloat16()
+    with pytest.raises(RuntimeError, match="GPU only"):
+        llsa_amd.llsa_l1(x, x, x, 8, 16)
+
+
+@pytest.mark.parametrize("N,strided,rope", [(512, True, True), (4096, False, False), (16384, True, True)])
+def test_pool_pyramid(dev, N, strided, rope):
+    P.check_pool_pyramid(dev, B=2, H=3, N=N, strided=strided, rope=rope)
+
+
+def test_mean_pool1d(dev):
+    P.check_mean_pool1d(dev, torch.bfloat16, 16, 64, 1024, 'bhsc')
+    P.check_mean_pool1d(dev, torch.float32, 4, 24, 32, 'bhsc')
+    P.check_mean_pool1d(dev, torch.bfloat16, 8, 100, 64, 'bsc')
+
+
+def test_rope(dev):
+    P.check_rope(dev, B=2, H=3, side=32, strided=True)
+    P.check_rope(dev, B=1, H=2, side=8, strided=False)
+
+
+def test_topk_dense(dev):
+    P.check_topk_dense(dev, B=2, H=3, n=256, T=16, round_scores=True)
+    P.check_topk_dense(dev, B=1, H=2, n=64, T=16, round_scores=False, min_safe=0.9)
+    P.check_topk_dense(dev, B=1, H=2, n=1024, T=16, round_scores=False, min_safe=0.9)
+    P.check_topk_dense_ties(dev)
+
+
+def test_topk_sparse(dev):
+    P.check_topk_sparse(dev, B=2, H=3, N1=1024, T=16, T2=16)
+    P.check_topk_sparse(dev, B=1, H=1, N1=256, T=8, T2=4)
+
+
+def test_transpose(dev):
+    P.check_transpose(dev, B=2, H=3, Mb=1024, T=16)
+    P.check_transpose(dev, B=1, H=2, Mb=64, T=16)
+    P.check_transpose(dev, B=1, H=1, Mb=64, T=4, Kb=16)
+    P.check_transpose_hot_block(dev)
+
+
+def test_transpose_largest(dev):
+    P.check_transpose(dev, B=1, H=1, Mb=16384, T=16)
+
+
+@pytest.mark.parametrize("strided,smooth", [(False, False), (True, False), (False, True)])
+def test_attn_l1(dev, strided, smooth):
+    P.check_attn_l1(dev, B=2, H=3, N=4096, T=16, strided=strided, smooth=smooth)
+
+
+def test_attn_l1_small(dev):
+    P.check_attn_l1(dev, B=1, H=2, N=1024, T=8)
+
+
+def test_attn_special_cases(dev):
+    P.check_attn_reduces_to_sdpa(dev, B=1, H=2, N=1024)
+    P.check_constant_v(dev)
+
+
+@pytest.mark.parametrize("smooth", [False, True])
+def test_attn_l2(dev, smooth):
+    P.check_attn_l2(dev, B=1, H=2, N=16384, T=16, T2=16, smooth=smooth)
+
+
+@pytest.mark.parametrize("fused,rope,strided", [(True, False, False), (True, True, True), (False, False, True), (False, True, False)])
+def test_op_l1(dev, fused, rope, strided):
+    P.check_op_l1(dev, B=2, H=2, N=4096, T=16, fused=fused, rope=rope, strided=strided, smooth=not strided)
+
+
+@pytest.mark.parametrize("fused,rope", [(True, False), (True, True), (False, True)])
+def test_op_l2(dev, fused, rope):
+    P.check_op_l2(dev, B=1, H=2, N=16384, T=16, T2=16, fused=fused, rope=rope, smooth=True)
