@@ -1,0 +1,285 @@
+#!/usr/bin/env python3
+"""Benchmark of the llsa hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c5|n65536] [--no-extras]
+
+A step is one forward + backward of the operator on one batch of synthetic input that is
+already resident in HBM.  The default workload is the configuration the headline metric is
+quoted on: llsa_l2, B=2, H=6, N=16384 (128x128 Z-ordered), D=64, bf16, topk 16/16, 2-D RoPE
+applied in-kernel, smooth-field inputs, dO ~ N(0,1).
+
+One JSON line is printed:
+  value        effective TFLOP/s = 14*B*H*N*D*n_kv / step time (algorithmic FLOPs: forward 4, backward 10)
+  ms_per_step  forward + backward wall time per step
+  roofline     the dominant kernel of the step, timed with HIP events on the launch stream in a
+               second pass that runs the same kernels stage by stage
+  cpu_baseline the CPU oracle (plain PyTorch restatement) on the host cores, same workload in fp32
+  kernels      per-stage times of that second pass (ms), with the achieved rate of each
+  dense_sdpa   F.scaled_dot_product_attention forward+backward on the same shapes, same GPU
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+
+WORKLOADS = {
+    # name: (op, B, H, N, topk1, topk2, rope)
+    "c2": ("l1", 4, 6, 4096, 16, 0, False),
+    "c3": ("l2", 2, 6, 16384, 16, 16, True),
+    "c5": ("l2", 1, 6, 262144, 16, 16, True),
+    "n65536": ("l2", 1, 6, 65536, 16, 16, True),
+}
+
+
+def n_kv(op, N, t1, t2):
+    return 16 * t1 + N // 16 if op == "l1" else 16 * t1 + 16 * t2 + N // 256
+
+
+def make_inputs(B, H, N, D, dev):
+    import torch
+    from llsa_amd.utils.synth import smooth_field
+    q = smooth_field(1, B, H, N, D).to(dev)
+    k = smooth_field(2, B, H, N, D).to(dev)
+    v = smooth_field(3, B, H, N, D).to(dev)
+    do = torch.randn(B, H, N, D, generator=torch.Generator().manual_seed(4)).bfloat16().to(dev)
+    return q, k, v, do
+
+
+def timed(fn, iters, torch):
+    """Average ms of fn() over iters calls, HIP events on the current stream."""
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
+def stage_profile(op, q, k, v, do, t1, t2, freq, iters, torch):
+    """Runs the kernels of one forward + backward one stage at a time, the same launches the
+    fused operator makes, and times each stage with events on the launch stream."""
+    from llsa_amd.kernel.hip import _attention as A
+    from llsa_amd.kernel.hip.indices_transpose import transpose_indices
+    from llsa_amd.kernel.hip.mean_pool import PoolSpec, block_transpose, pool_bwd_accum, pool_pyramid
+    from llsa_amd.kernel.hip.topk import compute_topk_indices_sparse, gen_sparse_indices
+    B, H, N, D = q.shape
+    l2 = op == "l2"
+    rope = freq is not None
+    res = {}
+
+    def pyramid():
+        return pool_pyramid([PoolSpec(q, y1=True, y2=l2, xt=True, rope=rope),
+                             PoolSpec(k, y1=True, y2=l2, xt=True, y1t=True, rope=rope),
+                             PoolSpec(v, y1=True, y2=l2, xt=True, y1t=True)], freq)
+
+    oq, ok, ov = pyramid()
+    res["pool_pyramid"] = timed(pyramid, iters, torch)
+    qr, kr = (oq["xrot"], ok["xrot"]) if rope else (q, k)
+    pq, pk, pv = oq["y1"], ok["y1"], ov["y1"]
+    if l2:
+        pq2, pk2, pv2 = oq["y2"], ok["y2"], ov["y2"]
+        pv2t, pk2t = block_transpose(pv2, pk2)
+        res["pool_level2_transpose"] = timed(lambda: block_transpose(pv2, pk2), iters, torch)
+        pidx = gen_sparse_indices(pq2, pk2, t2)
+        res["topk_dense"] = timed(lambda: gen_sparse_indices(pq2, pk2, t2), iters, torch)
+        idx = compute_topk_indices_sparse(pq, pk, pidx, t1, t2)
+        res["topk_sparse"] = timed(lambda: compute_topk_indices_sparse(pq, pk, pidx, t1, t2), iters, torch)
+        kw = dict(pk2=pk2, pv2=pv2, p_indices=pidx, token_weight_2=256.0)
+        fkw = dict(kw, vt=ov["xt"], pvt=ov["y1t"], pv2t=pv2t)
+        cgw = 16.0
+    else:
+        pidx = None
+        idx = gen_sparse_indices(pq, pk, t1)
+        res["topk_dense"] = timed(lambda: gen_sparse_indices(pq, pk, t1), iters, torch)
+        kw = {}
+        fkw = dict(vt=ov["xt"], pvt=ov["y1t"])
+        cgw = 1.0
+        pk2t = None
+    o, lse = A.attn_fwd(qr, kr, v, pk, pv, idx, 16.0, **fkw)
+    res["attn_fwd"] = timed(lambda: A.attn_fwd(qr, kr, v, pk, pv, idx, 16.0, **fkw), iters, torch)
+
+    def transposes():
+        r = transpose_indices(idx, N // 16)
+        return r + transpose_indices(pidx, N // 256) if l2 else r
+
+    csr = transposes()
+    res["transpose_indices"] = timed(transposes, iters, torch)
+    bkw = dict(kw, qt=oq["xt"], kt=ok["xt"], pkt=ok["y1t"], pk2t=pk2t, csr=csr)
+    run = lambda st, f=None: A.attn_bwd(do, qr, kr, v, pk, pv, o, lse, idx, 16.0, cgw, stages=st, freq_dq=f, **bkw)
+    run(1)
+    for name, st in (("bwd_delta_dOt", 1), ("bwd_dq", 2), ("bwd_dkv", 4), ("bwd_dpkv1_sparse", 8), ("bwd_dpkv_dense", 16)):
+        if st == 8 and not l2:
+            continue
+        # a stage run alone reads whatever workspace the allocator hands back (the block stage 1
+        # just filled); only its duration is used
+        res[name] = timed(lambda: run(st, freq if st == 2 else None), iters, torch)
+    outs = run(0, freq)
+    dk, dv, dpk, dpv = outs[1], outs[2], outs[3], outs[4]
+    dpk2, dpv2 = (outs[5], outs[6]) if l2 else (None, None)
+    res["pool_bwd_accum"] = timed(lambda: (pool_bwd_accum(dk, dpk, dpk2, freq), pool_bwd_accum(dv, dpv, dpv2, None)),
+                                  iters, torch)
+    return res
+
+
+def cpu_baseline(op, B, H, N, D, t1, t2, rope):
+    """The CPU oracle (plain PyTorch restatement of the reference's algorithm), forward + backward in
+    fp32 on the host cores, on the same synthetic inputs."""
+    import torch
+    from llsa_amd.utils.synth import smooth_field
+    from oracle import llsa_oracle as O
+    # whole workload when it is small enough for ~20 s of CPU time, else one (b,h) slice; the
+    # oracle is run slice by slice to bound its memory
+    Bs, Hs = (B, H) if N <= 16384 else (1, 1)
+    q, k, v = (smooth_field(s, Bs, Hs, N, D).float() for s in (1, 2, 3))
+    do = torch.randn(Bs, Hs, N, D, generator=torch.Generator().manual_seed(4))
+    if rope:
+        freq = O.rope_table(math.isqrt(N), dtype=torch.float32)
+    reps, t_best, t0_all = 0, float("inf"), time.time()
+    while reps < 3 and (time.time() - t0_all) < 20.0:
+        t0 = time.time()
+        for b in range(Bs):
+            for h in range(Hs):
+                qs, ks, vs, ds = (t[b:b + 1, h:h + 1] for t in (q, k, v, do))
+                qr, kr = (O.rope_apply(qs, freq), O.rope_apply(ks, freq)) if rope else (qs, ks)
+                if op == "l2":
+                    o, ctx = O.llsa_l2_fwd(qr, kr, vs, t1, t2)
+                    dq, dk, dv, _ = O.llsa_l2_bwd(ds, ctx)
+                else:
+                    o, ctx = O.llsa_l1_fwd(qr, kr, vs, t1)
+                    dq, dk, dv, _ = O.llsa_l1_bwd(ds, ctx)
+                if rope:
+                    dq, dk = O.rope_apply_bwd(dq, freq), O.rope_apply_bwd(dk, freq)
+        t_best = min(t_best, time.time() - t0)
+        reps += 1
+    flops = 14.0 * Bs * Hs * N * D * n_kv(op, N, t1, t2)
+    return {"value": flops / t_best / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"oracle llsa_{op} fwd+bwd fp32, B={Bs} H={Hs} N={N} (best of {reps}), {t_best * 1e3:.0f} ms",
+            "ms": t_best * 1e3}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-extras", action="store_true", help="skip stage profile, CPU baseline and dense SDPA")
+    ap.add_argument("--unfused", action="store_true", help="use the reference's composition (separate pools, autograd adds)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (one MI355X per box); --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    import llsa_amd
+    from llsa_amd._lib import get_lib
+    from llsa_amd.utils.rope_table import rope_table
+    get_lib()
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    dev = torch.device("cuda:0")
+    op, B, H, N, t1, t2, rope = WORKLOADS[args.workload]
+    D = 64
+    q, k, v, do = make_inputs(B, H, N, D, dev)
+    freq = rope_table(math.isqrt(N), dtype=torch.bfloat16).to(dev) if rope else None
+    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+
+    def step():
+        q.grad = k.grad = v.grad = None
+        if args.unfused:
+            qq, kk = (llsa_amd.my_rope_fn(q, freq), llsa_amd.my_rope_fn(k, freq)) if rope else (q, k)
+            o = llsa_amd.llsa_l2_unfused(qq, kk, v, t1, t2, 16) if op == "l2" else llsa_amd.llsa_l1_unfused(qq, kk, v, t1, 16)
+        else:
+            o = llsa_amd.llsa_l2(q, k, v, t1, t2, 16, rope=freq) if op == "l2" else llsa_amd.llsa_l1(q, k, v, t1, 16, rope=freq)
+        o.backward(do)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    nkv = n_kv(op, N, t1, t2)
+    unit_flops = B * H * N * D * nkv                    # one "GEMM unit": 2 * this = one product
+    flops = 14.0 * unit_flops
+    out = {
+        "metric": f"llsa_{op} fwd+bwd effective TFLOP/s at N={N}, D={D}, bf16",
+        "value": flops / (ms * 1e-3) / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload}: llsa_{op} fwd+bwd B={B} H={H} N={N} D={D} block_size=16 topk={t1}"
+                               + (f"/{t2}" if op == "l2" else "") + (" rope=in-kernel" if rope else "")
+                               + (" (unfused composition)" if args.unfused else ""),
+                   "n_kv_per_query": nkv, "algorithmic_gflop": flops / 1e9},
+        "frac_of_bf16_mfma_peak": flops / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+    }
+
+    if not args.no_extras:
+        prof_iters = max(5, min(args.steps, 20))
+        with torch.no_grad():
+            st = stage_profile(op, q.detach(), k.detach(), v.detach(), do, t1, t2, freq, prof_iters, torch)
+        alg = {"attn_fwd": 4.0 * unit_flops, "bwd_dq": 6.0 * unit_flops, "bwd_dkv": 4.0 * B * H * N * D * 16 * t1}
+        if op == "l2":
+            alg["bwd_dpkv1_sparse"] = 4.0 * B * H * N * D * 16 * t2
+            alg["bwd_dpkv_dense"] = 4.0 * B * H * N * D * (N // 256)
+        else:
+            alg["bwd_dpkv_dense"] = 4.0 * B * H * N * D * (N // 16)
+        el = 2 * B * H * N * D
+        hbm = {"pool_pyramid": 3 * el * (1 + 1 / 16 + (1 / 256 if op == "l2" else 0)),
+               "pool_bwd_accum": 2 * 2 * el, "bwd_delta_dOt": 2 * el + 4 * B * H * N}
+        kernels = {}
+        for name, t in st.items():
+            e = {"ms": t}
+            if name in alg:
+                e["tflops"] = alg[name] / (t * 1e-3) / 1e12
+                e["frac_mfma_peak"] = e["tflops"] / PEAK_BF16_TFLOPS
+            if name in hbm:
+                e["gbs"] = hbm[name] / (t * 1e-3) / 1e9
+                e["frac_hbm_peak"] = e["gbs"] / PEAK_HBM_GBS
+            kernels[name] = e
+        out["kernels"] = kernels
+        out["stage_sum_ms"] = sum(st.values())
+        dom = max(alg, key=lambda n: st[n])
+        out["roofline"] = {"kernel": dom, "bound": "mfma", "achieved": kernels[dom]["tflops"], "peak": PEAK_BF16_TFLOPS,
+                           "unit": "TFLOP/s", "frac": kernels[dom]["frac_mfma_peak"], "traffic": None,
+                           "avg_launch_ms": st[dom], "algorithmic_gflop_per_launch": alg[dom] / 1e9}
+        out["roofline_hbm"] = {"kernel": "pool_pyramid", "bound": "hbm", "achieved": kernels["pool_pyramid"]["gbs"],
+                               "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": kernels["pool_pyramid"]["frac_hbm_peak"],
+                               "traffic": None}
+        # dense attention on the same GPU
+        try:
+            import torch.nn.functional as F
+            qd, kd, vd = (t.detach().clone().requires_grad_(True) for t in (q, k, v))
+
+            def dense():
+                qd.grad = kd.grad = vd.grad = None
+                F.scaled_dot_product_attention(qd, kd, vd).backward(do)
+
+            for _ in range(2):
+                dense()
+            torch.cuda.synchronize()
+            n_d = 3 if N > 16384 else 10
+            t_d = timed(dense, n_d, torch)
+            out["dense_sdpa"] = {"ms_per_step": t_d, "speedup_llsa_over_dense": t_d / ms,
+                                 "dense_tflops": 14.0 * B * H * N * D * N / (t_d * 1e-3) / 1e12}
+        except Exception as e:                      # dense attention may not fit at the largest sizes
+            out["dense_sdpa"] = {"error": str(e)[:200]}
+        out["cpu_baseline"] = cpu_baseline(op, B, H, N, D, t1, t2, rope)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -165,7 +165,15 @@ typedef struct llsa_attn_bwd_args {
     const void* freq_dq;                         /* (N,64) or NULL: rotate dq back (fused rope)   */
     int32_t B, H, N, T, T2, levels;
     float w1, w2, cgw1;
+    int32_t stages;                              /* 0 = everything; else a mask of LLSA_BWD_* to
+                                                    launch only those kernels (profiling)        */
 } llsa_attn_bwd_args;
+
+#define LLSA_BWD_PRE 1      /* delta + block-transposed dO (everything below needs it)           */
+#define LLSA_BWD_DQ 2
+#define LLSA_BWD_DKV 4      /* dK/dV of the fine tokens                                          */
+#define LLSA_BWD_DPKV1 8    /* sparse level-1 pooled gradients (levels == 2)                     */
+#define LLSA_BWD_DENSE 16   /* dense coarsest pooled gradients (partials + reduction)            */
 
 int64_t llsa_attn_bwd_workspace_bytes(int B, int H, int N, int levels);
 int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream);

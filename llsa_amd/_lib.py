@@ -51,7 +51,7 @@ class AttnBwdArgs(C.Structure):
         + [("dpk", c_void_p), ("dpv", c_void_p), ("dpk2", c_void_p), ("dpv2", c_void_p),
            ("workspace", c_void_p), ("workspace_bytes", c_int64), ("freq_dq", c_void_p),
            ("B", c_int32), ("H", c_int32), ("N", c_int32), ("T", c_int32), ("T2", c_int32), ("levels", c_int32),
-           ("w1", c_float), ("w2", c_float), ("cgw1", c_float)])
+           ("w1", c_float), ("w2", c_float), ("cgw1", c_float), ("stages", c_int32)])
 
 
 P64 = C.POINTER(c_int64)

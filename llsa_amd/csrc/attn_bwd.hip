@@ -185,6 +185,7 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, cons
     for (int dt = 0; dt < 4; dt++) {
         bf16x4 o = cvt4(dq[dt] * kScale);
         if (fq != nullptr) {                    // rotate the gradient back: [sin, cos] pairs
+#pragma clang fp contract(off)
             const bf16x4 f = ld8(fq + dt * 16);
             bf16x4 y;
 #pragma unroll
@@ -450,8 +451,9 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     ws += align256((int64_t)d.chunks * BH * d.n_tok * 64 * 4);
     float* part_v = (float*)ws;
 
-    hipLaunchKernelGGL(bwd_pre_kernel, dim3((N1 + 15) / 16, BH), dim3(128), 0, s, *a, delta, dot);
-    hipLaunchKernelGGL(attn_dq_kernel, dim3((N1 + 3) / 4, BH), dim3(256), 0, s, *a, (const float*)delta);
+    const int stages = a->stages ? a->stages : 0x7fffffff;
+    if (stages & LLSA_BWD_PRE) hipLaunchKernelGGL(bwd_pre_kernel, dim3((N1 + 15) / 16, BH), dim3(128), 0, s, *a, delta, dot);
+    if (stages & LLSA_BWD_DQ) hipLaunchKernelGGL(attn_dq_kernel, dim3((N1 + 3) / 4, BH), dim3(256), 0, s, *a, (const float*)delta);
 
     KSideParams p;
     p.q = (const bf16*)a->q; p.sqb = a->sqb; p.sqh = a->sqh; p.sqn = a->sqn;
@@ -466,11 +468,12 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     p.dk = (bf16*)a->dk; p.sdkb = a->sdkb; p.sdkh = a->sdkh; p.sdkn = a->sdkn;
     p.dv = (bf16*)a->dv; p.sdvb = a->sdvb; p.sdvh = a->sdvh; p.sdvn = a->sdvn;
     p.n_units = N1; p.w = 1.f;
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_FINE>), dim3((N1 + 3) / 4, BH), dim3(256), 0, s, p);
+    if (stages & LLSA_BWD_DKV)
+        hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_FINE>), dim3((N1 + 3) / 4, BH), dim3(256), 0, s, p);
 
     const int64_t s1b = (int64_t)H * N1 * 64, s1h = (int64_t)N1 * 64;
     const int64_t s2b = (int64_t)H * N2 * 64, s2h = (int64_t)N2 * 64;
-    if (a->levels == 2) {
+    if (a->levels == 2 && (stages & LLSA_BWD_DPKV1)) {
         // level-1 pooled tokens, through the transposed coarse index
         p.kk = (const bf16*)a->pk; p.skb = s1b; p.skh = s1h; p.skn = 64;
         p.vv = (const bf16*)a->pv; p.svb = s1b; p.svh = s1h; p.svn = 64;
@@ -481,6 +484,7 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
         hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_SPARSE1>), dim3(N2, BH), dim3(256), 0, s, p);
     }
     // dense coarsest level
+    if (!(stages & LLSA_BWD_DENSE)) return launch_status("attn_bwd");
     if (a->levels == 2) {
         p.kk = (const bf16*)a->pk2; p.skb = s2b; p.skh = s2h; p.skn = 64;
         p.vv = (const bf16*)a->pv2; p.svb = s2b; p.svh = s2h; p.svn = 64;

@@ -11,7 +11,11 @@ namespace llsa {
 // rotation of one 8-channel chunk (4 interleaved pairs) with bf16 rounding after every
 // multiply and add, the arithmetic the reference performs in the tensor dtype
 // ---------------------------------------------------------------------------------------
+//
+// Contraction must stay off here: with it the compiler narrows the fp32 expression to bf16
+// arithmetic and then fuses multiply and add into one bf16 FMA, i.e. one rounding fewer.
 __device__ __forceinline__ bf16x8 rope_chunk_fwd(bf16x8 x, bf16x8 f) {
+#pragma clang fp contract(off)
     bf16x8 y;
 #pragma unroll
     for (int j = 0; j < 4; j++) {
@@ -23,6 +27,7 @@ __device__ __forceinline__ bf16x8 rope_chunk_fwd(bf16x8 x, bf16x8 f) {
     return y;
 }
 __device__ __forceinline__ bf16x8 rope_chunk_bwd(bf16x8 g, bf16x8 f) {
+#pragma clang fp contract(off)
     bf16x8 y;
 #pragma unroll
     for (int j = 0; j < 4; j++) {

@@ -67,10 +67,11 @@ def attn_fwd(q, k, v, pk, pv, indices, token_weight, pk2=None, pv2=None, p_indic
 
 def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_weight, pk2=None, pv2=None,
              p_indices=None, token_weight_2=1.0, qt=None, kt=None, pkt=None, pk2t=None,
-             freq_dq: Optional[torch.Tensor] = None):
+             freq_dq: Optional[torch.Tensor] = None, stages: int = 0, csr=None):
     """Backward.  Returns (dq, dk, dv, dpk, dpv[, dpk2, dpv2]) with the reference's conventions:
     every gradient is `empty_like` of its primal; the pooled gradients are NOT yet folded
-    into dk / dv (autograd, or pool_bwd_accum, does that)."""
+    into dk / dv (autograd, or pool_bwd_accum, does that).  `stages` (a mask of the LLSA_BWD_*
+    bits of include/llsa_hip.h) launches only some of the kernels, for profiling."""
     levels = 1 if pk2 is None else 2
     lib = lib_for(do, q, k, v, pk, pv, pk2, pv2, o, lse)
     require_bf16(do, q, k, v, pk, pv, pk2, pv2, o)
@@ -94,10 +95,16 @@ def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_wei
         if levels == 2 and pk2t is None:
             pk2t = next(got)
     idx = indices.to(torch.int32).contiguous()
-    off, flat = transpose_indices(idx, N // BLOCK)
     if levels == 2:
         pidx = p_indices.to(torch.int32).contiguous()
-        poff, pflat = transpose_indices(pidx, N // (BLOCK * BLOCK))
+    if csr is not None:                       # (off, flat[, poff, pflat]) from transpose_indices
+        off, flat = csr[0], csr[1]
+        if levels == 2:
+            poff, pflat = csr[2], csr[3]
+    else:
+        off, flat = transpose_indices(idx, N // BLOCK)
+        if levels == 2:
+            poff, pflat = transpose_indices(pidx, N // (BLOCK * BLOCK))
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dpk, dpv = torch.empty_like(pk), torch.empty_like(pv)
     ws_bytes = lib.attn_bwd_workspace_bytes(B, H, N, levels)
@@ -130,5 +137,6 @@ def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_wei
         a.freq_dq = freq_dq.data_ptr()
     a.B, a.H, a.N, a.T, a.T2, a.levels = B, H, N, T, T2, levels
     a.w1, a.w2, a.cgw1 = float(token_weight), float(token_weight_2), float(coarse_grad_weight)
+    a.stages = stages
     lib.check(lib.attn_bwd(C.byref(a), stream_of(lib, q)), "attn_bwd")
     return tuple(outs)
