@@ -110,8 +110,8 @@ def stage_profile(op, q, k, v, do, t1, t2, freq, iters, torch):
     res["attn_fwd"] = timed(lambda: A.attn_fwd(qr, kr, v, pk, pv, idx, 16.0, **fkw), iters, torch)
 
     def transposes():
-        r = transpose_indices(idx, N // 16)
-        return r + transpose_indices(pidx, N // 256) if l2 else r
+        r = transpose_indices(idx, N // 16, 32)
+        return r + transpose_indices(pidx, N // 256, 8) if l2 else r
 
     csr = transposes()
     res["transpose_indices"] = timed(transposes, iters, torch)

@@ -129,8 +129,18 @@ int llsa_attn_fwd(const llsa_attn_fwd_args* a, void* stream);
  * flat lists the query blocks that selected key block n in ASCENDING order (the reference's
  * order is whatever its atomics produce).  Rows of idx must hold distinct values.
  * ---------------------------------------------------------------------------------------- */
-int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, int B, int H, int Mb, int Kb,
-                           int T, void* stream);
+int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, int32_t* work /* or NULL */,
+                           int B, int H, int Mb, int Kb, int T, int chunk, void* stream);
+
+/* Work list for the K-side backward kernels, written by llsa_transpose_indices when `work` is
+ * given: every key block's segment is cut into chunks of at most `chunk` entries, one work item
+ * per chunk, so that a key block selected by very many query blocks is spread over many waves
+ * (the reference walks each segment serially, sparse_attention_res_1.py:300-322).  `work` is
+ * (B,H,llsa_work_list_len(Mb,Kb,T,chunk)) int32; llsa_attn_bwd needs chunk = LLSA_CHUNK_FINE
+ * for idx and chunk = LLSA_CHUNK_COARSE for pidx. */
+int64_t llsa_work_list_len(int Mb, int Kb, int T, int chunk);
+#define LLSA_CHUNK_FINE 32
+#define LLSA_CHUNK_COARSE 8
 
 /* ------------------------------------------------------------------------------------------
  * Backward.  Replaces sparse_indices_attn_res_scatter_bwd_v2 (sparse_attention_res_1.py:403-471)
@@ -154,8 +164,8 @@ typedef struct llsa_attn_bwd_args {
     const void* pkt;                             /* block-transposed pk     (B,H,N/256,64,16)     */
     const void* pk2t;                            /* block-transposed pk2    (B,H,N/4096,64,16)    */
     const int32_t* idx;  const int32_t* pidx;
-    const int32_t* off;  const int32_t* flat;    /* transposed idx  (Kb = N/16)                   */
-    const int32_t* poff; const int32_t* pflat;   /* transposed pidx (Kb = N/256), levels == 2     */
+    const int32_t* off;  const int32_t* flat;  const int32_t* work;    /* transposed idx  (Kb = N/16)     */
+    const int32_t* poff; const int32_t* pflat; const int32_t* pwork;   /* transposed pidx (Kb = N/256)    */
     void* dq; int64_t sdqb, sdqh, sdqn;
     void* dk; int64_t sdkb, sdkh, sdkn;
     void* dv; int64_t sdvb, sdvh, sdvn;
@@ -175,7 +185,7 @@ typedef struct llsa_attn_bwd_args {
 #define LLSA_BWD_DPKV1 8    /* sparse level-1 pooled gradients (levels == 2)                     */
 #define LLSA_BWD_DENSE 16   /* dense coarsest pooled gradients (partials + reduction)            */
 
-int64_t llsa_attn_bwd_workspace_bytes(int B, int H, int N, int levels);
+int64_t llsa_attn_bwd_workspace_bytes(int B, int H, int N, int T, int T2, int levels);
 int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream);
 
 #ifdef __cplusplus

@@ -43,8 +43,8 @@ class AttnBwdArgs(C.Structure):
         + _t3("q") + _t3("k") + _t3("v") + _t3("o")
         + [("lse", c_void_p), ("pk", c_void_p), ("pv", c_void_p), ("pk2", c_void_p), ("pv2", c_void_p),
            ("qt", c_void_p), ("kt", c_void_p), ("pkt", c_void_p), ("pk2t", c_void_p),
-           ("idx", c_void_p), ("pidx", c_void_p), ("off", c_void_p), ("flat", c_void_p),
-           ("poff", c_void_p), ("pflat", c_void_p)]
+           ("idx", c_void_p), ("pidx", c_void_p), ("off", c_void_p), ("flat", c_void_p), ("work", c_void_p),
+           ("poff", c_void_p), ("pflat", c_void_p), ("pwork", c_void_p)]
         + [("dq", c_void_p), ("sdqb", c_int64), ("sdqh", c_int64), ("sdqn", c_int64),
            ("dk", c_void_p), ("sdkb", c_int64), ("sdkh", c_int64), ("sdkn", c_int64),
            ("dv", c_void_p), ("sdvb", c_int64), ("sdvh", c_int64), ("sdvn", c_int64)]
@@ -68,12 +68,14 @@ _SIGNATURES = {
     "llsa_topk_dense": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llsa_topk_sparse": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llsa_attn_fwd": (c_int, [C.POINTER(AttnFwdArgs), c_void_p]),
-    "llsa_transpose_indices": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
-    "llsa_attn_bwd_workspace_bytes": (c_int64, [c_int, c_int, c_int, c_int]),
+    "llsa_transpose_indices": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "llsa_work_list_len": (c_int64, [c_int, c_int, c_int, c_int]),
+    "llsa_attn_bwd_workspace_bytes": (c_int64, [c_int, c_int, c_int, c_int, c_int, c_int]),
     "llsa_attn_bwd": (c_int, [C.POINTER(AttnBwdArgs), c_void_p]),
 }
 
 EXPORTS = tuple(_SIGNATURES)
+CHUNK_FINE, CHUNK_COARSE = 32, 8          # LLSA_CHUNK_FINE / LLSA_CHUNK_COARSE of include/llsa_hip.h
 
 
 class LlsaError(RuntimeError):

@@ -216,11 +216,14 @@ struct KSideParams {
     const bf16* kk;  int64_t skb, skh, skn;       // the unit's key rows come from here
     const bf16* vv;  int64_t svb, svh, svn;
     const int* off;  const int* flat;             // CSR of the list (FINE: per K block, SPARSE1: per coarse block)
+    const int* work;                              // work list over that CSR (see transpose.hip)
     bf16* dk; int64_t sdkb, sdkh, sdkn;           // bf16 outputs (FINE, SPARSE1)
     bf16* dv; int64_t sdvb, sdvh, sdvn;
-    float* part_k; float* part_v;                 // fp32 partial outputs (DENSE): (chunks, BH, n_units*16, 64)
+    f32x4* part;                                  // fp32 partials: slots (FINE, SPARSE1) or chunks (DENSE)
     int H, N, n_units, chunk_len;
     int64_t flat_stride;                          // entries of `flat` per (b,h)
+    int64_t work_stride;                          // ints of `work` per (b,h)
+    int64_t slot_stride;                          // partial slots per (b,h)
     float w;
 };
 
@@ -260,18 +263,50 @@ __device__ __forceinline__ void kside_pair(f32x4 dk[4], f32x4 dv[4], const bf16x
     }
 }
 
+// A partial sum of one unit (16 key rows x 64 channels, dK and dV) is kept in the MFMA
+// accumulator layout: 8 f32x4 registers per lane (4 channel tiles of dK, then 4 of dV).
+__device__ __forceinline__ f32x4* part_slot(f32x4* part, int64_t slot) { return part + slot * (8 * kWave); }
+
 template <int MODE>
 __global__ __launch_bounds__(256) void attn_kside_kernel(KSideParams p) {
-    constexpr int W = (MODE == MODE_FINE) ? 1 : 4;            // waves per unit
+    constexpr int W = (MODE == MODE_FINE) ? 1 : 4;            // waves per work item
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int N1 = p.N / kBlk;
     const int bh = blockIdx.y, b = bh / p.H, h = bh % p.H;
     const int r = lane & 15, quad = lane >> 4;
-    const int unit = (MODE == MODE_FINE) ? blockIdx.x * 4 + wave : blockIdx.x;
     const int sub = (MODE == MODE_FINE) ? 0 : wave;
-    const int chunk = (MODE == MODE_DENSE) ? blockIdx.z : 0;
-    const bool active = unit < p.n_units;
+
+    // which 16 key rows, which part of their query-block list, and where the result goes
+    int unit, start, cnt;
+    int64_t slot = -1;                                        // >= 0: write an fp32 partial
+    const int* fl = nullptr;
+    if (MODE == MODE_DENSE) {
+        unit = blockIdx.x;
+        start = blockIdx.z * p.chunk_len;
+        cnt = min(p.chunk_len, N1 - start);
+        slot = ((int64_t)blockIdx.z * gridDim.y + bh) * p.n_units + unit;
+    } else {
+        const int* work = p.work + (int64_t)bh * p.work_stride;
+        const int item = (MODE == MODE_FINE) ? blockIdx.x * 4 + wave : blockIdx.x;
+        if (item >= work[0]) return;                          // uniform over the item's waves
+        const int it = work[2 + p.n_units + item];
+        const int ci = it & 0xffff;
+        unit = it >> 16;
+        const int chunk = (MODE == MODE_FINE) ? LLSA_CHUNK_FINE : LLSA_CHUNK_COARSE;
+        const int* o = p.off + (int64_t)bh * (p.n_units + 1) + unit;
+        start = o[0] + ci * chunk;
+        cnt = min(chunk, o[1] - start);
+        if (MODE == MODE_SPARSE1) cnt *= kBlk;                // every parent stands for its 16 children
+        const int sb = work[2 + unit];
+        if (sb >= 0) slot = (int64_t)bh * p.slot_stride + sb + ci;
+        fl = p.flat + (int64_t)bh * p.flat_stride;
+    }
+    auto entry = [&](int i) -> int {                          // i-th query block of this item
+        if (MODE == MODE_FINE) return clampi(fl[start + i], 0, N1 - 1);
+        if (MODE == MODE_SPARSE1) return clampi(fl[start + i / kBlk], 0, N1 / kBlk - 1) * kBlk + (i % kBlk);
+        return start + i;
+    };
 
     f32x4 dk[4], dv[4];
 #pragma unroll
@@ -279,35 +314,14 @@ __global__ __launch_bounds__(256) void attn_kside_kernel(KSideParams p) {
         dk[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
         dv[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
-    if (active) {
+    {
         bf16x8 bk[2], bv[2];
-        {
-            const bf16* kp = p.kk + b * p.skb + h * p.skh + (int64_t)(unit * kBlk + r) * p.skn + quad * 8;
-            const bf16* vp = p.vv + b * p.svb + h * p.svh + (int64_t)(unit * kBlk + r) * p.svn + quad * 8;
-            bk[0] = ld16(kp);
-            bk[1] = ld16(kp + 32);
-            bv[0] = ld16(vp);
-            bv[1] = ld16(vp + 32);
-        }
-        int start = 0, cnt = 0;
-        if (MODE == MODE_FINE) {
-            const int* o = p.off + (int64_t)bh * (p.n_units + 1) + unit;
-            start = o[0];
-            cnt = o[1] - o[0];
-        } else if (MODE == MODE_SPARSE1) {
-            const int* o = p.off + (int64_t)bh * (p.n_units + 1) + unit;
-            start = o[0];
-            cnt = (o[1] - o[0]) * kBlk;
-        } else {
-            start = chunk * p.chunk_len;
-            cnt = min(p.chunk_len, N1 - start);
-        }
-        const int* fl = (MODE == MODE_DENSE) ? nullptr : p.flat + (int64_t)bh * p.flat_stride;
-        auto entry = [&](int i) -> int {          // i-th query block of this unit's list
-            if (MODE == MODE_FINE) return clampi(fl[start + i], 0, N1 - 1);
-            if (MODE == MODE_SPARSE1) return clampi(fl[start + i / kBlk], 0, N1 / kBlk - 1) * kBlk + (i % kBlk);
-            return start + i;
-        };
+        const bf16* kp = p.kk + b * p.skb + h * p.skh + (int64_t)(unit * kBlk + r) * p.skn + quad * 8;
+        const bf16* vp = p.vv + b * p.svb + h * p.svh + (int64_t)(unit * kBlk + r) * p.svn + quad * 8;
+        bk[0] = ld16(kp);
+        bk[1] = ld16(kp + 32);
+        bv[0] = ld16(vp);
+        bv[1] = ld16(vp + 32);
         const bf16* qb = p.q + b * p.sqb + h * p.sqh;
         const bf16* gb = p.dout + b * p.sdob + h * p.sdoh;
         const bf16* qtb = p.qt + (int64_t)bh * N1 * (kD * kBlk);
@@ -322,7 +336,15 @@ __global__ __launch_bounds__(256) void attn_kside_kernel(KSideParams p) {
     }
 
     if (MODE == MODE_FINE) {
-        if (!active) return;
+        if (slot >= 0) {
+            f32x4* ps = part_slot(p.part, slot);
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) {
+                ps[dt * kWave + lane] = dk[dt];
+                ps[(4 + dt) * kWave + lane] = dv[dt];
+            }
+            return;
+        }
         bf16* kp = p.dk + b * p.sdkb + h * p.sdkh + (int64_t)(unit * kBlk + r) * p.sdkn + quad * 4;
         bf16* vp = p.dv + b * p.sdvb + h * p.sdvh + (int64_t)(unit * kBlk + r) * p.sdvn + quad * 4;
 #pragma unroll
@@ -332,7 +354,7 @@ __global__ __launch_bounds__(256) void attn_kside_kernel(KSideParams p) {
         }
         return;
     }
-    // four waves per unit: reduce through LDS, wave w finishes channel tile w
+    // four waves per item: reduce through LDS, wave w finishes channel tile w
     __shared__ f32x4 red[4][8][kWave];
 #pragma unroll
     for (int dt = 0; dt < 4; dt++) {
@@ -347,31 +369,58 @@ __global__ __launch_bounds__(256) void attn_kside_kernel(KSideParams p) {
         sk += red[w][dt][lane];
         sv += red[w][4 + dt][lane];
     }
-    if (MODE == MODE_SPARSE1) {
+    if (slot >= 0) {
+        f32x4* ps = part_slot(p.part, slot);
+        ps[dt * kWave + lane] = sk;
+        ps[(4 + dt) * kWave + lane] = sv;
+    } else {
         bf16* kp = p.dk + b * p.sdkb + h * p.sdkh + (int64_t)(unit * kBlk + r) * p.sdkn + quad * 4 + dt * 16;
         bf16* vp = p.dv + b * p.sdvb + h * p.sdvh + (int64_t)(unit * kBlk + r) * p.sdvn + quad * 4 + dt * 16;
         st8(kp, cvt4(sk * kScale));
         st8(vp, cvt4(sv));
-    } else {
-        const int64_t row = ((int64_t)chunk * gridDim.y + bh) * ((int64_t)p.n_units * kBlk) + unit * kBlk + r;
-        *reinterpret_cast<f32x4*>(p.part_k + row * kD + dt * 16 + quad * 4) = sk;
-        *reinterpret_cast<f32x4*>(p.part_v + row * kD + dt * 16 + quad * 4) = sv;
     }
 }
 
-// sums the per-chunk fp32 partials of the dense pass in chunk order and rounds to bf16
-__global__ __launch_bounds__(256) void dense_reduce_kernel(const float* __restrict__ part_k, const float* __restrict__ part_v,
-                                                           bf16* __restrict__ dpk, bf16* __restrict__ dpv, int64_t n_elem4,
-                                                           int chunks) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= n_elem4) return;
-    f32x4 sk = {0.f, 0.f, 0.f, 0.f}, sv = {0.f, 0.f, 0.f, 0.f};
-    for (int c = 0; c < chunks; c++) {
-        sk += reinterpret_cast<const f32x4*>(part_k)[c * n_elem4 + i];
-        sv += reinterpret_cast<const f32x4*>(part_v)[c * n_elem4 + i];
+// Finishes the units the K-side kernel did not write itself: a unit whose list was cut into
+// several chunks is the sum of its partial slots (added in chunk order, so the result does not
+// depend on scheduling); a unit nobody selected gets zeros.  One wave per unit.
+// DENSE mode: every unit has `n_chunks` partials at stride `chunk_stride` slots.
+__global__ __launch_bounds__(64) void kside_reduce_kernel(const f32x4* __restrict__ part, const int* __restrict__ off,
+                                                          const int* __restrict__ work, bf16* dk, int64_t sdkb, int64_t sdkh,
+                                                          int64_t sdkn, bf16* dv, int64_t sdvb, int64_t sdvh, int64_t sdvn,
+                                                          int H, int n_units, int chunk, int64_t work_stride,
+                                                          int64_t slot_stride, int n_chunks, int64_t chunk_stride) {
+    const int lane = threadIdx.x, unit = blockIdx.x, bh = blockIdx.y, b = bh / H, h = bh % H;
+    const int r = lane & 15, quad = lane >> 4;
+    int64_t first, stride;
+    int n;
+    if (work != nullptr) {
+        const int* o = off + (int64_t)bh * (n_units + 1) + unit;
+        const int len = o[1] - o[0];
+        n = (len + chunk - 1) / chunk;
+        if (n == 1) return;                                   // written by the K-side kernel
+        first = (int64_t)bh * slot_stride + work[(int64_t)bh * work_stride + 2 + unit];
+        stride = 1;
+    } else {
+        n = n_chunks;
+        first = (int64_t)bh * n_units + unit;
+        stride = chunk_stride;
     }
-    st8(dpk + i * 4, cvt4(sk * kScale));
-    st8(dpv + i * 4, cvt4(sv));
+    f32x4 acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int c = 0; c < n; c++) {
+        const f32x4* ps = part + (first + c * stride) * (8 * kWave);
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[i] += ps[i * kWave + lane];
+    }
+    bf16* kp = dk + b * sdkb + h * sdkh + (int64_t)(unit * kBlk + r) * sdkn + quad * 4;
+    bf16* vp = dv + b * sdvb + h * sdvh + (int64_t)(unit * kBlk + r) * sdvn + quad * 4;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++) {
+        st8(kp + dt * 16, cvt4(acc[dt] * kScale));
+        st8(vp + dt * 16, cvt4(acc[4 + dt]));
+    }
 }
 
 struct DensePlan {
@@ -396,19 +445,38 @@ static DensePlan dense_plan(int B, int H, int N, int levels) {
 }
 
 static int64_t align256(int64_t x) { return (x + 255) & ~(int64_t)255; }
+constexpr int64_t kSlotBytes = 8 * kWave * sizeof(f32x4);     // one partial: 16 rows x 64 ch x (dK, dV) fp32
+
+struct BwdWorkspace {
+    int64_t delta, dot, part_fine, part_coarse, part_dense, total;
+    int64_t slots_fine, slots_coarse;                           // per (b,h)
+};
+
+static BwdWorkspace bwd_workspace(int B, int H, int N, int T, int T2, int levels) {
+    const int64_t BH = (int64_t)B * H, N1 = N / 16, N2 = N1 / 16;
+    const DensePlan d = dense_plan(B, H, N, levels);
+    BwdWorkspace w;
+    // a key block has several chunks only if it has more than `chunk` entries, so at most
+    // E/chunk such blocks with at most E/chunk + E/chunk chunks in total
+    w.slots_fine = 2 * (N1 * T / LLSA_CHUNK_FINE) + 2;
+    w.slots_coarse = (levels == 2) ? 2 * (N2 * T2 / LLSA_CHUNK_COARSE) + 2 : 0;
+    int64_t o = 0;
+    w.delta = o;        o += align256(BH * N * 4);
+    w.dot = o;          o += align256(BH * N * 64 * 2);
+    w.part_fine = o;    o += align256(BH * w.slots_fine * kSlotBytes);
+    w.part_coarse = o;  o += align256(BH * w.slots_coarse * kSlotBytes);
+    w.part_dense = o;   o += align256((int64_t)d.chunks * BH * (d.n_tok / 16) * kSlotBytes);
+    w.total = o;
+    return w;
+}
 
 }  // namespace llsa
 
 using namespace llsa;
 
-extern "C" int64_t llsa_attn_bwd_workspace_bytes(int B, int H, int N, int levels) {
-    if (B <= 0 || H <= 0 || N <= 0 || N % 16 != 0 || (levels != 1 && levels != 2)) return -1;
-    const DensePlan d = dense_plan(B, H, N, levels);
-    const int64_t BH = (int64_t)B * H;
-    int64_t bytes = align256(BH * N * 4);                       // delta
-    bytes += align256(BH * N * 64 * 2);                         // block-transposed dO
-    bytes += 2 * align256((int64_t)d.chunks * BH * d.n_tok * 64 * 4);   // dense partials (k, v)
-    return bytes;
+extern "C" int64_t llsa_attn_bwd_workspace_bytes(int B, int H, int N, int T, int T2, int levels) {
+    if (B <= 0 || H <= 0 || N <= 0 || N % 16 != 0 || T <= 0 || (levels != 1 && levels != 2)) return -1;
+    return bwd_workspace(B, H, N, T, T2, levels).total;
 }
 
 extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
@@ -436,20 +504,17 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     for (int64_t s : st) LLSA_REQUIRE(stride_ok(s), "attn_bwd: input row strides must keep rows 16-byte aligned");
     const int64_t so[] = {a->sdqb, a->sdqh, a->sdqn, a->sdkb, a->sdkh, a->sdkn, a->sdvb, a->sdvh, a->sdvn};
     for (int64_t s : so) LLSA_REQUIRE(s % 4 == 0, "attn_bwd: output row strides must keep rows 8-byte aligned");
-    const int64_t need = llsa_attn_bwd_workspace_bytes(a->B, a->H, a->N, a->levels);
-    LLSA_REQUIRE(a->workspace_bytes >= need, "attn_bwd: workspace too small (%lld < %lld)", (long long)a->workspace_bytes, (long long)need);
+    const BwdWorkspace wsp = bwd_workspace(a->B, a->H, a->N, a->T, a->T2, a->levels);
+    LLSA_REQUIRE(a->workspace_bytes >= wsp.total, "attn_bwd: workspace too small (%lld < %lld)", (long long)a->workspace_bytes,
+                 (long long)wsp.total);
+    LLSA_REQUIRE(a->work != nullptr && (a->levels == 1 || a->pwork != nullptr), "attn_bwd: work lists missing");
 
     hipStream_t s = (hipStream_t)stream;
     const int B = a->B, H = a->H, N = a->N, N1 = N / 16, N2 = N1 / 16, BH = B * H;
     const DensePlan d = dense_plan(B, H, N, a->levels);
     char* ws = (char*)a->workspace;
-    float* delta = (float*)ws;
-    ws += align256((int64_t)BH * N * 4);
-    bf16* dot = (bf16*)ws;
-    ws += align256((int64_t)BH * N * 64 * 2);
-    float* part_k = (float*)ws;
-    ws += align256((int64_t)d.chunks * BH * d.n_tok * 64 * 4);
-    float* part_v = (float*)ws;
+    float* delta = (float*)(ws + wsp.delta);
+    bf16* dot = (bf16*)(ws + wsp.dot);
 
     const int stages = a->stages ? a->stages : 0x7fffffff;
     if (stages & LLSA_BWD_PRE) hipLaunchKernelGGL(bwd_pre_kernel, dim3((N1 + 15) / 16, BH), dim3(128), 0, s, *a, delta, dot);
@@ -459,17 +524,24 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     p.q = (const bf16*)a->q; p.sqb = a->sqb; p.sqh = a->sqh; p.sqn = a->sqn;
     p.dout = (const bf16*)a->dout; p.sdob = a->sdob; p.sdoh = a->sdoh; p.sdon = a->sdon;
     p.qt = (const bf16*)a->qt; p.dot = dot; p.lse = a->lse; p.delta = delta;
-    p.H = H; p.N = N; p.part_k = nullptr; p.part_v = nullptr; p.chunk_len = 0;
+    p.H = H; p.N = N; p.chunk_len = 0;
 
     // fine K/V blocks
     p.kk = (const bf16*)a->k; p.skb = a->skb; p.skh = a->skh; p.skn = a->skn;
     p.vv = (const bf16*)a->v; p.svb = a->svb; p.svh = a->svh; p.svn = a->svn;
     p.off = a->off; p.flat = a->flat; p.flat_stride = (int64_t)N1 * a->T;
+    p.work = a->work; p.work_stride = llsa_work_list_len(N1, N1, a->T, LLSA_CHUNK_FINE);
+    p.part = (f32x4*)(ws + wsp.part_fine); p.slot_stride = wsp.slots_fine;
     p.dk = (bf16*)a->dk; p.sdkb = a->sdkb; p.sdkh = a->sdkh; p.sdkn = a->sdkn;
     p.dv = (bf16*)a->dv; p.sdvb = a->sdvb; p.sdvh = a->sdvh; p.sdvn = a->sdvn;
     p.n_units = N1; p.w = 1.f;
-    if (stages & LLSA_BWD_DKV)
-        hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_FINE>), dim3((N1 + 3) / 4, BH), dim3(256), 0, s, p);
+    if (stages & LLSA_BWD_DKV) {
+        const int max_items = N1 * a->T / LLSA_CHUNK_FINE + N1;
+        hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_FINE>), dim3((max_items + 3) / 4, BH), dim3(256), 0, s, p);
+        hipLaunchKernelGGL(kside_reduce_kernel, dim3(N1, BH), dim3(64), 0, s, (const f32x4*)p.part, p.off, p.work, p.dk, p.sdkb,
+                           p.sdkh, p.sdkn, p.dv, p.sdvb, p.sdvh, p.sdvn, H, N1, LLSA_CHUNK_FINE, p.work_stride, p.slot_stride,
+                           0, (int64_t)0);
+    }
 
     const int64_t s1b = (int64_t)H * N1 * 64, s1h = (int64_t)N1 * 64;
     const int64_t s2b = (int64_t)H * N2 * 64, s2h = (int64_t)N2 * 64;
@@ -478,30 +550,40 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
         p.kk = (const bf16*)a->pk; p.skb = s1b; p.skh = s1h; p.skn = 64;
         p.vv = (const bf16*)a->pv; p.svb = s1b; p.svh = s1h; p.svn = 64;
         p.off = a->poff; p.flat = a->pflat; p.flat_stride = (int64_t)N2 * a->T2;
+        p.work = a->pwork; p.work_stride = llsa_work_list_len(N2, N2, a->T2, LLSA_CHUNK_COARSE);
+        p.part = (f32x4*)(ws + wsp.part_coarse); p.slot_stride = wsp.slots_coarse;
         p.dk = (bf16*)a->dpk; p.sdkb = s1b; p.sdkh = s1h; p.sdkn = 64;
         p.dv = (bf16*)a->dpv; p.sdvb = s1b; p.sdvh = s1h; p.sdvn = 64;
         p.n_units = N2; p.w = a->cgw1;
-        hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_SPARSE1>), dim3(N2, BH), dim3(256), 0, s, p);
+        const int max_items = N2 * a->T2 / LLSA_CHUNK_COARSE + N2;
+        hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_SPARSE1>), dim3(max_items, BH), dim3(256), 0, s, p);
+        hipLaunchKernelGGL(kside_reduce_kernel, dim3(N2, BH), dim3(64), 0, s, (const f32x4*)p.part, p.off, p.work, p.dk, p.sdkb,
+                           p.sdkh, p.sdkn, p.dv, p.sdvb, p.sdvh, p.sdvn, H, N2, LLSA_CHUNK_COARSE, p.work_stride,
+                           p.slot_stride, 0, (int64_t)0);
     }
-    // dense coarsest level
+    // dense coarsest level: every unit (16 pooled tokens) meets every query block; the query
+    // range is cut into d.chunks pieces whose partial sums are added afterwards
     if (!(stages & LLSA_BWD_DENSE)) return launch_status("attn_bwd");
     if (a->levels == 2) {
         p.kk = (const bf16*)a->pk2; p.skb = s2b; p.skh = s2h; p.skn = 64;
         p.vv = (const bf16*)a->pv2; p.svb = s2b; p.svh = s2h; p.svn = 64;
+        p.dk = (bf16*)a->dpk2; p.dv = (bf16*)a->dpv2;
+        p.sdkb = p.sdvb = s2b; p.sdkh = p.sdvh = s2h;
         p.w = a->w2;
     } else {
         p.kk = (const bf16*)a->pk; p.skb = s1b; p.skh = s1h; p.skn = 64;
         p.vv = (const bf16*)a->pv; p.svb = s1b; p.svh = s1h; p.svn = 64;
+        p.dk = (bf16*)a->dpk; p.dv = (bf16*)a->dpv;
+        p.sdkb = p.sdvb = s1b; p.sdkh = p.sdvh = s1h;
         p.w = a->cgw1;
     }
-    p.off = nullptr; p.flat = nullptr; p.flat_stride = 0; p.dk = nullptr; p.dv = nullptr;
-    p.part_k = part_k; p.part_v = part_v;
+    p.sdkn = p.sdvn = 64;
+    p.off = nullptr; p.flat = nullptr; p.flat_stride = 0; p.work = nullptr; p.work_stride = 0; p.slot_stride = 0;
+    p.part = (f32x4*)(ws + wsp.part_dense);
     p.n_units = d.n_tok / 16; p.chunk_len = d.chunk_len;
     hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_DENSE>), dim3(p.n_units, BH, d.chunks), dim3(256), 0, s, p);
-    const int64_t n4 = (int64_t)BH * d.n_tok * 64 / 4;
-    bf16* odk = (bf16*)(a->levels == 2 ? a->dpk2 : a->dpk);
-    bf16* odv = (bf16*)(a->levels == 2 ? a->dpv2 : a->dpv);
-    hipLaunchKernelGGL(dense_reduce_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, s, (const float*)part_k,
-                       (const float*)part_v, odk, odv, n4, d.chunks);
+    hipLaunchKernelGGL(kside_reduce_kernel, dim3(p.n_units, BH), dim3(64), 0, s, (const f32x4*)p.part, (const int*)nullptr,
+                       (const int*)nullptr, p.dk, p.sdkb, p.sdkh, p.sdkn, p.dv, p.sdvb, p.sdvh, p.sdvn, H, p.n_units, 1,
+                       (int64_t)0, (int64_t)0, d.chunks, (int64_t)BH * p.n_units);
     return launch_status("attn_bwd");
 }

@@ -22,12 +22,18 @@ __device__ __forceinline__ int wave_incl_scan(int v, int lane) {
     return v;
 }
 
+// Work list (optional): the K-side kernels walk each key block's segment in chunks of at most
+// `chunk` entries so that a popular key block does not serialise on one wave.  Per (b,h):
+//   work[0] = number of items, work[1] = number of partial-sum slots,
+//   work[2 + n] = first slot of key block n, or -1 when n has at most one chunk,
+//   work[2 + Kb + i] = item i = (n << 16) | chunk index   (items of one key block are adjacent)
 __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int* __restrict__ idx, int* __restrict__ offsets,
-                                                                      int* __restrict__ flat, int Mb, int Kb, int T) {
+                                                                      int* __restrict__ flat, int* __restrict__ work,
+                                                                      int Mb, int Kb, int T, int chunk, int work_stride) {
     HIP_DYNAMIC_SHARED(int, smem)
     const int words = (Mb + 31) / 32;
     int* pos = smem;                               // Kb
-    int* wave_tot = smem + Kb;                     // kTrWaves (+ padding to 64)
+    int* wave_tot = smem + Kb;                     // 3 * kTrWaves (+ padding to 64)
     unsigned* bitmaps = (unsigned*)(smem + Kb + 64);   // kTrWaves * words
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -45,20 +51,48 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
     // exclusive scan over pos[0..Kb): each thread owns `per` consecutive counters
     const int per = (Kb + kTrThreads - 1) / kTrThreads;
     const int c0 = min(tid * per, Kb), c1 = min(c0 + per, Kb);
-    int local = 0;
-    for (int i = c0; i < c1; i++) local += pos[i];
+    int local = 0, l_items = 0, l_slots = 0;
+    for (int i = c0; i < c1; i++) {
+        const int c = pos[i];
+        const int nch = (c + chunk - 1) / chunk;
+        local += c;
+        l_items += nch;
+        l_slots += (nch > 1) ? nch : 0;
+    }
     const int incl = wave_incl_scan(local, lane);
-    if (lane == kWave - 1) wave_tot[wave] = incl;
+    const int incl_i = wave_incl_scan(l_items, lane);
+    const int incl_s = wave_incl_scan(l_slots, lane);
+    if (lane == kWave - 1) {
+        wave_tot[wave] = incl;
+        wave_tot[kTrWaves + wave] = incl_i;
+        wave_tot[2 * kTrWaves + wave] = incl_s;
+    }
     __syncthreads();
-    int run = incl - local;
-    for (int w = 0; w < wave; w++) run += wave_tot[w];
+    int run = incl - local, run_i = incl_i - l_items, run_s = incl_s - l_slots;
+    for (int w = 0; w < wave; w++) {
+        run += wave_tot[w];
+        run_i += wave_tot[kTrWaves + w];
+        run_s += wave_tot[2 * kTrWaves + w];
+    }
+    if (work != nullptr) work += (int64_t)bh * work_stride;
     for (int i = c0; i < c1; i++) {
         const int c = pos[i];
         offsets[i] = run;
         pos[i] = run;
         run += c;
+        if (work != nullptr) {
+            const int nch = (c + chunk - 1) / chunk;
+            work[2 + i] = (nch > 1) ? run_s : -1;
+            for (int ci = 0; ci < nch; ci++) work[2 + Kb + run_i + ci] = (i << 16) | ci;
+            run_i += nch;
+            run_s += (nch > 1) ? nch : 0;
+        }
     }
     if (tid == 0) offsets[Kb] = E;
+    if (work != nullptr && tid == kTrThreads - 1) {
+        work[0] = run_i;
+        work[1] = run_s;
+    }
     __syncthreads();
 
     for (int e = tid; e < E; e += kTrThreads) {
@@ -102,17 +136,27 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
 
 using namespace llsa;
 
-extern "C" int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, int B, int H, int Mb, int Kb,
-                                      int T, void* stream) {
+extern "C" int64_t llsa_work_list_len(int Mb, int Kb, int T, int chunk) {
+    if (Mb <= 0 || Kb <= 0 || T <= 0 || chunk <= 0) return -1;
+    return 2 + (int64_t)Kb + ((int64_t)Mb * T / chunk + Kb);
+}
+
+extern "C" int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, int32_t* work, int B, int H, int Mb,
+                                      int Kb, int T, int chunk, void* stream) {
     LLSA_REQUIRE(idx && offsets && flat, "transpose_indices: null argument");
     LLSA_REQUIRE(B > 0 && H > 0 && Mb > 0 && Kb > 0 && T > 0, "transpose_indices: bad shape");
+    LLSA_REQUIRE(work == nullptr || (chunk >= 1 && Kb < 32768 && (int64_t)Mb * T / chunk + 1 < 65536),
+                 "transpose_indices: work list needs chunk >= 1, Kb < 32768 and fewer than 65536 chunks per key block");
+    if (chunk < 1) chunk = 1;
     const int words = (Mb + 31) / 32;
     const size_t lds = sizeof(int) * ((size_t)Kb + 64 + (size_t)kTrWaves * words);
+    static_assert(3 * kTrWaves <= 64, "wave totals must fit their LDS slot");
     LLSA_REQUIRE(lds <= 160 * 1024, "transpose_indices: Kb=%d, Mb=%d need %zu bytes of LDS (limit 163840)", Kb, Mb, lds);
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void*)transpose_indices_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return fail(-101, "transpose_indices: cannot raise dynamic LDS to %zu bytes: %s", lds, hipGetErrorString(e));
     }
-    hipLaunchKernelGGL(transpose_indices_kernel, dim3(B * H), dim3(kTrThreads), lds, (hipStream_t)stream, idx, offsets, flat, Mb, Kb, T);
+    hipLaunchKernelGGL(transpose_indices_kernel, dim3(B * H), dim3(kTrThreads), lds, (hipStream_t)stream, idx, offsets, flat, work, Mb, Kb, T, chunk,
+                       (int)llsa_work_list_len(Mb, Kb, T, chunk));
     return launch_status("transpose_indices");
 }

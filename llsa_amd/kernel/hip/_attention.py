@@ -6,7 +6,7 @@ from typing import Optional
 
 import torch
 
-from ..._lib import AttnBwdArgs, AttnFwdArgs
+from ..._lib import CHUNK_COARSE, CHUNK_FINE, AttnBwdArgs, AttnFwdArgs
 from ._common import BLOCK, as_rows, lib_for, ptr, require_bf16, require_head_dim, s3, stream_of
 from .indices_transpose import transpose_indices
 from .mean_pool import block_transpose
@@ -97,17 +97,17 @@ def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_wei
     idx = indices.to(torch.int32).contiguous()
     if levels == 2:
         pidx = p_indices.to(torch.int32).contiguous()
-    if csr is not None:                       # (off, flat[, poff, pflat]) from transpose_indices
-        off, flat = csr[0], csr[1]
+    if csr is not None:                       # (off, flat, work[, poff, pflat, pwork]) from transpose_indices
+        off, flat, work = csr[:3]
         if levels == 2:
-            poff, pflat = csr[2], csr[3]
+            poff, pflat, pwork = csr[3:6]
     else:
-        off, flat = transpose_indices(idx, N // BLOCK)
+        off, flat, work = transpose_indices(idx, N // BLOCK, CHUNK_FINE)
         if levels == 2:
-            poff, pflat = transpose_indices(pidx, N // (BLOCK * BLOCK))
+            poff, pflat, pwork = transpose_indices(pidx, N // (BLOCK * BLOCK), CHUNK_COARSE)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dpk, dpv = torch.empty_like(pk), torch.empty_like(pv)
-    ws_bytes = lib.attn_bwd_workspace_bytes(B, H, N, levels)
+    ws_bytes = lib.attn_bwd_workspace_bytes(B, H, N, T, T2, levels)
     ws = torch.empty(ws_bytes, device=q.device, dtype=torch.uint8)
     a = AttnBwdArgs()
     a.dout, (a.sdob, a.sdoh, a.sdon) = do.data_ptr(), s3(do)
@@ -118,7 +118,7 @@ def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_wei
     lse = lse.contiguous()
     a.lse, a.pk, a.pv = lse.data_ptr(), pk.data_ptr(), pv.data_ptr()
     a.qt, a.kt, a.pkt = qt.data_ptr(), kt.data_ptr(), pkt.data_ptr()
-    a.idx, a.off, a.flat = idx.data_ptr(), off.data_ptr(), flat.data_ptr()
+    a.idx, a.off, a.flat, a.work = idx.data_ptr(), off.data_ptr(), flat.data_ptr(), work.data_ptr()
     a.dq, (a.sdqb, a.sdqh, a.sdqn) = dq.data_ptr(), s3(dq)
     a.dk, (a.sdkb, a.sdkh, a.sdkn) = dk.data_ptr(), s3(dk)
     a.dv, (a.sdvb, a.sdvh, a.sdvn) = dv.data_ptr(), s3(dv)
@@ -127,7 +127,7 @@ def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_wei
     if levels == 2:
         dpk2, dpv2 = torch.empty_like(pk2), torch.empty_like(pv2)
         a.pk2, a.pv2, a.pk2t = pk2.data_ptr(), pv2.data_ptr(), pk2t.data_ptr()
-        a.pidx, a.poff, a.pflat = pidx.data_ptr(), poff.data_ptr(), pflat.data_ptr()
+        a.pidx, a.poff, a.pflat, a.pwork = pidx.data_ptr(), poff.data_ptr(), pflat.data_ptr(), pwork.data_ptr()
         a.dpk2, a.dpv2 = dpk2.data_ptr(), dpv2.data_ptr()
         outs += [dpk2, dpv2]
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws_bytes

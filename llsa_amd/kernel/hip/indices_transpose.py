@@ -6,9 +6,11 @@ import torch
 from ._common import lib_for, ptr, stream_of
 
 
-def transpose_indices(q_topk_indices, k_ntx=None):
+def transpose_indices(q_topk_indices, k_ntx=None, chunk=0):
     """indices_transpose.py:104-109.  Returns (offsets (B,H,1+Kb), flat (B,H,Mb*T)), int32; the
-    entries of each segment are in ascending query-block order."""
+    entries of each segment are in ascending query-block order.  With chunk > 0 a third tensor
+    is returned: the work list the backward kernels use to walk every segment in pieces of at
+    most `chunk` entries (layout in include/llsa_hip.h)."""
     lib = lib_for(q_topk_indices)
     B, H, Mb, T = q_topk_indices.shape
     if k_ntx is None:
@@ -16,6 +18,9 @@ def transpose_indices(q_topk_indices, k_ntx=None):
     idx = q_topk_indices.to(torch.int32).contiguous()
     offsets = torch.empty(B, H, 1 + k_ntx, device=idx.device, dtype=torch.int32)
     flat = torch.empty(B, H, Mb * T, device=idx.device, dtype=torch.int32)
-    lib.check(lib.transpose_indices(ptr(idx), ptr(offsets), ptr(flat), B, H, Mb, k_ntx, T, stream_of(lib, idx)),
-              "transpose_indices")
-    return offsets, flat
+    work = None
+    if chunk > 0:
+        work = torch.empty(B, H, lib.work_list_len(Mb, k_ntx, T, chunk), device=idx.device, dtype=torch.int32)
+    lib.check(lib.transpose_indices(ptr(idx), ptr(offsets), ptr(flat), ptr(work), B, H, Mb, k_ntx, T, max(chunk, 1),
+                                    stream_of(lib, idx)), "transpose_indices")
+    return (offsets, flat) if work is None else (offsets, flat, work)

@@ -200,13 +200,25 @@ def _selection_l1(q, k, T):
     return O.topk_lowest_index(O.dense_scores(pq, pk), T)
 
 
-def check_attn_l1(dev, B=1, H=2, N=1024, T=8, strided=False, smooth=False, weight=16.0):
-    """Forward and backward kernels with oracle-chosen indices."""
+def _hot_indices(B, H, Mb, Kb, T, hot, seed):
+    """Every row selects block `hot` first; the rest are distinct random blocks."""
+    g = torch.Generator().manual_seed(seed)
+    rows = []
+    for _ in range(B * H * Mb):
+        rest = torch.randperm(Kb - 1, generator=g)[:T - 1]
+        rest = rest + (rest >= hot).long()
+        rows.append(torch.cat([torch.tensor([hot]), rest]))
+    return torch.stack(rows).reshape(B, H, Mb, T)
+
+
+def check_attn_l1(dev, B=1, H=2, N=1024, T=8, strided=False, smooth=False, weight=16.0, hot=None):
+    """Forward and backward kernels with oracle-chosen indices (or, with `hot`, indices in which
+    one key block is selected by every query block, so that its list is cut into chunks)."""
     from llsa_amd.kernel.hip._attention import attn_bwd, attn_fwd
     q, k, v, do = smooth_inputs(B, H, N, 64, dev) if smooth else randn_inputs(B, H, N, 64, dev, seed=14, strided=strided)
     qc, kc, vc, doc = (t.cpu() for t in (q, k, v, do))
     pk, pv = O.mean_pool(kc), O.mean_pool(vc)
-    idx = _selection_l1(qc, kc, T)
+    idx = _selection_l1(qc, kc, T) if hot is None else _hot_indices(B, H, N // 16, N // 16, T, hot, 21)
     o, lse = attn_fwd(q, k, v, pk.to(dev), pv.to(dev), idx.int().to(dev), weight)
     ro, rl = O.attn_fwd_l1(qc, kc, vc, pk, pv, idx, weight)
     assert o.stride() == q.stride(), "o must have q's strides"
@@ -218,13 +230,16 @@ def check_attn_l1(dev, B=1, H=2, N=1024, T=8, strided=False, smooth=False, weigh
         close(name, a, b)
 
 
-def check_attn_l2(dev, B=1, H=1, N=16384, T=8, T2=4, smooth=False):
+def check_attn_l2(dev, B=1, H=1, N=16384, T=8, T2=4, smooth=False, hot=None):
     from llsa_amd.kernel.hip._attention import attn_bwd, attn_fwd
     q, k, v, do = smooth_inputs(B, H, N, 64, dev) if smooth else randn_inputs(B, H, N, 64, dev, seed=15)
     qc, kc, vc, doc = (t.cpu() for t in (q, k, v, do))
     pq, pk, pv = O.mean_pool(qc), O.mean_pool(kc), O.mean_pool(vc)
     pq2, pk2, pv2 = O.mean_pool(pq), O.mean_pool(pk), O.mean_pool(pv)
-    pidx = O.topk_lowest_index(O.dense_scores(pq2, pk2), T2)
+    if hot is None:
+        pidx = O.topk_lowest_index(O.dense_scores(pq2, pk2), T2)
+    else:                     # every parent selects coarse block `hot`: its parent list is cut into chunks
+        pidx = _hot_indices(B, H, N // 256, N // 256, T2, hot, 22)
     idx = O.topk_sparse(pq, pk, pidx, T)
     d = lambda t: t.to(dev)
     o, lse = attn_fwd(q, k, v, d(pk), d(pv), d(idx), 16.0, pk2=d(pk2), pv2=d(pv2), p_indices=d(pidx.int()),

@@ -57,6 +57,10 @@ def test_attn_l1():
     P.check_attn_l1(DEV, B=1, H=2, N=1024, T=8, strided=True)
 
 
+def test_attn_l1_hot_block():
+    P.check_attn_l1(DEV, B=1, H=1, N=2048, T=4, hot=5)        # 128 query blocks on one key block: 4 chunks
+
+
 def test_attn_special_cases():
     P.check_attn_reduces_to_sdpa(DEV, B=1, H=1, N=1024)
     P.check_constant_v(DEV)
@@ -69,6 +73,10 @@ def test_op_l1(fused, rope):
 
 def test_attn_l2():
     P.check_attn_l2(DEV, B=1, H=1, N=16384, T=4, T2=4)
+
+
+def test_attn_l2_hot_coarse_block():
+    P.check_attn_l2(DEV, B=1, H=1, N=16384, T=4, T2=4, hot=3)  # 64 parents on one coarse block: 8 chunks
 
 
 def test_op_l2_fused_rope():

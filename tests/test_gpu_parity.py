@@ -79,6 +79,11 @@ def test_attn_l1_small(dev):
     P.check_attn_l1(dev, B=1, H=2, N=1024, T=8)
 
 
+def test_attn_hot_blocks(dev):
+    P.check_attn_l1(dev, B=1, H=2, N=4096, T=8, hot=5)
+    P.check_attn_l2(dev, B=1, H=1, N=16384, T=8, T2=8, hot=3)
+
+
 def test_attn_special_cases(dev):
     P.check_attn_reduces_to_sdpa(dev, B=1, H=2, N=1024)
     P.check_constant_v(dev)
