@@ -103,9 +103,10 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, cons
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int N1 = a.N / kBlk, N2 = N1 / kBlk;
-    const int g = blockIdx.x * 4 + wave;
+    const int lid = xcd_logical_id();
+    const int g = (lid % (int)gridDim.x) * 4 + wave;
     if (g >= N1) return;
-    const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+    const int bh = lid / (int)gridDim.x, b = bh / a.H, h = bh % a.H;
     const int r = lane & 15, quad = lane >> 4;
     const int tok = g * kBlk + r;
 
@@ -132,11 +133,13 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, cons
     const bf16* pkt = (const bf16*)a.pkt + (int64_t)bh * N2 * (kD * kBlk);
     const bf16 *kb[2], *vb[2], *ktb[2];
 
-    const int* ip = a.idx + ((int64_t)bh * N1 + g) * a.T;
+    __shared__ int ids_lds[4][2][kWave];
+    wave_sort_ids(a.idx + ((int64_t)bh * N1 + g) * a.T, a.T, ids_lds[wave][0], ids_lds[wave][1], lane);
+    const int* ip = ids_lds[wave][1];
     for (int t = 0; t < a.T / 2; t++) {
 #pragma unroll
         for (int j = 0; j < 2; j++) {
-            const int blk = clampi(ip[2 * t + j], 0, N1 - 1);
+            const int blk = clampi(__builtin_amdgcn_readfirstlane(ip[2 * t + j]), 0, N1 - 1);
             kb[j] = kbase + (int64_t)blk * kBlk * a.skn;
             vb[j] = vbase + (int64_t)blk * kBlk * a.svn;
             ktb[j] = kt + (int64_t)blk * (kD * kBlk);
@@ -273,7 +276,9 @@ __global__ __launch_bounds__(256) void attn_kside_kernel(KSideParams p) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int N1 = p.N / kBlk;
-    const int bh = blockIdx.y, b = bh / p.H, h = bh % p.H;
+    const int lid = xcd_logical_id();
+    const int bx = lid % (int)gridDim.x;
+    const int bh = lid / (int)gridDim.x, b = bh / p.H, h = bh % p.H;
     const int r = lane & 15, quad = lane >> 4;
     const int sub = (MODE == MODE_FINE) ? 0 : wave;
 
@@ -282,13 +287,13 @@ __global__ __launch_bounds__(256) void attn_kside_kernel(KSideParams p) {
     int64_t slot = -1;                                        // >= 0: write an fp32 partial
     const int* fl = nullptr;
     if (MODE == MODE_DENSE) {
-        unit = blockIdx.x;
+        unit = bx;
         start = blockIdx.z * p.chunk_len;
         cnt = min(p.chunk_len, N1 - start);
         slot = ((int64_t)blockIdx.z * gridDim.y + bh) * p.n_units + unit;
     } else {
         const int* work = p.work + (int64_t)bh * p.work_stride;
-        const int item = (MODE == MODE_FINE) ? blockIdx.x * 4 + wave : blockIdx.x;
+        const int item = (MODE == MODE_FINE) ? bx * 4 + wave : bx;
         if (item >= work[0]) return;                          // uniform over the item's waves
         const int it = work[2 + p.n_units + item];
         const int ci = it & 0xffff;

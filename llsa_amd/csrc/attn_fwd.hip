@@ -19,6 +19,10 @@
 #include "llsa_host.h"
 #include "../../include/llsa_hip.h"
 
+#ifndef LLSA_FWD_NB
+#define LLSA_FWD_NB 2          // 16-key blocks per pipeline step (2 or 4)
+#endif
+
 namespace llsa {
 
 struct SoftmaxState {
@@ -27,31 +31,59 @@ struct SoftmaxState {
     f32x4 acc[4];    // O^T: channel 16*dt + 4*(l/16) + e of query l%16
 };
 
-// One 64-key tile = four 16-key blocks.  kb[j] points at row 0 of block j (row stride ks
-// elements), vtb[j] at the block-transposed values of block j.
-__device__ __forceinline__ void fwd_tile(SoftmaxState& st, const bf16x8 bq[2], const bf16* const kb[4], int64_t ks,
-                                         const bf16* const vtb[4], float wratio, int lane) {
+// Operands of one step = NB 16-key blocks, as they sit in registers between load and use.
+template <int NB>
+struct KvRegs {
+    bf16x8 k[NB][2];     // K rows: block j, channel half
+    bf16x4 v[NB][4];     // block-transposed V: block j, channel tile dt, keys 4*(l/16)..+3
+};
+
+// Where one step's blocks live.  kb[j] points at row 0 of block j (row stride ks elements),
+// vtb[j] at the block-transposed values of block j.
+template <int NB>
+struct StepDesc {
+    const bf16* kb[NB];
+    const bf16* vtb[NB];
+    int64_t ks;
+    float wratio;        // weight(previous segment) / weight(this segment) on the first step of a segment
+};
+
+template <int NB>
+__device__ __forceinline__ void load_step(KvRegs<NB>& t, const StepDesc<NB>& d, int lane) {
     const int r = lane & 15, quad = lane >> 4;
-    f32x4 s[4];
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const bf16* p = kb[j] + r * ks + quad * 8;
+    for (int j = 0; j < NB; j++) {
+        const bf16* p = d.kb[j] + r * d.ks + quad * 8;
+        t.k[j][0] = ld16(p);
+        t.k[j][1] = ld16(p + 32);
+    }
+#pragma unroll
+    for (int j = 0; j < NB; j++)
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) t.v[j][dt] = ld8(d.vtb[j] + (dt * 16 + r) * kBlk + quad * 4);
+}
+
+template <int NB>
+__device__ __forceinline__ void compute_step(SoftmaxState& st, const bf16x8 bq[2], const KvRegs<NB>& t, float wratio) {
+    f32x4 s[NB];
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
         f32x4 z = {0.f, 0.f, 0.f, 0.f};
-        z = mfma_bf16(ld16(p), bq[0], z);
-        s[j] = mfma_bf16(ld16(p + 32), bq[1], z);
+        z = mfma_bf16(t.k[j][0], bq[0], z);
+        s[j] = mfma_bf16(t.k[j][1], bq[1], z);
     }
     float mx = s[0][0];
 #pragma unroll
-    for (int j = 0; j < 4; j++)
+    for (int j = 0; j < NB; j++)
 #pragma unroll
         for (int e = 0; e < 4; e++) mx = fmaxf(mx, s[j][e]);
     mx = quad_max(mx);
     const float m2n = fmaxf(st.m2, mx * kScaleLog2e);
     const float alpha = exp2_fast(st.m2 - m2n) * wratio;
     float rs = 0.f;
-    bf16x8 bp[2];
+    bf16x8 bp[NB / 2];
 #pragma unroll
-    for (int j = 0; j < 4; j++)
+    for (int j = 0; j < NB; j++)
 #pragma unroll
         for (int e = 0; e < 4; e++) {
             const float p = exp2_fast(fmaf(s[j][e], kScaleLog2e, -m2n));
@@ -60,24 +92,28 @@ __device__ __forceinline__ void fwd_tile(SoftmaxState& st, const bf16x8 bq[2], c
         }
     st.lsum = st.lsum * alpha + rs;
     st.m2 = m2n;
+    if (__ballot(alpha != 1.f) != 0) {        // the running max moved (or a new segment starts) somewhere in the wave
 #pragma unroll
-    for (int dt = 0; dt < 4; dt++) st.acc[dt] *= alpha;
+        for (int dt = 0; dt < 4; dt++) st.acc[dt] *= alpha;
+    }
 #pragma unroll
-    for (int c = 0; c < 2; c++)
+    for (int c = 0; c < NB / 2; c++)
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++) {
-            const int off = (dt * 16 + r) * kBlk + quad * 4;
-            st.acc[dt] = mfma_bf16(cat(ld8(vtb[2 * c] + off), ld8(vtb[2 * c + 1] + off)), bp[c], st.acc[dt]);
-        }
+        for (int dt = 0; dt < 4; dt++)
+            st.acc[dt] = mfma_bf16(cat(t.v[2 * c][dt], t.v[2 * c + 1][dt]), bp[c], st.acc[dt]);
 }
 
+// One wave per query block; the KV list is walked in steps of NB blocks with the loads of
+// step t+1 issued before the arithmetic of step t (two register buffers, ping-pong).
+template <int NB>
 __global__ __launch_bounds__(256) void attn_fwd_kernel(llsa_attn_fwd_args a) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int N1 = a.N / kBlk, N2 = N1 / kBlk;
-    const int g = blockIdx.x * 4 + wave;
+    const int lid = xcd_logical_id();
+    const int g = (lid % (int)gridDim.x) * 4 + wave;
     if (g >= N1) return;
-    const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
+    const int bh = lid / (int)gridDim.x, b = bh / a.H, h = bh % a.H;
     const int r = lane & 15, quad = lane >> 4;
 
     bf16x8 bq[2];
@@ -96,52 +132,73 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(llsa_attn_fwd_args a) {
     const bf16* vt = (const bf16*)a.vt + (int64_t)bh * N1 * (kD * kBlk);
     const bf16* pk = (const bf16*)a.pk + (int64_t)bh * N1 * kD;
     const bf16* pvt = (const bf16*)a.pvt + (int64_t)bh * N2 * (kD * kBlk);
-    const bf16* kb[4];
-    const bf16* vtb[4];
+    const bf16* pk2 = (a.levels == 2) ? (const bf16*)a.pk2 + (int64_t)bh * N2 * kD : nullptr;
+    const bf16* pv2t = (a.levels == 2) ? (const bf16*)a.pv2t + (int64_t)bh * (N2 / kBlk) * (kD * kBlk) : nullptr;
+    __shared__ int ids_lds[4][2][kWave];
+    wave_sort_ids(a.idx + ((int64_t)bh * N1 + g) * a.T, a.T, ids_lds[wave][0], ids_lds[wave][1], lane);
+    const int* ip = ids_lds[wave][1];
+    const int* pip = (a.levels == 2) ? a.pidx + ((int64_t)bh * N2 + g / kBlk) * a.T2 : nullptr;
 
-    const int* ip = a.idx + ((int64_t)bh * N1 + g) * a.T;
-    for (int t = 0; t < a.T / 4; t++) {
+    // step t of the KV list: fine blocks, then (l2) the parent's level-1 pooled blocks, then
+    // every block of the coarsest pooled level
+    const int n_fine = a.T / NB;
+    const int n_mid = (a.levels == 2) ? a.T2 / NB : 0;
+    const int n_dense = ((a.levels == 2) ? N2 / kBlk : N1 / kBlk) / NB;
+    const int n_steps = n_fine + n_mid + n_dense;
+    const float w_last = (a.levels == 2) ? a.w2 : a.w1;
+    auto describe = [&](int t, StepDesc<NB>& d) {
+        if (t < n_fine) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const int blk = clampi(ip[4 * t + j], 0, N1 - 1);
-            kb[j] = kbase + (int64_t)blk * kBlk * a.skn;
-            vtb[j] = vt + (int64_t)blk * (kD * kBlk);
-        }
-        fwd_tile(st, bq, kb, a.skn, vtb, 1.f, lane);
-    }
-    float wcur;
-    if (a.levels == 2) {
-        const int* pip = a.pidx + ((int64_t)bh * N2 + g / kBlk) * a.T2;
-        for (int t = 0; t < a.T2 / 4; t++) {
-#pragma unroll
-            for (int j = 0; j < 4; j++) {
-                const int blk = clampi(pip[4 * t + j], 0, N2 - 1);
-                kb[j] = pk + (int64_t)blk * kBlk * kD;
-                vtb[j] = pvt + (int64_t)blk * (kD * kBlk);
+            for (int j = 0; j < NB; j++) {
+                const int blk = clampi(__builtin_amdgcn_readfirstlane(ip[NB * t + j]), 0, N1 - 1);
+                d.kb[j] = kbase + (int64_t)blk * kBlk * a.skn;
+                d.vtb[j] = vt + (int64_t)blk * (kD * kBlk);
             }
-            fwd_tile(st, bq, kb, kD, vtb, t == 0 ? 1.f / a.w1 : 1.f, lane);
-        }
-        const bf16* pk2 = (const bf16*)a.pk2 + (int64_t)bh * N2 * kD;
-        const bf16* pv2t = (const bf16*)a.pv2t + (int64_t)bh * (N2 / kBlk) * (kD * kBlk);
-        for (int t = 0; t < N2 / 64; t++) {
+            d.ks = a.skn;
+            d.wratio = 1.f;
+        } else if (t < n_fine + n_mid) {
+            const int u = t - n_fine;
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                kb[j] = pk2 + (int64_t)(4 * t + j) * kBlk * kD;
-                vtb[j] = pv2t + (int64_t)(4 * t + j) * (kD * kBlk);
+            for (int j = 0; j < NB; j++) {
+                const int blk = clampi(pip[NB * u + j], 0, N2 - 1);
+                d.kb[j] = pk + (int64_t)blk * kBlk * kD;
+                d.vtb[j] = pvt + (int64_t)blk * (kD * kBlk);
             }
-            fwd_tile(st, bq, kb, kD, vtb, t == 0 ? a.w1 / a.w2 : 1.f, lane);
-        }
-        wcur = a.w2;
-    } else {
-        for (int t = 0; t < N1 / 64; t++) {
+            d.ks = kD;
+            d.wratio = (u == 0) ? 1.f / a.w1 : 1.f;
+        } else {
+            const int u = t - n_fine - n_mid;
+            const bf16* kk = (a.levels == 2) ? pk2 : pk;
+            const bf16* vv = (a.levels == 2) ? pv2t : pvt;
 #pragma unroll
-            for (int j = 0; j < 4; j++) {
-                kb[j] = pk + (int64_t)(4 * t + j) * kBlk * kD;
-                vtb[j] = pvt + (int64_t)(4 * t + j) * (kD * kBlk);
+            for (int j = 0; j < NB; j++) {
+                d.kb[j] = kk + (int64_t)(NB * u + j) * kBlk * kD;
+                d.vtb[j] = vv + (int64_t)(NB * u + j) * (kD * kBlk);
             }
-            fwd_tile(st, bq, kb, kD, vtb, t == 0 ? 1.f / a.w1 : 1.f, lane);
+            d.ks = kD;
+            d.wratio = (u == 0) ? ((a.levels == 2) ? a.w1 / a.w2 : 1.f / a.w1) : 1.f;
         }
-        wcur = a.w1;
+    };
+
+    // The prefetch is unconditional (past the end it re-reads the last step) so that the loop
+    // body is straight-line code: with the loads inside a branch the compiler has to drain the
+    // memory queue (s_waitcnt vmcnt(0)) before every step and the overlap is lost.
+    KvRegs<NB> ra, rb;
+    StepDesc<NB> d;
+    float wa, wb;
+    describe(0, d);
+    load_step(ra, d, lane);
+    wa = d.wratio;
+    for (int t = 0; t < n_steps; t += 2) {
+        describe(min(t + 1, n_steps - 1), d);
+        load_step(rb, d, lane);
+        wb = d.wratio;
+        compute_step(st, bq, ra, wa);
+        if (t + 1 >= n_steps) break;
+        describe(min(t + 2, n_steps - 1), d);
+        load_step(ra, d, lane);
+        wa = d.wratio;
+        compute_step(st, bq, rb, wb);
     }
 
     const float L = quad_sum(st.lsum);
@@ -149,7 +206,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(llsa_attn_fwd_args a) {
     bf16* op = (bf16*)a.o + b * a.sob + h * a.soh + (int64_t)(g * kBlk + r) * a.son + quad * 4;
 #pragma unroll
     for (int dt = 0; dt < 4; dt++) st8(op + dt * 16, cvt4(st.acc[dt] * inv));
-    if (quad == 0) a.lse[(int64_t)bh * a.N + g * kBlk + r] = (st.m2 + __builtin_amdgcn_logf(L * wcur)) * kLn2;
+    if (quad == 0) a.lse[(int64_t)bh * a.N + g * kBlk + r] = (st.m2 + __builtin_amdgcn_logf(L * w_last)) * kLn2;
 }
 
 }  // namespace llsa
@@ -178,6 +235,7 @@ extern "C" int llsa_attn_fwd(const llsa_attn_fwd_args* a, void* stream) {
                      stride_ok(a->skn) && (a->sob % 4 == 0) && (a->soh % 4 == 0) && (a->son % 4 == 0),
                  "attn_fwd: row strides must keep rows 16-byte aligned");
     const int N1 = a->N / 16;
-    hipLaunchKernelGGL(attn_fwd_kernel, dim3((N1 + 3) / 4, a->B * a->H), dim3(256), 0, (hipStream_t)stream, *a);
+    hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_fwd_kernel<LLSA_FWD_NB>), dim3((N1 + 3) / 4, a->B * a->H), dim3(256), 0,
+                       (hipStream_t)stream, *a);
     return launch_status("attn_fwd");
 }

@@ -76,6 +76,45 @@ __device__ __forceinline__ float quad_sum(float v) {
     return v;
 }
 
+// XCD-aware workgroup order.  The 8 XCDs of the chip each have a private L2 and receive
+// workgroups round-robin by linear id (id % 8).  Neighbouring logical work items (query or
+// key blocks that are close in Z-order) read overlapping K/V/Q rows, so they should share an
+// L2: this maps the hardware id to a logical id such that every XCD walks one contiguous
+// range of the (x, y) grid.  Returns the logical linear id in [0, gridDim.x * gridDim.y).
+constexpr int kXcds = 8;
+__device__ __forceinline__ int xcd_logical_id() {
+    const int total = gridDim.x * gridDim.y;
+    const int lin = blockIdx.y * gridDim.x + blockIdx.x;
+    const int xcd = lin % kXcds, slot = lin / kXcds;
+    const int q = total / kXcds, rem = total % kXcds;
+    return xcd * q + (xcd < rem ? xcd : rem) + slot;
+}
+
+// Sorts the T (<= 64) block ids at src ascending into `out` (LDS, 64 ints; `tmp` is another 64
+// ints of LDS scratch), one wave, no workgroup barrier.  Attention is invariant to the order of
+// the selected blocks; walking them in ascending order makes sibling waves, whose selections
+// overlap heavily on spatially coherent inputs, touch the same K/V rows at about the same time,
+// so that they hit in the CU's L1 instead of going to L2 again.
+__device__ __forceinline__ void wave_sort_ids(const int* src, int T, int* tmp, int* out, int lane) {
+    int v = 0;
+    if (lane < T) {
+        v = src[lane];
+        tmp[lane] = v;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    if (lane < T) {
+        int rank = 0;
+        for (int j = 0; j < T; j++) {
+            const int o = tmp[j];
+            rank += (o < v || (o == v && j < lane)) ? 1 : 0;
+        }
+        out[rank] = v;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
 __device__ __forceinline__ int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
 
 }  // namespace llsa
