@@ -19,10 +19,15 @@
  *   - return value: 0 on success, negative on a rejected argument or a launch error;
  *     llsa_last_error_string() describes the last failure on the calling thread
  *
- * Block-transposed layout ("xt" below): a (B,H,n,64) tensor viewed as blocks of 16 rows,
- * each block stored channel-major: xt[b][h][blk][d][t] = x[b][h][16*blk + t][d].  The
- * MFMA kernels read one operand of every product whose contraction runs over tokens
- * (P.V, dS.K, P^T.dO, dS^T.Q) from this layout with plain 8-byte loads.
+ * Operand tiles ("xr", "xt" below).  The attention kernels do not read K/V/Q/dO row-major: a
+ * (B,H,n,64) tensor is cut into blocks of 16 rows and every block (1024 elements) is stored
+ * in the order the 64 lanes of a wave consume it as an MFMA operand, so that each operand
+ * load is one contiguous, fully coalesced access.  Element (row t of the block, channel c):
+ *   R tile (products that contract over channels: Q.K^T, dO.V^T)
+ *        offset = ((c >> 3) * 16 + t) * 8 + (c & 7)
+ *   T tile (products that contract over the block's 16 tokens: P.V, dS.K, P^T.dO, dS^T.Q)
+ *        offset = (((c >> 4) * 4 + (t >> 2)) * 16 + (c & 15)) * 4 + (t & 3)
+ * Tiled tensors are (B,H,n/16,1024) contiguous.  llsa_pool_pyramid_fwd writes them.
  */
 #ifndef LLSA_HIP_H
 #define LLSA_HIP_H
@@ -51,11 +56,13 @@ typedef struct llsa_pool_item {
     const void* x;          /* (B,H,n,64) bf16, strides below                                   */
     int64_t sxb, sxh, sxn;
     int32_t n;              /* rows of this item, multiple of 16                                */
-    int32_t rope;           /* rotate x with `freq` first (needs xrot)                          */
+    int32_t rope;           /* rotate x with `freq` first                                       */
     void* y1;               /* (B,H,n/16,64)   mean over 16 rows, contiguous, or NULL           */
     void* y2;               /* (B,H,n/256,64)  mean over 16 rows of y1, or NULL (n % 256 == 0)  */
-    void* xt;               /* (B,H,n/16,64,16) block-transposed (rotated) x, or NULL           */
-    void* y1t;              /* (B,H,n/256,64,16) block-transposed y1, or NULL (n % 256 == 0)    */
+    void* xr;               /* (B,H,n/16,1024)  R tiles of (rotated) x, or NULL                 */
+    void* xt;               /* (B,H,n/16,1024)  T tiles of (rotated) x, or NULL                 */
+    void* y1r;              /* (B,H,n/256,1024) R tiles of y1, or NULL (n % 256 == 0)           */
+    void* y1t;              /* (B,H,n/256,1024) T tiles of y1, or NULL (n % 256 == 0)           */
     void* xrot;             /* (B,H,n,64) contiguous rotated x, or NULL                         */
 } llsa_pool_item;
 
@@ -106,13 +113,13 @@ int llsa_topk_sparse(const void* pq, const void* pk, const int32_t* parent_idx, 
  * levels == 2.
  * ---------------------------------------------------------------------------------------- */
 typedef struct llsa_attn_fwd_args {
-    const void* q;  int64_t sqb, sqh, sqn;     /* (B,H,N,64)                                      */
-    const void* k;  int64_t skb, skh, skn;     /* (B,H,N,64)                                      */
-    const void* vt;                            /* (B,H,N/16,64,16)  block-transposed v            */
-    const void* pk;                            /* (B,H,N/16,64)     level-1 pooled k, contiguous  */
-    const void* pvt;                           /* (B,H,N/256,64,16) block-transposed pooled v     */
-    const void* pk2;                           /* (B,H,N/256,64)    level-2 pooled k (levels==2)  */
-    const void* pv2t;                          /* (B,H,N/4096,64,16)                              */
+    const void* qr;                            /* (B,H,N/16,1024)   R tiles of q                  */
+    const void* kr;                            /* (B,H,N/16,1024)   R tiles of k                  */
+    const void* vt;                            /* (B,H,N/16,1024)   T tiles of v                  */
+    const void* pkr;                           /* (B,H,N/256,1024)  R tiles of level-1 pooled k   */
+    const void* pvt;                           /* (B,H,N/256,1024)  T tiles of level-1 pooled v   */
+    const void* pk2r;                          /* (B,H,N/4096,1024) R tiles of level-2 pooled k   */
+    const void* pv2t;                          /* (B,H,N/4096,1024) T tiles of level-2 pooled v   */
     const int32_t* idx;                        /* (B,H,N/16,T)   selected fine blocks             */
     const int32_t* pidx;                       /* (B,H,N/256,T2) selected coarse blocks (l2)      */
     void* o;        int64_t sob, soh, son;     /* (B,H,N,64) out                                  */
@@ -153,16 +160,15 @@ int64_t llsa_work_list_len(int Mb, int Kb, int T, int chunk);
  * ---------------------------------------------------------------------------------------- */
 typedef struct llsa_attn_bwd_args {
     const void* dout; int64_t sdob, sdoh, sdon;  /* (B,H,N,64) upstream gradient                 */
-    const void* q;    int64_t sqb, sqh, sqn;
-    const void* k;    int64_t skb, skh, skn;
-    const void* v;    int64_t svb, svh, svn;
-    const void* o;    int64_t sob, soh, son;
+    const void* o;    int64_t sob, soh, son;     /* (B,H,N,64) forward output                     */
     const float* lse;                            /* (B,H,N)                                       */
-    const void* pk;  const void* pv;             /* (B,H,N/16,64) contiguous                      */
-    const void* pk2; const void* pv2;            /* (B,H,N/256,64) contiguous (levels == 2)       */
-    const void* qt;  const void* kt;             /* block-transposed q, k   (B,H,N/16,64,16)      */
-    const void* pkt;                             /* block-transposed pk     (B,H,N/256,64,16)     */
-    const void* pk2t;                            /* block-transposed pk2    (B,H,N/4096,64,16)    */
+    const void* qr;  const void* qt;             /* R and T tiles of q   (B,H,N/16,1024)          */
+    const void* kr;  const void* kt;             /* R and T tiles of k                            */
+    const void* vr;                              /* R tiles of v                                  */
+    const void* pkr; const void* pkt;            /* R and T tiles of pk  (B,H,N/256,1024)         */
+    const void* pvr;                             /* R tiles of pv                                 */
+    const void* pk2r; const void* pk2t;          /* R and T tiles of pk2 (B,H,N/4096,1024)        */
+    const void* pv2r;                            /* R tiles of pv2                                */
     const int32_t* idx;  const int32_t* pidx;
     const int32_t* off;  const int32_t* flat;  const int32_t* work;    /* transposed idx  (Kb = N/16)     */
     const int32_t* poff; const int32_t* pflat; const int32_t* pwork;   /* transposed pidx (Kb = N/256)    */

@@ -19,13 +19,13 @@ c_void_p, c_int, c_int32, c_int64, c_float = C.c_void_p, C.c_int, C.c_int32, C.c
 class PoolItem(C.Structure):
     _fields_ = [("x", c_void_p), ("sxb", c_int64), ("sxh", c_int64), ("sxn", c_int64),
                 ("n", c_int32), ("rope", c_int32),
-                ("y1", c_void_p), ("y2", c_void_p), ("xt", c_void_p), ("y1t", c_void_p), ("xrot", c_void_p)]
+                ("y1", c_void_p), ("y2", c_void_p), ("xr", c_void_p), ("xt", c_void_p), ("y1r", c_void_p),
+                ("y1t", c_void_p), ("xrot", c_void_p)]
 
 
 class AttnFwdArgs(C.Structure):
-    _fields_ = [("q", c_void_p), ("sqb", c_int64), ("sqh", c_int64), ("sqn", c_int64),
-                ("k", c_void_p), ("skb", c_int64), ("skh", c_int64), ("skn", c_int64),
-                ("vt", c_void_p), ("pk", c_void_p), ("pvt", c_void_p), ("pk2", c_void_p), ("pv2t", c_void_p),
+    _fields_ = [("qr", c_void_p), ("kr", c_void_p), ("vt", c_void_p), ("pkr", c_void_p), ("pvt", c_void_p),
+                ("pk2r", c_void_p), ("pv2t", c_void_p),
                 ("idx", c_void_p), ("pidx", c_void_p),
                 ("o", c_void_p), ("sob", c_int64), ("soh", c_int64), ("son", c_int64),
                 ("lse", c_void_p),
@@ -40,9 +40,10 @@ def _t3(name):
 class AttnBwdArgs(C.Structure):
     _fields_ = (
         [("dout", c_void_p), ("sdob", c_int64), ("sdoh", c_int64), ("sdon", c_int64)]
-        + _t3("q") + _t3("k") + _t3("v") + _t3("o")
-        + [("lse", c_void_p), ("pk", c_void_p), ("pv", c_void_p), ("pk2", c_void_p), ("pv2", c_void_p),
-           ("qt", c_void_p), ("kt", c_void_p), ("pkt", c_void_p), ("pk2t", c_void_p),
+        + _t3("o")
+        + [("lse", c_void_p), ("qr", c_void_p), ("qt", c_void_p), ("kr", c_void_p), ("kt", c_void_p), ("vr", c_void_p),
+           ("pkr", c_void_p), ("pkt", c_void_p), ("pvr", c_void_p), ("pk2r", c_void_p), ("pk2t", c_void_p),
+           ("pv2r", c_void_p),
            ("idx", c_void_p), ("pidx", c_void_p), ("off", c_void_p), ("flat", c_void_p), ("work", c_void_p),
            ("poff", c_void_p), ("pflat", c_void_p), ("pwork", c_void_p)]
         + [("dq", c_void_p), ("sdqb", c_int64), ("sdqh", c_int64), ("sdqn", c_int64),

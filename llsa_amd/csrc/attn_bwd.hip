@@ -19,11 +19,11 @@
 namespace llsa {
 
 // ---------------------------------------------------------------------------------------
-// delta = rowsum(O * dO) in fp32, and the block-transposed copy of dO.
+// delta = rowsum(O * dO) in fp32, and the R and T operand tiles of dO.
 // Same thread mapping as the pooling kernel: 16 blocks x 8 channel chunks per workgroup.
 // ---------------------------------------------------------------------------------------
 __global__ __launch_bounds__(128) void bwd_pre_kernel(llsa_attn_bwd_args a, float* __restrict__ delta,
-                                                      bf16* __restrict__ dot) {
+                                                      bf16* __restrict__ dor, bf16* __restrict__ dot) {
     const int N1 = a.N / kBlk;
     const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
     const int t = threadIdx.x, c = t & 7, r = t >> 3;
@@ -55,37 +55,49 @@ __global__ __launch_bounds__(128) void bwd_pre_kernel(llsa_attn_bwd_args a, floa
 #pragma unroll
         for (int i = 0; i < 16; i++) dp[i] = part[i];
     }
-    bf16* xt = dot + (((int64_t)bh * N1 + blk) * kD + c * 8) * kBlk;
+    bf16* xr = dor + ((int64_t)bh * N1 + blk) * kTile + c * 128;
 #pragma unroll
-    for (int e = 0; e < 8; e++) {
-        bf16x8 lo, hi;
+    for (int i = 0; i < 16; i++) st16(xr + i * 8, gv[i]);
+    bf16* xt = dot + ((int64_t)bh * N1 + blk) * kTile;
 #pragma unroll
-        for (int i = 0; i < 8; i++) {
-            lo[i] = gv[i][e];
-            hi[i] = gv[8 + i][e];
+    for (int e = 0; e < 8; e++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            bf16x4 v;
+#pragma unroll
+            for (int j = 0; j < 4; j++) v[j] = gv[4 * q + j][e];
+            st8(xt + t_tile_off(4 * q, 8 * c + e), v);
         }
-        st16(xt + e * kBlk, lo);
-        st16(xt + e * kBlk + 8, hi);
-    }
 }
 
 // ---------------------------------------------------------------------------------------
 // dQ: one wave per query block, key blocks taken two at a time (32 keys = one MFMA K step)
 // ---------------------------------------------------------------------------------------
+// kb / vb / ktb: R tile of K, R tile of V, T tile of K for the two key blocks of the pair
 __device__ __forceinline__ void dq_pair(f32x4 dq[4], const bf16x8 bq[2], const bf16x8 bdo[2], float lse2, float delta,
-                                        float w, const bf16* const kb[2], int64_t ks, const bf16* const vb[2], int64_t vs,
+                                        float w, const bf16* const kb[2], const bf16* const vb[2],
                                         const bf16* const ktb[2], int lane) {
-    const int r = lane & 15, quad = lane >> 4;
+    bf16x8 kreg[2][2], vreg[2][2];
+    bf16x4 ktreg[2][4];
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        kreg[j][0] = ld16(kb[j] + lane * 8);
+        kreg[j][1] = ld16(kb[j] + 512 + lane * 8);
+        vreg[j][0] = ld16(vb[j] + lane * 8);
+        vreg[j][1] = ld16(vb[j] + 512 + lane * 8);
+    }
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) ktreg[j][dt] = ld8(ktb[j] + dt * 256 + lane * 4);
     bf16x8 bds;
 #pragma unroll
     for (int j = 0; j < 2; j++) {
-        const bf16* kp = kb[j] + r * ks + quad * 8;
-        const bf16* vp = vb[j] + r * vs + quad * 8;
         f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
-        s = mfma_bf16(ld16(kp), bq[0], s);
-        s = mfma_bf16(ld16(kp + 32), bq[1], s);
-        dp = mfma_bf16(ld16(vp), bdo[0], dp);
-        dp = mfma_bf16(ld16(vp + 32), bdo[1], dp);
+        s = mfma_bf16(kreg[j][0], bq[0], s);
+        s = mfma_bf16(kreg[j][1], bq[1], s);
+        dp = mfma_bf16(vreg[j][0], bdo[0], dp);
+        dp = mfma_bf16(vreg[j][1], bdo[1], dp);
 #pragma unroll
         for (int e = 0; e < 4; e++) {
             const float p = exp2_fast(fmaf(s[e], kScaleLog2e, -lse2)) * w;
@@ -93,13 +105,11 @@ __device__ __forceinline__ void dq_pair(f32x4 dq[4], const bf16x8 bq[2], const b
         }
     }
 #pragma unroll
-    for (int dt = 0; dt < 4; dt++) {
-        const int off = (dt * 16 + r) * kBlk + quad * 4;
-        dq[dt] = mfma_bf16(cat(ld8(ktb[0] + off), ld8(ktb[1] + off)), bds, dq[dt]);
-    }
+    for (int dt = 0; dt < 4; dt++) dq[dt] = mfma_bf16(cat(ktreg[0][dt], ktreg[1][dt]), bds, dq[dt]);
 }
 
-__global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, const float* __restrict__ delta) {
+__global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, const float* __restrict__ delta,
+                                                      const bf16* __restrict__ dor) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int N1 = a.N / kBlk, N2 = N1 / kBlk;
@@ -112,12 +122,12 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, cons
 
     bf16x8 bq[2], bdo[2];
     {
-        const bf16* qp = (const bf16*)a.q + b * a.sqb + h * a.sqh + (int64_t)tok * a.sqn + quad * 8;
-        const bf16* gp = (const bf16*)a.dout + b * a.sdob + h * a.sdoh + (int64_t)tok * a.sdon + quad * 8;
+        const bf16* qp = (const bf16*)a.qr + ((int64_t)bh * N1 + g) * kTile + lane * 8;
+        const bf16* gp = dor + ((int64_t)bh * N1 + g) * kTile + lane * 8;
         bq[0] = ld16(qp);
-        bq[1] = ld16(qp + 32);
+        bq[1] = ld16(qp + 512);
         bdo[0] = ld16(gp);
-        bdo[1] = ld16(gp + 32);
+        bdo[1] = ld16(gp + 512);
     }
     const float lse2 = a.lse[(int64_t)bh * a.N + tok] * kLog2e;
     const float dl = delta[(int64_t)bh * a.N + tok];
@@ -125,12 +135,12 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, cons
 #pragma unroll
     for (int dt = 0; dt < 4; dt++) dq[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const bf16* kbase = (const bf16*)a.k + b * a.skb + h * a.skh;
-    const bf16* vbase = (const bf16*)a.v + b * a.svb + h * a.svh;
-    const bf16* kt = (const bf16*)a.kt + (int64_t)bh * N1 * (kD * kBlk);
-    const bf16* pk = (const bf16*)a.pk + (int64_t)bh * N1 * kD;
-    const bf16* pv = (const bf16*)a.pv + (int64_t)bh * N1 * kD;
-    const bf16* pkt = (const bf16*)a.pkt + (int64_t)bh * N2 * (kD * kBlk);
+    const bf16* kr = (const bf16*)a.kr + (int64_t)bh * N1 * kTile;
+    const bf16* vr = (const bf16*)a.vr + (int64_t)bh * N1 * kTile;
+    const bf16* kt = (const bf16*)a.kt + (int64_t)bh * N1 * kTile;
+    const bf16* pk = (const bf16*)a.pkr + (int64_t)bh * N2 * kTile;
+    const bf16* pv = (const bf16*)a.pvr + (int64_t)bh * N2 * kTile;
+    const bf16* pkt = (const bf16*)a.pkt + (int64_t)bh * N2 * kTile;
     const bf16 *kb[2], *vb[2], *ktb[2];
 
     __shared__ int ids_lds[4][2][kWave];
@@ -140,11 +150,11 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, cons
 #pragma unroll
         for (int j = 0; j < 2; j++) {
             const int blk = clampi(__builtin_amdgcn_readfirstlane(ip[2 * t + j]), 0, N1 - 1);
-            kb[j] = kbase + (int64_t)blk * kBlk * a.skn;
-            vb[j] = vbase + (int64_t)blk * kBlk * a.svn;
-            ktb[j] = kt + (int64_t)blk * (kD * kBlk);
+            kb[j] = kr + (int64_t)blk * kTile;
+            vb[j] = vr + (int64_t)blk * kTile;
+            ktb[j] = kt + (int64_t)blk * kTile;
         }
-        dq_pair(dq, bq, bdo, lse2, dl, 1.f, kb, a.skn, vb, a.svn, ktb, lane);
+        dq_pair(dq, bq, bdo, lse2, dl, 1.f, kb, vb, ktb, lane);
     }
     if (a.levels == 2) {
         const int* pip = a.pidx + ((int64_t)bh * N2 + g / kBlk) * a.T2;
@@ -152,33 +162,33 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, cons
 #pragma unroll
             for (int j = 0; j < 2; j++) {
                 const int blk = clampi(pip[2 * t + j], 0, N2 - 1);
-                kb[j] = pk + (int64_t)blk * kBlk * kD;
-                vb[j] = pv + (int64_t)blk * kBlk * kD;
-                ktb[j] = pkt + (int64_t)blk * (kD * kBlk);
+                kb[j] = pk + (int64_t)blk * kTile;
+                vb[j] = pv + (int64_t)blk * kTile;
+                ktb[j] = pkt + (int64_t)blk * kTile;
             }
-            dq_pair(dq, bq, bdo, lse2, dl, a.w1, kb, kD, vb, kD, ktb, lane);
+            dq_pair(dq, bq, bdo, lse2, dl, a.w1, kb, vb, ktb, lane);
         }
-        const bf16* pk2 = (const bf16*)a.pk2 + (int64_t)bh * N2 * kD;
-        const bf16* pv2 = (const bf16*)a.pv2 + (int64_t)bh * N2 * kD;
-        const bf16* pk2t = (const bf16*)a.pk2t + (int64_t)bh * (N2 / kBlk) * (kD * kBlk);
+        const bf16* pk2 = (const bf16*)a.pk2r + (int64_t)bh * (N2 / kBlk) * kTile;
+        const bf16* pv2 = (const bf16*)a.pv2r + (int64_t)bh * (N2 / kBlk) * kTile;
+        const bf16* pk2t = (const bf16*)a.pk2t + (int64_t)bh * (N2 / kBlk) * kTile;
         for (int t = 0; t < N2 / 32; t++) {
 #pragma unroll
             for (int j = 0; j < 2; j++) {
-                kb[j] = pk2 + (int64_t)(2 * t + j) * kBlk * kD;
-                vb[j] = pv2 + (int64_t)(2 * t + j) * kBlk * kD;
-                ktb[j] = pk2t + (int64_t)(2 * t + j) * (kD * kBlk);
+                kb[j] = pk2 + (int64_t)(2 * t + j) * kTile;
+                vb[j] = pv2 + (int64_t)(2 * t + j) * kTile;
+                ktb[j] = pk2t + (int64_t)(2 * t + j) * kTile;
             }
-            dq_pair(dq, bq, bdo, lse2, dl, a.w2, kb, kD, vb, kD, ktb, lane);
+            dq_pair(dq, bq, bdo, lse2, dl, a.w2, kb, vb, ktb, lane);
         }
     } else {
         for (int t = 0; t < N1 / 32; t++) {
 #pragma unroll
             for (int j = 0; j < 2; j++) {
-                kb[j] = pk + (int64_t)(2 * t + j) * kBlk * kD;
-                vb[j] = pv + (int64_t)(2 * t + j) * kBlk * kD;
-                ktb[j] = pkt + (int64_t)(2 * t + j) * (kD * kBlk);
+                kb[j] = pk + (int64_t)(2 * t + j) * kTile;
+                vb[j] = pv + (int64_t)(2 * t + j) * kTile;
+                ktb[j] = pkt + (int64_t)(2 * t + j) * kTile;
             }
-            dq_pair(dq, bq, bdo, lse2, dl, a.w1, kb, kD, vb, kD, ktb, lane);
+            dq_pair(dq, bq, bdo, lse2, dl, a.w1, kb, vb, ktb, lane);
         }
     }
 
@@ -212,12 +222,10 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, cons
 enum { MODE_FINE = 0, MODE_SPARSE1 = 1, MODE_DENSE = 2 };
 
 struct KSideParams {
-    const bf16* q;   int64_t sqb, sqh, sqn;
-    const bf16* dout; int64_t sdob, sdoh, sdon;
-    const bf16* qt;  const bf16* dot;             // block-transposed q and dO, (BH, N1, 64, 16)
+    const bf16* qr;  const bf16* dor;             // R tiles of q and dO, (BH, N1, 1024)
+    const bf16* qt;  const bf16* dot;             // T tiles of q and dO
     const float* lse; const float* delta;         // (BH, N)
-    const bf16* kk;  int64_t skb, skh, skn;       // the unit's key rows come from here
-    const bf16* vv;  int64_t svb, svh, svn;
+    const bf16* kk;  const bf16* vv;              // R tiles the unit's 16 key rows come from, (BH, n_units, 1024)
     const int* off;  const int* flat;             // CSR of the list (FINE: per K block, SPARSE1: per coarse block)
     const int* work;                              // work list over that CSR (see transpose.hip)
     bf16* dk; int64_t sdkb, sdkh, sdkn;           // bf16 outputs (FINE, SPARSE1)
@@ -230,39 +238,54 @@ struct KSideParams {
     float w;
 };
 
+// Two query blocks (g0, g1; g1 < 0: only one) against the unit's 16 key rows.  All operands of
+// both blocks are fetched first -- eight 1 KB and eight 512 B coalesced loads -- then used.
 __device__ __forceinline__ void kside_pair(f32x4 dk[4], f32x4 dv[4], const bf16x8 bk[2], const bf16x8 bv[2], float w,
-                                           int g0, int g1, const KSideParams& p, const bf16* qb, const bf16* gb,
-                                           const bf16* qtb, const bf16* dotb, const float* lseb, const float* dlb,
-                                           int lane) {
-    const int r = lane & 15, quad = lane >> 4;
+                                           int g0, int g1, const bf16* qrb, const bf16* dorb, const bf16* qtb,
+                                           const bf16* dotb, const float* lseb, const float* dlb, int lane) {
+    const int quad = lane >> 4;
+    const int gg[2] = {g0, (g1 < 0) ? g0 : g1};
+    bf16x8 aq[2][2], ag[2][2];
+    bf16x4 tq[2][4], tg[2][4];
+    f32x4 l4[2], d4[2];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const int64_t base = (int64_t)gg[u] * kTile;
+        aq[u][0] = ld16(qrb + base + lane * 8);
+        aq[u][1] = ld16(qrb + base + 512 + lane * 8);
+        ag[u][0] = ld16(dorb + base + lane * 8);
+        ag[u][1] = ld16(dorb + base + 512 + lane * 8);
+        l4[u] = *reinterpret_cast<const f32x4*>(lseb + gg[u] * kBlk + quad * 4);
+        d4[u] = *reinterpret_cast<const f32x4*>(dlb + gg[u] * kBlk + quad * 4);
+    }
+#pragma unroll
+    for (int u = 0; u < 2; u++)
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+            tq[u][dt] = ld8(qtb + (int64_t)gg[u] * kTile + dt * 256 + lane * 4);
+            tg[u][dt] = ld8(dotb + (int64_t)gg[u] * kTile + dt * 256 + lane * 4);
+        }
     bf16x8 bp, bds;
 #pragma unroll
     for (int u = 0; u < 2; u++) {
         const bool valid = (u == 0) || (g1 >= 0);
-        const int g = (u == 0 || g1 < 0) ? g0 : g1;
-        const bf16* qp = qb + (int64_t)(g * kBlk + r) * p.sqn + quad * 8;
-        const bf16* gp = gb + (int64_t)(g * kBlk + r) * p.sdon + quad * 8;
         f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
-        s = mfma_bf16(ld16(qp), bk[0], s);
-        s = mfma_bf16(ld16(qp + 32), bk[1], s);
-        dp = mfma_bf16(ld16(gp), bv[0], dp);
-        dp = mfma_bf16(ld16(gp + 32), bv[1], dp);
-        const f32x4 l4 = *reinterpret_cast<const f32x4*>(lseb + g * kBlk + quad * 4);
-        const f32x4 d4 = *reinterpret_cast<const f32x4*>(dlb + g * kBlk + quad * 4);
+        s = mfma_bf16(aq[u][0], bk[0], s);
+        s = mfma_bf16(aq[u][1], bk[1], s);
+        dp = mfma_bf16(ag[u][0], bv[0], dp);
+        dp = mfma_bf16(ag[u][1], bv[1], dp);
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            float pe = exp2_fast(fmaf(s[e], kScaleLog2e, -l4[e] * kLog2e)) * w;
+            float pe = exp2_fast(fmaf(s[e], kScaleLog2e, -l4[u][e] * kLog2e)) * w;
             if (!valid) pe = 0.f;
             bp[u * 4 + e] = (bf16)pe;
-            bds[u * 4 + e] = (bf16)(pe * (dp[e] - d4[e]));
+            bds[u * 4 + e] = (bf16)(pe * (dp[e] - d4[u][e]));
         }
     }
-    const int ga = g0, gb2 = (g1 < 0) ? g0 : g1;
 #pragma unroll
     for (int dt = 0; dt < 4; dt++) {
-        const int off = (dt * 16 + r) * kBlk + quad * 4;
-        dv[dt] = mfma_bf16(cat(ld8(dotb + (int64_t)ga * (kD * kBlk) + off), ld8(dotb + (int64_t)gb2 * (kD * kBlk) + off)), bp, dv[dt]);
-        dk[dt] = mfma_bf16(cat(ld8(qtb + (int64_t)ga * (kD * kBlk) + off), ld8(qtb + (int64_t)gb2 * (kD * kBlk) + off)), bds, dk[dt]);
+        dv[dt] = mfma_bf16(cat(tg[0][dt], tg[1][dt]), bp, dv[dt]);
+        dk[dt] = mfma_bf16(cat(tq[0][dt], tq[1][dt]), bds, dk[dt]);
     }
 }
 
@@ -321,22 +344,22 @@ __global__ __launch_bounds__(256) void attn_kside_kernel(KSideParams p) {
     }
     {
         bf16x8 bk[2], bv[2];
-        const bf16* kp = p.kk + b * p.skb + h * p.skh + (int64_t)(unit * kBlk + r) * p.skn + quad * 8;
-        const bf16* vp = p.vv + b * p.svb + h * p.svh + (int64_t)(unit * kBlk + r) * p.svn + quad * 8;
+        const bf16* kp = p.kk + ((int64_t)bh * p.n_units + unit) * kTile + lane * 8;
+        const bf16* vp = p.vv + ((int64_t)bh * p.n_units + unit) * kTile + lane * 8;
         bk[0] = ld16(kp);
-        bk[1] = ld16(kp + 32);
+        bk[1] = ld16(kp + 512);
         bv[0] = ld16(vp);
-        bv[1] = ld16(vp + 32);
-        const bf16* qb = p.q + b * p.sqb + h * p.sqh;
-        const bf16* gb = p.dout + b * p.sdob + h * p.sdoh;
-        const bf16* qtb = p.qt + (int64_t)bh * N1 * (kD * kBlk);
-        const bf16* dotb = p.dot + (int64_t)bh * N1 * (kD * kBlk);
+        bv[1] = ld16(vp + 512);
+        const bf16* qrb = p.qr + (int64_t)bh * N1 * kTile;
+        const bf16* dorb = p.dor + (int64_t)bh * N1 * kTile;
+        const bf16* qtb = p.qt + (int64_t)bh * N1 * kTile;
+        const bf16* dotb = p.dot + (int64_t)bh * N1 * kTile;
         const float* lseb = p.lse + (int64_t)bh * p.N;
         const float* dlb = p.delta + (int64_t)bh * p.N;
         for (int i = 2 * sub; i < cnt; i += 2 * W) {
             const int g0 = entry(i);
             const int g1 = (i + 1 < cnt) ? entry(i + 1) : -1;
-            kside_pair(dk, dv, bk, bv, p.w, g0, g1, p, qb, gb, qtb, dotb, lseb, dlb, lane);
+            kside_pair(dk, dv, bk, bv, p.w, g0, g1, qrb, dorb, qtb, dotb, lseb, dlb, lane);
         }
     }
 
@@ -453,7 +476,7 @@ static int64_t align256(int64_t x) { return (x + 255) & ~(int64_t)255; }
 constexpr int64_t kSlotBytes = 8 * kWave * sizeof(f32x4);     // one partial: 16 rows x 64 ch x (dK, dV) fp32
 
 struct BwdWorkspace {
-    int64_t delta, dot, part_fine, part_coarse, part_dense, total;
+    int64_t delta, dor, dot, part_fine, part_coarse, part_dense, total;
     int64_t slots_fine, slots_coarse;                           // per (b,h)
 };
 
@@ -467,6 +490,7 @@ static BwdWorkspace bwd_workspace(int B, int H, int N, int T, int T2, int levels
     w.slots_coarse = (levels == 2) ? 2 * (N2 * T2 / LLSA_CHUNK_COARSE) + 2 : 0;
     int64_t o = 0;
     w.delta = o;        o += align256(BH * N * 4);
+    w.dor = o;          o += align256(BH * N * 64 * 2);
     w.dot = o;          o += align256(BH * N * 64 * 2);
     w.part_fine = o;    o += align256(BH * w.slots_fine * kSlotBytes);
     w.part_coarse = o;  o += align256(BH * w.slots_coarse * kSlotBytes);
@@ -488,7 +512,7 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     LLSA_REQUIRE(a != nullptr, "attn_bwd: null args");
     LLSA_REQUIRE(a->levels == 1 || a->levels == 2, "attn_bwd: levels must be 1 or 2");
     LLSA_REQUIRE(a->B > 0 && a->H > 0 && a->N > 0, "attn_bwd: bad B/H/N");
-    LLSA_REQUIRE(a->dout && a->q && a->k && a->v && a->o && a->lse && a->pk && a->pv && a->qt && a->kt && a->pkt && a->idx &&
+    LLSA_REQUIRE(a->dout && a->o && a->lse && a->qr && a->qt && a->kr && a->kt && a->vr && a->pkr && a->pkt && a->pvr && a->idx &&
                      a->off && a->flat && a->dq && a->dk && a->dv && a->dpk && a->dpv && a->workspace,
                  "attn_bwd: null tensor");
     LLSA_REQUIRE(a->T >= 4 && a->T % 4 == 0 && a->T <= a->N / 16, "attn_bwd: topk=%d must be a multiple of 4 and <= N/16", a->T);
@@ -497,15 +521,14 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
         LLSA_REQUIRE(a->N % 1024 == 0, "attn_bwd: llsa_l1 needs N %% 1024 == 0 (N=%d)", a->N);
     } else {
         LLSA_REQUIRE(a->N % 16384 == 0, "attn_bwd: llsa_l2 needs N %% 16384 == 0 (N=%d)", a->N);
-        LLSA_REQUIRE(a->pk2 && a->pv2 && a->pk2t && a->pidx && a->poff && a->pflat && a->dpk2 && a->dpv2, "attn_bwd: level-2 tensors missing");
+        LLSA_REQUIRE(a->pk2r && a->pv2r && a->pk2t && a->pidx && a->poff && a->pflat && a->dpk2 && a->dpv2, "attn_bwd: level-2 tensors missing");
         LLSA_REQUIRE(a->T2 >= 4 && a->T2 % 4 == 0 && a->T2 <= a->N / 256, "attn_bwd: topk2=%d must be a multiple of 4 and <= N/256", a->T2);
         LLSA_REQUIRE(a->w2 > 0.f, "attn_bwd: token_weight_2 must be > 0");
     }
-    const void* al[] = {a->dout, a->q, a->k, a->v, a->o, a->pk, a->pv, a->pk2, a->pv2, a->qt, a->kt, a->pkt, a->pk2t,
+    const void* al[] = {a->dout, a->o, a->qr, a->qt, a->kr, a->kt, a->vr, a->pkr, a->pkt, a->pvr, a->pk2r, a->pk2t, a->pv2r,
                         a->dq, a->dk, a->dv, a->dpk, a->dpv, a->dpk2, a->dpv2, a->workspace, a->freq_dq, a->lse};
     for (const void* p : al) LLSA_REQUIRE(aligned16(p), "attn_bwd: tensors must be 16-byte aligned");
-    const int64_t st[] = {a->sdob, a->sdoh, a->sdon, a->sqb, a->sqh, a->sqn, a->skb, a->skh, a->skn, a->svb, a->svh, a->svn,
-                          a->sob, a->soh, a->son};
+    const int64_t st[] = {a->sdob, a->sdoh, a->sdon, a->sob, a->soh, a->son};
     for (int64_t s : st) LLSA_REQUIRE(stride_ok(s), "attn_bwd: input row strides must keep rows 16-byte aligned");
     const int64_t so[] = {a->sdqb, a->sdqh, a->sdqn, a->sdkb, a->sdkh, a->sdkn, a->sdvb, a->sdvh, a->sdvn};
     for (int64_t s : so) LLSA_REQUIRE(s % 4 == 0, "attn_bwd: output row strides must keep rows 8-byte aligned");
@@ -519,21 +542,21 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     const DensePlan d = dense_plan(B, H, N, a->levels);
     char* ws = (char*)a->workspace;
     float* delta = (float*)(ws + wsp.delta);
+    bf16* dor = (bf16*)(ws + wsp.dor);
     bf16* dot = (bf16*)(ws + wsp.dot);
 
     const int stages = a->stages ? a->stages : 0x7fffffff;
-    if (stages & LLSA_BWD_PRE) hipLaunchKernelGGL(bwd_pre_kernel, dim3((N1 + 15) / 16, BH), dim3(128), 0, s, *a, delta, dot);
-    if (stages & LLSA_BWD_DQ) hipLaunchKernelGGL(attn_dq_kernel, dim3((N1 + 3) / 4, BH), dim3(256), 0, s, *a, (const float*)delta);
+    if (stages & LLSA_BWD_PRE) hipLaunchKernelGGL(bwd_pre_kernel, dim3((N1 + 15) / 16, BH), dim3(128), 0, s, *a, delta, dor, dot);
+    if (stages & LLSA_BWD_DQ)
+        hipLaunchKernelGGL(attn_dq_kernel, dim3((N1 + 3) / 4, BH), dim3(256), 0, s, *a, (const float*)delta, (const bf16*)dor);
 
     KSideParams p;
-    p.q = (const bf16*)a->q; p.sqb = a->sqb; p.sqh = a->sqh; p.sqn = a->sqn;
-    p.dout = (const bf16*)a->dout; p.sdob = a->sdob; p.sdoh = a->sdoh; p.sdon = a->sdon;
+    p.qr = (const bf16*)a->qr; p.dor = dor;
     p.qt = (const bf16*)a->qt; p.dot = dot; p.lse = a->lse; p.delta = delta;
     p.H = H; p.N = N; p.chunk_len = 0;
 
     // fine K/V blocks
-    p.kk = (const bf16*)a->k; p.skb = a->skb; p.skh = a->skh; p.skn = a->skn;
-    p.vv = (const bf16*)a->v; p.svb = a->svb; p.svh = a->svh; p.svn = a->svn;
+    p.kk = (const bf16*)a->kr; p.vv = (const bf16*)a->vr;
     p.off = a->off; p.flat = a->flat; p.flat_stride = (int64_t)N1 * a->T;
     p.work = a->work; p.work_stride = llsa_work_list_len(N1, N1, a->T, LLSA_CHUNK_FINE);
     p.part = (f32x4*)(ws + wsp.part_fine); p.slot_stride = wsp.slots_fine;
@@ -552,8 +575,7 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     const int64_t s2b = (int64_t)H * N2 * 64, s2h = (int64_t)N2 * 64;
     if (a->levels == 2 && (stages & LLSA_BWD_DPKV1)) {
         // level-1 pooled tokens, through the transposed coarse index
-        p.kk = (const bf16*)a->pk; p.skb = s1b; p.skh = s1h; p.skn = 64;
-        p.vv = (const bf16*)a->pv; p.svb = s1b; p.svh = s1h; p.svn = 64;
+        p.kk = (const bf16*)a->pkr; p.vv = (const bf16*)a->pvr;
         p.off = a->poff; p.flat = a->pflat; p.flat_stride = (int64_t)N2 * a->T2;
         p.work = a->pwork; p.work_stride = llsa_work_list_len(N2, N2, a->T2, LLSA_CHUNK_COARSE);
         p.part = (f32x4*)(ws + wsp.part_coarse); p.slot_stride = wsp.slots_coarse;
@@ -570,14 +592,12 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     // range is cut into d.chunks pieces whose partial sums are added afterwards
     if (!(stages & LLSA_BWD_DENSE)) return launch_status("attn_bwd");
     if (a->levels == 2) {
-        p.kk = (const bf16*)a->pk2; p.skb = s2b; p.skh = s2h; p.skn = 64;
-        p.vv = (const bf16*)a->pv2; p.svb = s2b; p.svh = s2h; p.svn = 64;
+        p.kk = (const bf16*)a->pk2r; p.vv = (const bf16*)a->pv2r;
         p.dk = (bf16*)a->dpk2; p.dv = (bf16*)a->dpv2;
         p.sdkb = p.sdvb = s2b; p.sdkh = p.sdvh = s2h;
         p.w = a->w2;
     } else {
-        p.kk = (const bf16*)a->pk; p.skb = s1b; p.skh = s1h; p.skn = 64;
-        p.vv = (const bf16*)a->pv; p.svb = s1b; p.svh = s1h; p.svn = 64;
+        p.kk = (const bf16*)a->pkr; p.vv = (const bf16*)a->pvr;
         p.dk = (bf16*)a->dpk; p.dv = (bf16*)a->dpv;
         p.sdkb = p.sdvb = s1b; p.sdkh = p.sdvh = s1h;
         p.w = a->cgw1;

@@ -2,8 +2,8 @@
 //
 // One wave owns one query block (16 queries).  All products run on the bf16 16x16x32 MFMA
 // in the "transposed" orientation, keys on the M axis and queries on the N axis:
-//     S^T (16 keys x 16 queries) = K_blk (16x64) . Q^T            A = K rows, B = Q rows
-//     O^T (64 ch  x 16 queries) += V_blk^T (64x32 keys) . P^T     A = block-transposed V, B = P^T
+//     S^T (16 keys x 16 queries) = K_blk (16x64) . Q^T            A = R tile of K, B = R tile of Q
+//     O^T (64 ch  x 16 queries) += V_blk^T (64x32 keys) . P^T     A = T tiles of V, B = P^T
 // With this orientation lane l holds, for query l%16, the scores of keys 4*(l/16)..+3 of a
 // tile -- which is exactly the B-operand layout of the second product -- and the O^T
 // accumulator of lane l belongs to the same query, so the soft-max statistics (running
@@ -34,33 +34,29 @@ struct SoftmaxState {
 // Operands of one step = NB 16-key blocks, as they sit in registers between load and use.
 template <int NB>
 struct KvRegs {
-    bf16x8 k[NB][2];     // K rows: block j, channel half
-    bf16x4 v[NB][4];     // block-transposed V: block j, channel tile dt, keys 4*(l/16)..+3
+    bf16x8 k[NB][2];     // K rows (R tile): block j, channel half
+    bf16x4 v[NB][4];     // V (T tile): block j, channel tile dt, keys 4*(l/16)..+3
 };
 
-// Where one step's blocks live.  kb[j] points at row 0 of block j (row stride ks elements),
-// vtb[j] at the block-transposed values of block j.
+// Where one step's blocks live: kb[j] is the R tile of key block j, vtb[j] the T tile of its values.
 template <int NB>
 struct StepDesc {
     const bf16* kb[NB];
     const bf16* vtb[NB];
-    int64_t ks;
     float wratio;        // weight(previous segment) / weight(this segment) on the first step of a segment
 };
 
 template <int NB>
 __device__ __forceinline__ void load_step(KvRegs<NB>& t, const StepDesc<NB>& d, int lane) {
-    const int r = lane & 15, quad = lane >> 4;
 #pragma unroll
     for (int j = 0; j < NB; j++) {
-        const bf16* p = d.kb[j] + r * d.ks + quad * 8;
-        t.k[j][0] = ld16(p);
-        t.k[j][1] = ld16(p + 32);
+        t.k[j][0] = ld16(d.kb[j] + lane * 8);
+        t.k[j][1] = ld16(d.kb[j] + 512 + lane * 8);
     }
 #pragma unroll
     for (int j = 0; j < NB; j++)
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++) t.v[j][dt] = ld8(d.vtb[j] + (dt * 16 + r) * kBlk + quad * 4);
+        for (int dt = 0; dt < 4; dt++) t.v[j][dt] = ld8(d.vtb[j] + dt * 256 + lane * 4);
 }
 
 template <int NB>
@@ -118,9 +114,9 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(llsa_attn_fwd_args a) {
 
     bf16x8 bq[2];
     {
-        const bf16* qp = (const bf16*)a.q + b * a.sqb + h * a.sqh + (int64_t)(g * kBlk + r) * a.sqn + quad * 8;
-        bq[0] = ld16(qp);      // 1/sqrt(64) is a power of two: scaling q before the product (as the
-        bq[1] = ld16(qp + 32); // reference does) equals scaling the fp32 scores, done in the exponent
+        const bf16* qp = (const bf16*)a.qr + ((int64_t)bh * N1 + g) * kTile + lane * 8;
+        bq[0] = ld16(qp);       // 1/sqrt(64) is a power of two: scaling q before the product (as the
+        bq[1] = ld16(qp + 512); // reference does) equals scaling the fp32 scores, done in the exponent
     }
     SoftmaxState st;
     st.m2 = -INFINITY;
@@ -128,12 +124,12 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(llsa_attn_fwd_args a) {
 #pragma unroll
     for (int dt = 0; dt < 4; dt++) st.acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const bf16* kbase = (const bf16*)a.k + b * a.skb + h * a.skh;
-    const bf16* vt = (const bf16*)a.vt + (int64_t)bh * N1 * (kD * kBlk);
-    const bf16* pk = (const bf16*)a.pk + (int64_t)bh * N1 * kD;
-    const bf16* pvt = (const bf16*)a.pvt + (int64_t)bh * N2 * (kD * kBlk);
-    const bf16* pk2 = (a.levels == 2) ? (const bf16*)a.pk2 + (int64_t)bh * N2 * kD : nullptr;
-    const bf16* pv2t = (a.levels == 2) ? (const bf16*)a.pv2t + (int64_t)bh * (N2 / kBlk) * (kD * kBlk) : nullptr;
+    const bf16* kr = (const bf16*)a.kr + (int64_t)bh * N1 * kTile;
+    const bf16* vt = (const bf16*)a.vt + (int64_t)bh * N1 * kTile;
+    const bf16* pk = (const bf16*)a.pkr + (int64_t)bh * N2 * kTile;
+    const bf16* pvt = (const bf16*)a.pvt + (int64_t)bh * N2 * kTile;
+    const bf16* pk2 = (a.levels == 2) ? (const bf16*)a.pk2r + (int64_t)bh * (N2 / kBlk) * kTile : nullptr;
+    const bf16* pv2t = (a.levels == 2) ? (const bf16*)a.pv2t + (int64_t)bh * (N2 / kBlk) * kTile : nullptr;
     __shared__ int ids_lds[4][2][kWave];
     wave_sort_ids(a.idx + ((int64_t)bh * N1 + g) * a.T, a.T, ids_lds[wave][0], ids_lds[wave][1], lane);
     const int* ip = ids_lds[wave][1];
@@ -151,20 +147,18 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(llsa_attn_fwd_args a) {
 #pragma unroll
             for (int j = 0; j < NB; j++) {
                 const int blk = clampi(__builtin_amdgcn_readfirstlane(ip[NB * t + j]), 0, N1 - 1);
-                d.kb[j] = kbase + (int64_t)blk * kBlk * a.skn;
-                d.vtb[j] = vt + (int64_t)blk * (kD * kBlk);
+                d.kb[j] = kr + (int64_t)blk * kTile;
+                d.vtb[j] = vt + (int64_t)blk * kTile;
             }
-            d.ks = a.skn;
             d.wratio = 1.f;
         } else if (t < n_fine + n_mid) {
             const int u = t - n_fine;
 #pragma unroll
             for (int j = 0; j < NB; j++) {
                 const int blk = clampi(pip[NB * u + j], 0, N2 - 1);
-                d.kb[j] = pk + (int64_t)blk * kBlk * kD;
-                d.vtb[j] = pvt + (int64_t)blk * (kD * kBlk);
+                d.kb[j] = pk + (int64_t)blk * kTile;
+                d.vtb[j] = pvt + (int64_t)blk * kTile;
             }
-            d.ks = kD;
             d.wratio = (u == 0) ? 1.f / a.w1 : 1.f;
         } else {
             const int u = t - n_fine - n_mid;
@@ -172,10 +166,9 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(llsa_attn_fwd_args a) {
             const bf16* vv = (a.levels == 2) ? pv2t : pvt;
 #pragma unroll
             for (int j = 0; j < NB; j++) {
-                d.kb[j] = kk + (int64_t)(NB * u + j) * kBlk * kD;
-                d.vtb[j] = vv + (int64_t)(NB * u + j) * (kD * kBlk);
+                d.kb[j] = kk + (int64_t)(NB * u + j) * kTile;
+                d.vtb[j] = vv + (int64_t)(NB * u + j) * kTile;
             }
-            d.ks = kD;
             d.wratio = (u == 0) ? ((a.levels == 2) ? a.w1 / a.w2 : 1.f / a.w1) : 1.f;
         }
     };
@@ -217,23 +210,21 @@ extern "C" int llsa_attn_fwd(const llsa_attn_fwd_args* a, void* stream) {
     LLSA_REQUIRE(a != nullptr, "attn_fwd: null args");
     LLSA_REQUIRE(a->levels == 1 || a->levels == 2, "attn_fwd: levels must be 1 or 2");
     LLSA_REQUIRE(a->B > 0 && a->H > 0 && a->N > 0, "attn_fwd: bad B/H/N");
-    LLSA_REQUIRE(a->q && a->k && a->vt && a->pk && a->pvt && a->idx && a->o && a->lse, "attn_fwd: null tensor");
+    LLSA_REQUIRE(a->qr && a->kr && a->vt && a->pkr && a->pvt && a->idx && a->o && a->lse, "attn_fwd: null tensor");
     LLSA_REQUIRE(a->T >= 4 && a->T % 4 == 0 && a->T <= a->N / 16, "attn_fwd: topk=%d must be a multiple of 4 and <= N/16", a->T);
     LLSA_REQUIRE(a->w1 > 0.f, "attn_fwd: token_weight must be > 0");
     if (a->levels == 1) {
         LLSA_REQUIRE(a->N % 1024 == 0, "attn_fwd: llsa_l1 needs N %% 1024 == 0 (N=%d): the coarse loop runs over 64-token tiles of N/16 pooled tokens", a->N);
     } else {
         LLSA_REQUIRE(a->N % 16384 == 0, "attn_fwd: llsa_l2 needs N %% 16384 == 0 (N=%d): the level-2 loop runs over 64-token tiles of N/256 pooled tokens", a->N);
-        LLSA_REQUIRE(a->pk2 && a->pv2t && a->pidx, "attn_fwd: level-2 tensors missing");
+        LLSA_REQUIRE(a->pk2r && a->pv2t && a->pidx, "attn_fwd: level-2 tensors missing");
         LLSA_REQUIRE(a->T2 >= 4 && a->T2 % 4 == 0 && a->T2 <= a->N / 256, "attn_fwd: topk2=%d must be a multiple of 4 and <= N/256", a->T2);
         LLSA_REQUIRE(a->w2 > 0.f, "attn_fwd: token_weight_2 must be > 0");
     }
-    LLSA_REQUIRE(aligned16(a->q) && aligned16(a->k) && aligned16(a->vt) && aligned16(a->pk) && aligned16(a->pvt) &&
-                     aligned16(a->pk2) && aligned16(a->pv2t) && aligned16(a->o),
+    LLSA_REQUIRE(aligned16(a->qr) && aligned16(a->kr) && aligned16(a->vt) && aligned16(a->pkr) && aligned16(a->pvt) &&
+                     aligned16(a->pk2r) && aligned16(a->pv2t) && aligned16(a->o),
                  "attn_fwd: tensors must be 16-byte aligned");
-    LLSA_REQUIRE(stride_ok(a->sqb) && stride_ok(a->sqh) && stride_ok(a->sqn) && stride_ok(a->skb) && stride_ok(a->skh) &&
-                     stride_ok(a->skn) && (a->sob % 4 == 0) && (a->soh % 4 == 0) && (a->son % 4 == 0),
-                 "attn_fwd: row strides must keep rows 16-byte aligned");
+    LLSA_REQUIRE((a->sob % 4 == 0) && (a->soh % 4 == 0) && (a->son % 4 == 0), "attn_fwd: rows of o must be 8-byte aligned");
     const int N1 = a->N / 16;
     hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_fwd_kernel<LLSA_FWD_NB>), dim3((N1 + 3) / 4, a->B * a->H), dim3(256), 0,
                        (hipStream_t)stream, *a);

@@ -76,6 +76,21 @@ __device__ __forceinline__ float quad_sum(float v) {
     return v;
 }
 
+// Operand tiles.  The attention kernels never read K/V/Q/dO row-major: a 16-row x 64-channel
+// block (1024 bf16 = 2 KB) is stored twice, each time in exactly the order the 64 lanes of a
+// wave consume it as an MFMA operand, so that every operand load is one fully coalesced
+// instruction (lane l reads bytes [16 l, 16 l + 16) or [8 l, 8 l + 8) of a contiguous piece)
+// instead of 64 scattered 16-byte accesses, which would saturate the L1's access rate.
+//   R tile ("rows", contraction over channels):  element (row i, channel c) at
+//        ((c >> 3) * 16 + i) * 8 + (c & 7)
+//     lane l, step s (channels 32 s ..) loads 8 elements at  s * 512 + l * 8
+//   T tile ("tokens", contraction over the 16 rows): element (row t, channel c) at
+//        (((c >> 4) * 4 + (t >> 2)) * 16 + (c & 15)) * 4 + (t & 3)
+//     lane l, channel tile dt (channels 16 dt ..) loads 4 elements at  dt * 256 + l * 4
+constexpr int kTile = kBlk * kD;     // elements per block tile
+__device__ __forceinline__ int r_tile_off(int i, int c) { return ((c >> 3) * 16 + i) * 8 + (c & 7); }
+__device__ __forceinline__ int t_tile_off(int t, int c) { return (((c >> 4) * 4 + (t >> 2)) * 16 + (c & 15)) * 4 + (t & 3); }
+
 // XCD-aware workgroup order.  The 8 XCDs of the chip each have a private L2 and receive
 // workgroups round-robin by linear id (id % 8).  Neighbouring logical work items (query or
 // key blocks that are close in Z-order) read overlapping K/V/Q rows, so they should share an

@@ -43,7 +43,8 @@ __device__ __forceinline__ bf16x8 rope_chunk_bwd(bf16x8 g, bf16x8 f) {
 // pooling pyramid: one workgroup = 256 consecutive tokens (16 blocks of 16) of one (b,h) of
 // one item.  Thread t owns block r = t/8 and the 8-channel chunk c = t%8: it streams the 16
 // rows of its block with 16-byte loads (8 neighbouring lanes cover one 128-byte row), keeps
-// them in registers, and emits everything that derives from them.
+// them in registers, and emits everything that derives from them: the pooled rows and the
+// operand tiles (R and T, see llsa_device.h) the attention kernels read.
 // ---------------------------------------------------------------------------------------
 struct PoolParams {
     llsa_pool_item it[4];
@@ -68,14 +69,15 @@ __global__ __launch_bounds__(128) void pool_pyramid_kernel(PoolParams p) {
         for (int i = 0; i < 16; i++) xv[i] = ld16(x + i * it.sxn);
         if (it.rope) {
             const bf16* f = p.freq + ((int64_t)blk * kBlk) * kD + c * 8;
-            bf16* xr = (bf16*)it.xrot + ((int64_t)bh * it.n + (int64_t)blk * kBlk) * kD + c * 8;
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                xv[i] = rope_chunk_fwd(xv[i], ld16(f + i * kD));
-                st16(xr + i * kD, xv[i]);
+            for (int i = 0; i < 16; i++) xv[i] = rope_chunk_fwd(xv[i], ld16(f + i * kD));
+            if (it.xrot != nullptr) {
+                bf16* xo = (bf16*)it.xrot + ((int64_t)bh * it.n + (int64_t)blk * kBlk) * kD + c * 8;
+#pragma unroll
+                for (int i = 0; i < 16; i++) st16(xo + i * kD, xv[i]);
             }
         }
-        if (it.y1 != nullptr || it.y2 != nullptr || it.y1t != nullptr) {
+        if (it.y1 != nullptr || it.y2 != nullptr || it.y1r != nullptr || it.y1t != nullptr) {
             float acc[8];
 #pragma unroll
             for (int e = 0; e < 8; e++) acc[e] = 0.f;
@@ -87,23 +89,27 @@ __global__ __launch_bounds__(128) void pool_pyramid_kernel(PoolParams p) {
             for (int e = 0; e < 8; e++) y[e] = (bf16)(acc[e] * 0.0625f);
             if (it.y1 != nullptr) st16((bf16*)it.y1 + ((int64_t)bh * n1 + blk) * kD + c * 8, y);
         }
-        if (it.xt != nullptr) {
-            bf16* xt = (bf16*)it.xt + (((int64_t)bh * n1 + blk) * kD + c * 8) * kBlk;
+        if (it.xr != nullptr) {          // R tile: chunk c of row i at (c * 16 + i) * 8
+            bf16* xr = (bf16*)it.xr + ((int64_t)bh * n1 + blk) * kTile + c * 128;
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-                bf16x8 lo, hi;
+            for (int i = 0; i < 16; i++) st16(xr + i * 8, xv[i]);
+        }
+        if (it.xt != nullptr) {          // T tile: channel 8c+e, tokens 4q..4q+3 at t_tile_off(4q, 8c+e)
+            bf16* xt = (bf16*)it.xt + ((int64_t)bh * n1 + blk) * kTile;
 #pragma unroll
-                for (int i = 0; i < 8; i++) {
-                    lo[i] = xv[i][e];
-                    hi[i] = xv[8 + i][e];
+            for (int e = 0; e < 8; e++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    bf16x4 v;
+#pragma unroll
+                    for (int j = 0; j < 4; j++) v[j] = xv[4 * q + j][e];
+                    st8(xt + t_tile_off(4 * q, 8 * c + e), v);
                 }
-                st16(xt + e * kBlk, lo);
-                st16(xt + e * kBlk + 8, hi);
-            }
         }
     }
-    if (it.y2 == nullptr && it.y1t == nullptr) return;      // uniform over the workgroup
+    if (it.y2 == nullptr && it.y1r == nullptr && it.y1t == nullptr) return;      // uniform over the workgroup
 
+    // the 16 pooled rows of this workgroup are one block of the next level
     __shared__ bf16 sm[16][kD];
     st16(&sm[r][c * 8], y);
     __syncthreads();
@@ -122,12 +128,17 @@ __global__ __launch_bounds__(128) void pool_pyramid_kernel(PoolParams p) {
         for (int e = 0; e < 8; e++) y2[e] = (bf16)(acc[e] * 0.0625f);
         st16((bf16*)it.y2 + ((int64_t)bh * n2 + blockIdx.x) * kD + t * 8, y2);
     }
-    if (it.y1t != nullptr) {
-        const int d = t & 63, half = t >> 6;
-        bf16x8 v;
+    if (it.y1r != nullptr)               // thread (r, c) holds chunk c of pooled row r
+        st16((bf16*)it.y1r + ((int64_t)bh * n2 + blockIdx.x) * kTile + (c * 16 + r) * 8, y);
+    if (it.y1t != nullptr) {             // thread -> (channel ch, token half)
+        const int ch = t & 63, half = t >> 6;
 #pragma unroll
-        for (int i = 0; i < 8; i++) v[i] = sm[half * 8 + i][d];
-        st16((bf16*)it.y1t + (((int64_t)bh * n2 + blockIdx.x) * kD + d) * kBlk + half * 8, v);
+        for (int q = 0; q < 2; q++) {
+            bf16x4 v;
+#pragma unroll
+            for (int j = 0; j < 4; j++) v[j] = sm[half * 8 + q * 4 + j][ch];
+            st8((bf16*)it.y1t + ((int64_t)bh * n2 + blockIdx.x) * kTile + t_tile_off(half * 8 + q * 4, ch), v);
+        }
     }
 }
 
@@ -219,10 +230,11 @@ extern "C" int llsa_pool_pyramid_fwd(const llsa_pool_item* items, int n_items, c
         LLSA_REQUIRE(it.x != nullptr && it.n > 0 && it.n % 16 == 0, "pool_pyramid: item %d: n=%d must be a positive multiple of 16", i, it.n);
         LLSA_REQUIRE(aligned16(it.x) && stride_ok(it.sxb) && stride_ok(it.sxh) && stride_ok(it.sxn),
                      "pool_pyramid: item %d: rows must be 16-byte aligned", i);
-        LLSA_REQUIRE((it.y2 == nullptr && it.y1t == nullptr) || it.n % 256 == 0,
+        LLSA_REQUIRE((it.y2 == nullptr && it.y1t == nullptr && it.y1r == nullptr) || it.n % 256 == 0,
                      "pool_pyramid: item %d: level-2 outputs need n %% 256 == 0 (n=%d)", i, it.n);
-        LLSA_REQUIRE(!it.rope || (freq != nullptr && it.xrot != nullptr), "pool_pyramid: item %d: rope needs freq and xrot", i);
-        LLSA_REQUIRE(aligned16(it.y1) && aligned16(it.y2) && aligned16(it.xt) && aligned16(it.y1t) && aligned16(it.xrot),
+        LLSA_REQUIRE(!it.rope || freq != nullptr, "pool_pyramid: item %d: rope needs freq", i);
+        LLSA_REQUIRE(aligned16(it.y1) && aligned16(it.y2) && aligned16(it.xr) && aligned16(it.xt) && aligned16(it.y1r) &&
+                         aligned16(it.y1t) && aligned16(it.xrot),
                      "pool_pyramid: item %d: outputs must be 16-byte aligned", i);
         p.it[i] = it;
         if (it.n > max_n) max_n = it.n;

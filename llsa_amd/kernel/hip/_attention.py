@@ -9,7 +9,6 @@ import torch
 from ..._lib import CHUNK_COARSE, CHUNK_FINE, AttnBwdArgs, AttnFwdArgs
 from ._common import BLOCK, as_rows, lib_for, ptr, require_bf16, require_head_dim, s3, stream_of
 from .indices_transpose import transpose_indices
-from .mean_pool import block_transpose
 
 
 def _check_shapes(q, k, v, pk, pv, pk2, pv2, levels):
@@ -26,10 +25,33 @@ def _check_shapes(q, k, v, pk, pv, pk2, pv2, levels):
         raise ValueError(f"llsa_l{levels} needs a token count that is a multiple of {mult} (got {N})")
 
 
+def _tiles(tiles, need):
+    """tiles: dict name -> tensor or None; need: dict name -> (source tensor, kind).  Computes the
+    missing ones with as few launches as possible and returns the completed dict."""
+    from .mean_pool import operand_tiles
+    tiles = dict(tiles or {})
+    by_src = {}
+    for name, (src, kind) in need.items():
+        if tiles.get(name) is None:
+            by_src.setdefault(id(src), [src, "", []])
+            by_src[id(src)][1] += kind
+            by_src[id(src)][2].append(name)
+    jobs = list(by_src.values())
+    for i in range(0, len(jobs), 4):
+        chunk = jobs[i:i + 4]
+        specs = [(src, "".join(k for k in "rt" if k in kinds)) for src, kinds, _ in chunk]
+        got = iter(operand_tiles(*specs))
+        for (src, kinds, names), (_, kk) in zip(chunk, specs):
+            made = {k: next(got) for k in kk}
+            for name in names:
+                tiles[name] = made[need[name][1]]
+    return tiles
+
+
 def attn_fwd(q, k, v, pk, pv, indices, token_weight, pk2=None, pv2=None, p_indices=None, token_weight_2=1.0,
-             vt=None, pvt=None, pv2t=None):
-    """Forward.  vt / pvt / pv2t are the block-transposed copies of v / pv / pv2; computed here
-    when the caller does not have them.  Returns (o, lse)."""
+             tiles=None):
+    """Forward.  `tiles` may carry operand tiles the caller already has (keys qr, kr, vt, pkr, pvt,
+    pk2r, pv2t); the rest are computed here.  Returns (o, lse)."""
     levels = 1 if pk2 is None else 2
     lib = lib_for(q, k, v, pk, pv, pk2, pv2)
     require_bf16(q, k, v, pk, pv, pk2, pv2)
@@ -37,25 +59,21 @@ def attn_fwd(q, k, v, pk, pv, indices, token_weight, pk2=None, pv2=None, p_indic
     _check_shapes(q, k, v, pk, pv, pk2, pv2, levels)
     B, H, N, D = q.shape
     T = indices.shape[-1]
+    if T > 64:
+        raise ValueError("topk must be <= 64")
     T2 = p_indices.shape[-1] if levels == 2 else 0
-    q, k = as_rows(q), as_rows(k)
-    pk = pk.contiguous()
-    if vt is None or pvt is None or (levels == 2 and pv2t is None):
-        if levels == 2:
-            vt, pvt, pv2t = block_transpose(v, pv, pv2)
-        else:
-            vt, pvt = block_transpose(v, pv)
+    need = dict(qr=(q, "r"), kr=(k, "r"), vt=(v, "t"), pkr=(pk, "r"), pvt=(pv, "t"))
+    if levels == 2:
+        need.update(pk2r=(pk2, "r"), pv2t=(pv2, "t"))
+    tl = _tiles(tiles, need)
     idx = indices.to(torch.int32).contiguous()
     pidx = p_indices.to(torch.int32).contiguous() if levels == 2 else None
-    o = torch.empty_like(q)
+    o = torch.empty_like(q) if rows_ok8(q) else torch.empty(q.shape, device=q.device, dtype=q.dtype)
     lse = torch.empty(B, H, N, device=q.device, dtype=torch.float32)
     a = AttnFwdArgs()
-    a.q, (a.sqb, a.sqh, a.sqn) = q.data_ptr(), s3(q)
-    a.k, (a.skb, a.skh, a.skn) = k.data_ptr(), s3(k)
-    a.vt, a.pk, a.pvt = vt.data_ptr(), pk.data_ptr(), pvt.data_ptr()
+    a.qr, a.kr, a.vt, a.pkr, a.pvt = (tl[n].data_ptr() for n in ("qr", "kr", "vt", "pkr", "pvt"))
     if levels == 2:
-        pk2 = pk2.contiguous()
-        a.pk2, a.pv2t, a.pidx = pk2.data_ptr(), pv2t.data_ptr(), pidx.data_ptr()
+        a.pk2r, a.pv2t, a.pidx = tl["pk2r"].data_ptr(), tl["pv2t"].data_ptr(), pidx.data_ptr()
     a.idx = idx.data_ptr()
     a.o, (a.sob, a.soh, a.son) = o.data_ptr(), s3(o)
     a.lse = lse.data_ptr()
@@ -65,13 +83,19 @@ def attn_fwd(q, k, v, pk, pv, indices, token_weight, pk2=None, pv2=None, p_indic
     return o, lse
 
 
+def rows_ok8(t):
+    """Rows start 8-byte aligned with unit channel stride (what the 8-byte output stores need)."""
+    return t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(s % 4 == 0 for s in t.stride()[:-1])
+
+
 def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_weight, pk2=None, pv2=None,
-             p_indices=None, token_weight_2=1.0, qt=None, kt=None, pkt=None, pk2t=None,
-             freq_dq: Optional[torch.Tensor] = None, stages: int = 0, csr=None):
+             p_indices=None, token_weight_2=1.0, tiles=None, freq_dq: Optional[torch.Tensor] = None, stages: int = 0,
+             csr=None):
     """Backward.  Returns (dq, dk, dv, dpk, dpv[, dpk2, dpv2]) with the reference's conventions:
     every gradient is `empty_like` of its primal; the pooled gradients are NOT yet folded
-    into dk / dv (autograd, or pool_bwd_accum, does that).  `stages` (a mask of the LLSA_BWD_*
-    bits of include/llsa_hip.h) launches only some of the kernels, for profiling."""
+    into dk / dv (autograd, or pool_bwd_accum, does that).  `tiles` may carry operand tiles the
+    caller already has (qr, qt, kr, kt, vr, pkr, pkt, pvr, pk2r, pk2t, pv2r).  `stages` (a mask of
+    the LLSA_BWD_* bits of include/llsa_hip.h) launches only some of the kernels, for profiling."""
     levels = 1 if pk2 is None else 2
     lib = lib_for(do, q, k, v, pk, pv, pk2, pv2, o, lse)
     require_bf16(do, q, k, v, pk, pv, pk2, pv2, o)
@@ -80,20 +104,12 @@ def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_wei
     B, H, N, D = q.shape
     T = indices.shape[-1]
     T2 = p_indices.shape[-1] if levels == 2 else 0
-    do, q, k, v, o = as_rows(do), as_rows(q), as_rows(k), as_rows(v), as_rows(o)
-    pk, pv = pk.contiguous(), pv.contiguous()
+    do, o = as_rows(do), as_rows(o)
+    need = dict(qr=(q, "r"), qt=(q, "t"), kr=(k, "r"), kt=(k, "t"), vr=(v, "r"), pkr=(pk, "r"), pkt=(pk, "t"),
+                pvr=(pv, "r"))
     if levels == 2:
-        pk2, pv2 = pk2.contiguous(), pv2.contiguous()
-    need = [t for t, have in ((q, qt), (k, kt), (pk, pkt)) if have is None]
-    if levels == 2 and pk2t is None:
-        need.append(pk2)
-    if need:
-        got = iter(block_transpose(*need))
-        qt = qt if qt is not None else next(got)
-        kt = kt if kt is not None else next(got)
-        pkt = pkt if pkt is not None else next(got)
-        if levels == 2 and pk2t is None:
-            pk2t = next(got)
+        need.update(pk2r=(pk2, "r"), pk2t=(pk2, "t"), pv2r=(pv2, "r"))
+    tl = _tiles(tiles, need)
     idx = indices.to(torch.int32).contiguous()
     if levels == 2:
         pidx = p_indices.to(torch.int32).contiguous()
@@ -105,19 +121,18 @@ def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_wei
         off, flat, work = transpose_indices(idx, N // BLOCK, CHUNK_FINE)
         if levels == 2:
             poff, pflat, pwork = transpose_indices(pidx, N // (BLOCK * BLOCK), CHUNK_COARSE)
-    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    dpk, dpv = torch.empty_like(pk), torch.empty_like(pv)
+    mk = lambda t: torch.empty_like(t) if rows_ok8(t) else torch.empty(t.shape, device=t.device, dtype=t.dtype)
+    dq, dk, dv = mk(q), mk(k), mk(v)
+    dpk, dpv = torch.empty_like(pk, memory_format=torch.contiguous_format), torch.empty_like(pv, memory_format=torch.contiguous_format)
     ws_bytes = lib.attn_bwd_workspace_bytes(B, H, N, T, T2, levels)
     ws = torch.empty(ws_bytes, device=q.device, dtype=torch.uint8)
     a = AttnBwdArgs()
     a.dout, (a.sdob, a.sdoh, a.sdon) = do.data_ptr(), s3(do)
-    a.q, (a.sqb, a.sqh, a.sqn) = q.data_ptr(), s3(q)
-    a.k, (a.skb, a.skh, a.skn) = k.data_ptr(), s3(k)
-    a.v, (a.svb, a.svh, a.svn) = v.data_ptr(), s3(v)
     a.o, (a.sob, a.soh, a.son) = o.data_ptr(), s3(o)
     lse = lse.contiguous()
-    a.lse, a.pk, a.pv = lse.data_ptr(), pk.data_ptr(), pv.data_ptr()
-    a.qt, a.kt, a.pkt = qt.data_ptr(), kt.data_ptr(), pkt.data_ptr()
+    a.lse = lse.data_ptr()
+    for n in ("qr", "qt", "kr", "kt", "vr", "pkr", "pkt", "pvr"):
+        setattr(a, n, tl[n].data_ptr())
     a.idx, a.off, a.flat, a.work = idx.data_ptr(), off.data_ptr(), flat.data_ptr(), work.data_ptr()
     a.dq, (a.sdqb, a.sdqh, a.sdqn) = dq.data_ptr(), s3(dq)
     a.dk, (a.sdkb, a.sdkh, a.sdkn) = dk.data_ptr(), s3(dk)
@@ -125,8 +140,10 @@ def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_wei
     a.dpk, a.dpv = dpk.data_ptr(), dpv.data_ptr()
     outs = [dq, dk, dv, dpk, dpv]
     if levels == 2:
-        dpk2, dpv2 = torch.empty_like(pk2), torch.empty_like(pv2)
-        a.pk2, a.pv2, a.pk2t = pk2.data_ptr(), pv2.data_ptr(), pk2t.data_ptr()
+        dpk2 = torch.empty_like(pk2, memory_format=torch.contiguous_format)
+        dpv2 = torch.empty_like(pv2, memory_format=torch.contiguous_format)
+        for n in ("pk2r", "pk2t", "pv2r"):
+            setattr(a, n, tl[n].data_ptr())
         a.pidx, a.poff, a.pflat, a.pwork = pidx.data_ptr(), poff.data_ptr(), pflat.data_ptr(), pwork.data_ptr()
         a.dpk2, a.dpv2 = dpk2.data_ptr(), dpv2.data_ptr()
         outs += [dpk2, dpv2]

@@ -81,16 +81,19 @@ def mean_pool1d(x: torch.Tensor, k: int, format='bhsc'):
 
 
 class PoolSpec:
-    """What to produce from one (B,H,n,64) bf16 tensor in a pool_pyramid launch."""
+    """What to produce from one (B,H,n,64) bf16 tensor in a pool_pyramid launch: y1 / y2 pooled
+    rows, xr / xt operand tiles of the (rotated) tensor, y1r / y1t operand tiles of y1, xrot a
+    row-major rotated copy."""
 
-    def __init__(self, x, y1=False, y2=False, xt=False, y1t=False, rope=False):
-        self.x, self.y1, self.y2, self.xt, self.y1t, self.rope = x, y1, y2, xt, y1t, rope
+    def __init__(self, x, y1=False, y2=False, xr=False, xt=False, y1r=False, y1t=False, rope=False, xrot=False):
+        self.x, self.y1, self.y2, self.xr, self.xt, self.y1r, self.y1t = x, y1, y2, xr, xt, y1r, y1t
+        self.rope, self.xrot = rope, xrot
 
 
 def pool_pyramid(specs: Sequence[PoolSpec], freq: Optional[torch.Tensor] = None):
     """One launch of llsa_pool_pyramid_fwd.  Returns, per spec, a dict with the requested
-    outputs: y1 (B,H,n/16,64), y2 (B,H,n/256,64), xt (B,H,n/16,64,16), y1t (B,H,n/256,64,16),
-    xrot (B,H,n,64)."""
+    outputs: y1 (B,H,n/16,64), y2 (B,H,n/256,64), xr / xt (B,H,n/16,1024), y1r / y1t
+    (B,H,n/256,1024), xrot (B,H,n,64).  The tile layouts are described in include/llsa_hip.h."""
     assert 1 <= len(specs) <= 4
     x0 = specs[0].x
     lib = lib_for(*[s.x for s in specs], freq)
@@ -106,7 +109,7 @@ def pool_pyramid(specs: Sequence[PoolSpec], freq: Optional[torch.Tensor] = None)
         n = x.shape[2]
         if n % BLOCK != 0:
             raise ValueError(f"token count {n} is not a multiple of {BLOCK}")
-        if (s.y2 or s.y1t) and n % (BLOCK * BLOCK) != 0:
+        if (s.y2 or s.y1t or s.y1r) and n % (BLOCK * BLOCK) != 0:
             raise ValueError(f"token count {n} is not a multiple of {BLOCK * BLOCK}")
         e = lambda *shape: torch.empty(shape, device=x.device, dtype=x.dtype)
         o = {}
@@ -114,17 +117,21 @@ def pool_pyramid(specs: Sequence[PoolSpec], freq: Optional[torch.Tensor] = None)
             o["y1"] = e(B, H, n // 16, 64)
         if s.y2:
             o["y2"] = e(B, H, n // 256, 64)
+        if s.xr:
+            o["xr"] = e(B, H, n // 16, 1024)
         if s.xt:
-            o["xt"] = e(B, H, n // 16, 64, 16)
+            o["xt"] = e(B, H, n // 16, 1024)
+        if s.y1r:
+            o["y1r"] = e(B, H, n // 256, 1024)
         if s.y1t:
-            o["y1t"] = e(B, H, n // 256, 64, 16)
-        if s.rope:
-            if freq is None:
-                raise ValueError("rope requested without a table")
+            o["y1t"] = e(B, H, n // 256, 1024)
+        if s.rope and freq is None:
+            raise ValueError("rope requested without a table")
+        if s.xrot:
             o["xrot"] = e(B, H, n, 64)
         outs.append(o)
         items.append(PoolItem(x.data_ptr(), x.stride(0), x.stride(1), x.stride(2), n, 1 if s.rope else 0,
-                              *(o[k].data_ptr() if k in o else None for k in ("y1", "y2", "xt", "y1t", "xrot"))))
+                              *(o[k].data_ptr() if k in o else None for k in ("y1", "y2", "xr", "xt", "y1r", "y1t", "xrot"))))
     if freq is not None:
         require_bf16(freq)
         freq = freq.contiguous()
@@ -135,10 +142,17 @@ def pool_pyramid(specs: Sequence[PoolSpec], freq: Optional[torch.Tensor] = None)
     return outs
 
 
-def block_transpose(*tensors):
-    """(B,H,n,64) -> (B,H,n/16,64,16) for up to 4 tensors in one launch."""
-    outs = pool_pyramid([PoolSpec(t, xt=True) for t in tensors])
-    return [o["xt"] for o in outs]
+def operand_tiles(*specs):
+    """specs: (tensor, 'r' | 't' | 'rt').  Up to 4 tensors in one launch; returns a flat list of the
+    requested tile tensors in order (R before T for 'rt')."""
+    outs = pool_pyramid([PoolSpec(t, xr='r' in k, xt='t' in k) for t, k in specs])
+    res = []
+    for o, (_, k) in zip(outs, specs):
+        if 'r' in k:
+            res.append(o["xr"])
+        if 't' in k:
+            res.append(o["xt"])
+    return res
 
 
 def pool_bwd_accum(dx, dy1, dy2=None, freq=None, out=None):

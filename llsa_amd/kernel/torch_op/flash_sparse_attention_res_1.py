@@ -42,38 +42,39 @@ flash_sparse_residual_attention_l1_op = FlashSparseResidualAttentionL1.apply
 
 
 class _LlsaL1Fused(Function):
-    """llsa_l1 as one autograd node: pooling pyramid (+RoPE, + the block-transposed copies the
-    kernels read) in one pass, selection, attention; the backward folds the pooled gradients
-    into dk / dv (what mean_pool's backward and autograd's accumulation do in the reference)
-    and rotates dq / dk back."""
+    """llsa_l1 as one autograd node: pooling pyramid (+RoPE, + the operand tiles the kernels
+    read) in one pass, selection, attention; the backward folds the pooled gradients into
+    dk / dv (what mean_pool's backward and autograd's accumulation do in the reference) and
+    rotates dq / dk back."""
 
     @staticmethod
     def forward(ctx, q, k, v, topk, block_size, freq):
         if block_size != 16:
             raise NotImplementedError("block_size must be 16")
-        need_grad = any(ctx.needs_input_grad[:3])
+        g = any(ctx.needs_input_grad[:3])
         rope = freq is not None
-        oq, ok, ov = pool_pyramid([PoolSpec(q, y1=True, xt=need_grad, rope=rope),
-                                   PoolSpec(k, y1=True, xt=need_grad, y1t=need_grad, rope=rope),
-                                   PoolSpec(v, y1=True, xt=True, y1t=True)], freq)
-        if rope:
-            q, k = oq["xrot"], ok["xrot"]
+        oq, ok, ov = pool_pyramid([PoolSpec(q, y1=True, xr=True, xt=g, rope=rope),
+                                   PoolSpec(k, y1=True, xr=True, xt=g, y1r=True, y1t=g, rope=rope),
+                                   PoolSpec(v, y1=True, xr=g, xt=True, y1r=g, y1t=True)], freq)
         pq, pk, pv = oq["y1"], ok["y1"], ov["y1"]
         indices = gen_sparse_indices(pq, pk, topk)
-        o, m = sparse_indices_attn_res_fwd(q, k, v, pk, pv, indices, indices.shape[-1], block_size, 4,
-                                           vt=ov["xt"], pvt=ov["y1t"])
-        if need_grad:
-            ctx.save_for_backward(q, k, v, pk, pv, o, m, indices, oq["xt"], ok["xt"], ok["y1t"], freq)
+        tiles = dict(qr=oq["xr"], kr=ok["xr"], vt=ov["xt"], pkr=ok["y1r"], pvt=ov["y1t"])
+        # q / k are only shape-and-stride templates below: the kernels read the (rotated) tiles
+        o, m = sparse_indices_attn_res_fwd(q, k, v, pk, pv, indices, indices.shape[-1], block_size, 4, tiles=tiles)
+        if g:
+            ctx.save_for_backward(q, k, v, pk, pv, o, m, indices, freq, oq["xr"], oq["xt"], ok["xr"], ok["xt"], ov["xr"],
+                                  ok["y1r"], ok["y1t"], ov["y1r"])
         ctx.block_size = block_size
         ctx.indices = indices
         return o
 
     @staticmethod
     def backward(ctx, do):
-        q, k, v, pk, pv, o, m, indices, qt, kt, pkt, freq = ctx.saved_tensors
+        q, k, v, pk, pv, o, m, indices, freq, qr, qt, kr, kt, vr, pkr, pkt, pvr = ctx.saved_tensors
         bs = ctx.block_size
+        tiles = dict(qr=qr, qt=qt, kr=kr, kt=kt, vr=vr, pkr=pkr, pkt=pkt, pvr=pvr)
         dq, dk, dv, _, dpk, dpv = sparse_indices_attn_res_scatter_bwd_v2(
-            do, q, k, v, pk, pv, o, m, indices, indices.shape[-1], bs, bs, qt=qt, kt=kt, pkt=pkt, freq_dq=freq)
+            do, q, k, v, pk, pv, o, m, indices, indices.shape[-1], bs, bs, tiles=tiles, freq_dq=freq)
         dk = pool_bwd_accum(dk, dpk, None, freq, out=dk)
         dv = pool_bwd_accum(dv, dpv, None, None, out=dv)
         return dq, dk, dv, None, None, None

@@ -48,12 +48,24 @@ def randn_inputs(B, H, N, D, dev, seed=0, strided=False):
 
 
 # ------------------------------------------------------------------------------------------
+def _r_tiles(x):
+    """(B,H,n,64) -> (B,H,n/16,1024) R tiles: element (row t, channel c) at ((c>>3)*16 + t)*8 + (c&7)."""
+    B, H, n, _ = x.shape
+    return x.reshape(B, H, n // 16, 16, 8, 8).permute(0, 1, 2, 4, 3, 5).reshape(B, H, n // 16, 1024)
+
+
+def _t_tiles(x):
+    """T tiles: element (row t, channel c) at (((c>>4)*4 + (t>>2))*16 + (c&15))*4 + (t&3)."""
+    B, H, n, _ = x.shape
+    return x.reshape(B, H, n // 16, 4, 4, 4, 16).permute(0, 1, 2, 5, 3, 6, 4).reshape(B, H, n // 16, 1024)
+
+
 def check_pool_pyramid(dev, B=1, H=2, N=512, strided=True, rope=True):
     from llsa_amd.kernel.hip.mean_pool import PoolSpec, pool_pyramid
     x, *_ = randn_inputs(B, H, N, 64, dev, seed=5, strided=strided)
     x = x * 2
     freq = torch.randn(N, 64, generator=torch.Generator().manual_seed(6)).bfloat16().to(dev) if rope else None
-    out, = pool_pyramid([PoolSpec(x, y1=True, y2=True, xt=True, y1t=True, rope=rope)], freq)
+    out, = pool_pyramid([PoolSpec(x, y1=True, y2=True, xr=True, xt=True, y1r=True, y1t=True, rope=rope, xrot=rope)], freq)
     xc = x.cpu()
     xr = O.rope_apply(xc, freq.cpu()) if rope else xc
     p1 = O.mean_pool(xr)
@@ -62,8 +74,10 @@ def check_pool_pyramid(dev, B=1, H=2, N=512, strided=True, rope=True):
         assert torch.equal(out["xrot"].cpu(), xr), "rotated copy differs"
     assert torch.equal(out["y1"].cpu(), p1), "level-1 pool differs"
     assert torch.equal(out["y2"].cpu(), p2), "level-2 pool differs"
-    assert torch.equal(out["xt"].cpu(), xr.reshape(B, H, N // 16, 16, 64).transpose(-1, -2)), "xt differs"
-    assert torch.equal(out["y1t"].cpu(), p1.reshape(B, H, N // 256, 16, 64).transpose(-1, -2)), "y1t differs"
+    assert torch.equal(out["xr"].cpu(), _r_tiles(xr)), "R tiles differ"
+    assert torch.equal(out["xt"].cpu(), _t_tiles(xr)), "T tiles differ"
+    assert torch.equal(out["y1r"].cpu(), _r_tiles(p1)), "R tiles of the pooled level differ"
+    assert torch.equal(out["y1t"].cpu(), _t_tiles(p1)), "T tiles of the pooled level differ"
 
 
 def check_mean_pool1d(dev, dtype=torch.bfloat16, K=16, C=64, S=128, fmt='bhsc'):
