@@ -1,10 +1,10 @@
 // Block selection: dense coarsest-level top-k and parent-guided fine top-k.
 //
-// Both kernels score one tile of 16 pooled queries against 16-key tiles with the bf16
-// MFMA, park the scores of the 16 rows in LDS and then let each wave pull the T best
-// entries out of "its" rows by repeated wave-wide arg-max.  The order is total --
-// higher score first, equal scores by smaller key index -- so the result does not
-// depend on how the work is split.
+// The kernels score one tile of 16 pooled queries against 16-key tiles with the bf16 MFMA,
+// park the scores of the 16 rows in LDS and then let each wave select the T best entries of
+// "its" rows: by radix selection when a row fits in LDS, by repeated wave-wide arg-max over
+// chunks otherwise.  The order is total -- higher score first, equal scores by smaller key
+// index -- so the result does not depend on how the work is split.
 #include "llsa_device.h"
 #include "llsa_host.h"
 #include "../../include/llsa_hip.h"
@@ -113,13 +113,151 @@ __global__ __launch_bounds__(256) void topk_dense_kernel(const bf16* __restrict_
     for (int i = tid; i < 16 * T; i += 256) out[((int64_t)bh * n + q0 + i / T) * T + i % T] = win_idx[i / T][i % T];
 }
 
+// ---------------------------------------------------------------------------------------
+// Radix selection.  Scores are mapped to unsigned integers that sort like the floats; the
+// T-th largest is found one bit at a time from the top with a wave-wide count per bit
+// (a compare, a ballot and a scalar popcount per entry, no cross-lane data movement), then
+// everything above it -- plus as many entries equal to it as are still needed, smallest
+// index first -- is compacted and put in final order by rank counting among the T winners.
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ unsigned ordered_bits(float f) {
+    if (f != f) return 0u;                                    // NaN sorts below everything
+    const unsigned b = __float_as_uint(f);
+    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+
+// u[0..npos): ordered scores of one row (LDS); gidx_of(pos): global index of a position.
+// Each lane keeps its E entries (positions lane, lane + 64, ...) in registers, so a bit step is
+// E compares + ballots + scalar popcounts with no memory access.
+// sel_u / sel_i: 64 entries of LDS scratch each.  out[0..T): result, global memory.
+template <int E, typename IdxFn>
+__device__ __forceinline__ void wave_topk_radix(const unsigned* u, int npos, int T, IdxFn gidx_of, unsigned* sel_u,
+                                                int* sel_i, int* out, int lane) {
+    unsigned uk[E];
+    unsigned gk[E];
+    bool ok[E];
+#pragma unroll
+    for (int e = 0; e < E; e++) {
+        const int pos = lane + e * kWave;
+        ok[e] = pos < npos;
+        uk[e] = ok[e] ? u[pos] : 0u;
+        gk[e] = ok[e] ? (unsigned)gidx_of(pos) : 0xFFFFFFFFu;
+    }
+    unsigned prefix = 0;
+    int remaining = T;
+    for (int bit = 31; bit >= 0; bit--) {
+        const unsigned msk = (bit == 31) ? 0x80000000u : ((0xFFFFFFFFu << (bit + 1)) | (1u << bit));
+        const unsigned want = prefix | (1u << bit);
+        int cnt1 = 0;
+#pragma unroll
+        for (int e = 0; e < E; e++) cnt1 += __popcll(__ballot(ok[e] && (uk[e] & msk) == want));
+        if (cnt1 >= remaining)
+            prefix = want;
+        else
+            remaining -= cnt1;
+    }
+    const unsigned tau = prefix;                              // the T-th largest score
+    int n_eq = 0;
+#pragma unroll
+    for (int e = 0; e < E; e++) n_eq += __popcll(__ballot(ok[e] && uk[e] == tau));
+    unsigned idx_thr = 0xFFFFFFFFu;
+    if (n_eq > remaining) {                                   // ties at the threshold: keep the smallest indices
+        unsigned p2 = 0;
+        int rem2 = remaining;
+        for (int bit = 30; bit >= 0; bit--) {
+            const unsigned msk = (0xFFFFFFFFu << (bit + 1)) | (1u << bit);
+            int cnt0 = 0;
+#pragma unroll
+            for (int e = 0; e < E; e++) cnt0 += __popcll(__ballot(ok[e] && uk[e] == tau && (gk[e] & msk) == p2));
+            if (cnt0 < rem2) {
+                rem2 -= cnt0;
+                p2 |= (1u << bit);
+            }
+        }
+        idx_thr = p2;
+    }
+    if (lane < T) {
+        sel_u[lane] = 0u;
+        sel_i[lane] = kNoIdx;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    int base_slot = 0;
+#pragma unroll
+    for (int e = 0; e < E; e++) {
+        const bool sel = ok[e] && (uk[e] > tau || (uk[e] == tau && gk[e] <= idx_thr));
+        const unsigned long long m = __ballot(sel);
+        const int slot = base_slot + __popcll(m & ((1ull << lane) - 1ull));
+        if (sel && slot < T) {
+            sel_u[slot] = uk[e];
+            sel_i[slot] = (int)gk[e];
+        }
+        base_slot += __popcll(m);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    if (lane < T) {
+        const unsigned mu = sel_u[lane];
+        const int mi = sel_i[lane];
+        int rank = 0;
+        for (int j = 0; j < T; j++) {
+            const unsigned ou = sel_u[j];
+            const int oi = sel_i[j];
+            rank += (ou > mu || (ou == mu && (oi < mi || (oi == mi && j < lane)))) ? 1 : 0;
+        }
+        out[rank] = mi;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
+// entries per lane as a compile-time bound: 1, 2, 4, 8 or 16
+template <typename IdxFn>
+__device__ __forceinline__ void wave_topk_radix_any(const unsigned* u, int npos, int T, IdxFn gidx_of, unsigned* sel_u,
+                                                    int* sel_i, int* out, int lane) {
+    if (npos <= 64) wave_topk_radix<1>(u, npos, T, gidx_of, sel_u, sel_i, out, lane);
+    else if (npos <= 128) wave_topk_radix<2>(u, npos, T, gidx_of, sel_u, sel_i, out, lane);
+    else if (npos <= 256) wave_topk_radix<4>(u, npos, T, gidx_of, sel_u, sel_i, out, lane);
+    else if (npos <= 512) wave_topk_radix<8>(u, npos, T, gidx_of, sel_u, sel_i, out, lane);
+    else wave_topk_radix<16>(u, npos, T, gidx_of, sel_u, sel_i, out, lane);
+}
+
+constexpr int kRadixMaxN = 1024;      // keys per row the radix kernels keep in LDS
+
+// dense selection for n <= kRadixMaxN: 16 query rows per workgroup, all n keys scored into LDS
+__global__ __launch_bounds__(256) void topk_dense_radix_kernel(const bf16* __restrict__ pq, const bf16* __restrict__ pk,
+                                                               int* __restrict__ out, int n, int T, int round_scores) {
+    HIP_DYNAMIC_SHARED(unsigned, su)                          // [16][n + 1]
+    __shared__ unsigned sel_u[4][kWave];
+    __shared__ int sel_i[4][kWave];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int bh = blockIdx.y, q0 = blockIdx.x * 16;
+    const int stride = n + 1;
+    const bf16* pqb = pq + ((int64_t)bh * n + q0) * kD;
+    const bf16* pkb = pk + (int64_t)bh * n * kD;
+    bf16x8 bq[2];
+    bq[0] = ld16(pqb + (lane & 15) * kD + (lane >> 4) * 8);
+    bq[1] = ld16(pqb + (lane & 15) * kD + (lane >> 4) * 8 + 32);
+    for (int tile = wave; tile < n / 16; tile += 4) {
+        f32x4 s = score_tile(pkb + (int64_t)tile * 16 * kD, bq);
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+            su[(lane & 15) * stride + tile * 16 + 4 * (lane >> 4) + e] = ordered_bits(round_scores ? rn_bf16(s[e]) : s[e]);
+    }
+    __syncthreads();
+    for (int row = wave; row < 16; row += 4)
+        wave_topk_radix_any(
+            su + row * stride, n, T, [](int pos) { return pos; }, sel_u[wave], sel_i[wave],
+            out + ((int64_t)bh * n + q0 + row) * T, lane);
+}
+
 __global__ __launch_bounds__(256) void topk_sparse_kernel(const bf16* __restrict__ pq, const bf16* __restrict__ pk,
                                                           const int* __restrict__ pidx, int* __restrict__ out, int N1,
                                                           int T, int T2) {
-    __shared__ float sc[16][kMaxCand + 1];
+    __shared__ unsigned su[16][kMaxCand + 1];
     __shared__ int cand[kMaxCand];
-    __shared__ float win_val[16][kMaxT];
-    __shared__ int win_idx[16][kMaxT];
+    __shared__ unsigned sel_u[4][kWave];
+    __shared__ int sel_i[4][kWave];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int bh = blockIdx.y, G = blockIdx.x;
@@ -137,15 +275,13 @@ __global__ __launch_bounds__(256) void topk_sparse_kernel(const bf16* __restrict
     for (int a = wave; a < T2; a += 4) {
         f32x4 s = score_tile(pkb + (int64_t)cand[a * kBlk] * kD, bq);
 #pragma unroll
-        for (int e = 0; e < 4; e++) sc[lane & 15][a * kBlk + 4 * (lane >> 4) + e] = s[e];
+        for (int e = 0; e < 4; e++) su[lane & 15][a * kBlk + 4 * (lane >> 4) + e] = ordered_bits(s[e]);
     }
     __syncthreads();
     for (int row = wave; row < 16; row += 4)
-        wave_topk_row(
-            sc[row], C, T, [&](int pos) { return cand[pos]; }, win_val[row], win_idx[row]);
-    __syncthreads();
-    for (int i = tid; i < 16 * T; i += 256)
-        out[((int64_t)bh * N1 + G * kBlk + i / T) * T + i % T] = win_idx[i / T][i % T];
+        wave_topk_radix_any(
+            su[row], C, T, [&](int pos) { return cand[pos]; }, sel_u[wave], sel_i[wave],
+            out + ((int64_t)bh * N1 + G * kBlk + row) * T, lane);
 }
 
 }  // namespace llsa
@@ -158,8 +294,17 @@ extern "C" int llsa_topk_dense(const void* pq, const void* pk, int32_t* out_idx,
     LLSA_REQUIRE(B > 0 && H > 0 && n > 0 && n % 16 == 0, "topk_dense: n=%d must be a positive multiple of 16", n);
     LLSA_REQUIRE(T >= 1 && T <= kMaxT && T <= n, "topk_dense: need 1 <= T <= min(%d, n=%d), got %d", kMaxT, n, T);
     LLSA_REQUIRE(aligned16(pq) && aligned16(pk), "topk_dense: inputs must be 16-byte aligned");
-    hipLaunchKernelGGL(topk_dense_kernel, dim3(n / 16, B * H), dim3(256), 0, (hipStream_t)stream, (const bf16*)pq,
-                       (const bf16*)pk, out_idx, n, T, round_scores);
+    if (n <= kRadixMaxN) {
+        const int lds = (int)sizeof(unsigned) * 16 * (n + 1);
+        if (lds > 60 * 1024) {
+            hipError_t e = hipFuncSetAttribute((const void*)topk_dense_radix_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+            if (e != hipSuccess) return fail(-101, "topk_dense: cannot raise dynamic LDS to %d bytes: %s", lds, hipGetErrorString(e));
+        }
+        hipLaunchKernelGGL(topk_dense_radix_kernel, dim3(n / 16, B * H), dim3(256), sizeof(unsigned) * 16 * (n + 1),
+                           (hipStream_t)stream, (const bf16*)pq, (const bf16*)pk, out_idx, n, T, round_scores);
+    } else
+        hipLaunchKernelGGL(topk_dense_kernel, dim3(n / 16, B * H), dim3(256), 0, (hipStream_t)stream, (const bf16*)pq,
+                           (const bf16*)pk, out_idx, n, T, round_scores);
     return launch_status("topk_dense");
 }
 

@@ -31,10 +31,8 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
                                                                       int* __restrict__ flat, int* __restrict__ work,
                                                                       int Mb, int Kb, int T, int chunk, int work_stride) {
     HIP_DYNAMIC_SHARED(int, smem)
-    const int words = (Mb + 31) / 32;
     int* pos = smem;                               // Kb
     int* wave_tot = smem + Kb;                     // 3 * kTrWaves (+ padding to 64)
-    unsigned* bitmaps = (unsigned*)(smem + Kb + 64);   // kTrWaves * words
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int bh = blockIdx.x;
@@ -99,36 +97,44 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
         const int slot = atomicAdd(&pos[clampi(idx[e], 0, Kb - 1)], 1);
         flat[slot] = e / T;
     }
-    __syncthreads();                                // pos[n] is now the END of segment n
+    // pos[n] is now the END of segment n; the segments are sorted by sort_segments_kernel
+}
 
+// Puts every segment of `flat` in ascending order: one wave per key block sets one bit per
+// entry in a private LDS bitmap over the query blocks and reads the bits back in order.
+__global__ __launch_bounds__(256) void sort_segments_kernel(const int* __restrict__ offsets, int* __restrict__ flat, int Mb,
+                                                            int Kb, int T) {
+    HIP_DYNAMIC_SHARED(unsigned, bitmaps)                     // 4 waves x words
+    const int words = (Mb + 31) / 32;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int bh = blockIdx.y, n = blockIdx.x * 4 + wave;
+    if (n >= Kb) return;                                      // no workgroup barrier below
+    flat += (int64_t)bh * Mb * T;
+    const int* o = offsets + (int64_t)bh * (Kb + 1) + n;
+    const int s = o[0], e = o[1];
+    if (e - s <= 1) return;
     unsigned* bm = bitmaps + wave * words;
-    for (int n = wave; n < Kb; n += kTrWaves) {
-        const int s = (n == 0) ? 0 : pos[n - 1], e = pos[n];
-        if (e - s <= 1) continue;
-        for (int w = lane; w < words; w += kWave) bm[w] = 0u;
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        for (int i = s + lane; i < e; i += kWave) {
-            const int q = flat[i];
-            atomicOr(&bm[q >> 5], 1u << (q & 31));
+    for (int w = lane; w < words; w += kWave) bm[w] = 0u;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    for (int i = s + lane; i < e; i += kWave) {
+        const int q = clampi(flat[i], 0, Mb - 1);
+        atomicOr(&bm[q >> 5], 1u << (q & 31));
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    int out = s;
+    for (int wb = 0; wb < words; wb += kWave) {
+        unsigned wd = (wb + lane < words) ? bm[wb + lane] : 0u;
+        const int cnt = __popc(wd);
+        const int incl2 = wave_incl_scan(cnt, lane);
+        int oo = out + incl2 - cnt;
+        while (wd) {
+            const int bit = __ffs((int)wd) - 1;
+            flat[oo++] = (wb + lane) * 32 + bit;
+            wd &= wd - 1;
         }
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        int out = s;
-        for (int wb = 0; wb < words; wb += kWave) {
-            unsigned wd = (wb + lane < words) ? bm[wb + lane] : 0u;
-            const int cnt = __popc(wd);
-            const int incl2 = wave_incl_scan(cnt, lane);
-            int o = out + incl2 - cnt;
-            while (wd) {
-                const int bit = __ffs((int)wd) - 1;
-                flat[o++] = (wb + lane) * 32 + bit;
-                wd &= wd - 1;
-            }
-            out += __shfl(incl2, kWave - 1);
-        }
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-        __builtin_amdgcn_wave_barrier();
+        out += __shfl(incl2, kWave - 1);
     }
 }
 
@@ -148,15 +154,18 @@ extern "C" int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int3
     LLSA_REQUIRE(work == nullptr || (chunk >= 1 && Kb < 32768 && (int64_t)Mb * T / chunk + 1 < 65536),
                  "transpose_indices: work list needs chunk >= 1, Kb < 32768 and fewer than 65536 chunks per key block");
     if (chunk < 1) chunk = 1;
-    const int words = (Mb + 31) / 32;
-    const size_t lds = sizeof(int) * ((size_t)Kb + 64 + (size_t)kTrWaves * words);
+    const size_t lds = sizeof(int) * ((size_t)Kb + 64);
     static_assert(3 * kTrWaves <= 64, "wave totals must fit their LDS slot");
-    LLSA_REQUIRE(lds <= 160 * 1024, "transpose_indices: Kb=%d, Mb=%d need %zu bytes of LDS (limit 163840)", Kb, Mb, lds);
+    LLSA_REQUIRE(lds <= 160 * 1024, "transpose_indices: Kb=%d needs %zu bytes of LDS (limit 163840)", Kb, lds);
+    const size_t lds_sort = sizeof(unsigned) * 4 * ((size_t)(Mb + 31) / 32);
+    LLSA_REQUIRE(lds_sort <= 64 * 1024, "transpose_indices: Mb=%d needs %zu bytes of LDS for the segment sort", Mb, lds_sort);
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute((const void*)transpose_indices_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return fail(-101, "transpose_indices: cannot raise dynamic LDS to %zu bytes: %s", lds, hipGetErrorString(e));
     }
     hipLaunchKernelGGL(transpose_indices_kernel, dim3(B * H), dim3(kTrThreads), lds, (hipStream_t)stream, idx, offsets, flat, work, Mb, Kb, T, chunk,
                        (int)llsa_work_list_len(Mb, Kb, T, chunk));
+    hipLaunchKernelGGL(sort_segments_kernel, dim3((Kb + 3) / 4, B * H), dim3(256), lds_sort, (hipStream_t)stream,
+                       (const int*)offsets, flat, Mb, Kb, T);
     return launch_status("transpose_indices");
 }

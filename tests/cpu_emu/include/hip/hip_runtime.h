@@ -120,6 +120,8 @@ inline T atomicMax(T* p, T v) { T o = *p; *p = o > v ? o : v; return o; }
 template <typename T>
 inline T atomicExch(T* p, T v) { T o = *p; *p = v; return o; }
 inline void __threadfence() {}
+inline unsigned __float_as_uint(float f) { unsigned u; memcpy(&u, &f, 4); return u; }
+inline float __uint_as_float(unsigned u) { float f; memcpy(&f, &u, 4); return f; }
 inline float __expf(float x) { return expf(x); }
 inline float __logf(float x) { return logf(x); }
 template <typename T> inline T min(T a, T b) { return a < b ? a : b; }
