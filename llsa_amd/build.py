@@ -24,6 +24,7 @@ ARCH = "gfx950"
 FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",     # no packed-fp32 VALU ops
+    "-mllvm", "-amdgpu-mfma-vgpr-form",      # MFMA results straight into VGPRs: no v_accvgpr copies around the soft-max
     "-Wall", "-Wno-unused-function", "-Wno-unknown-attributes",
 ]
 

@@ -143,13 +143,11 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, cons
     const bf16* pkt = (const bf16*)a.pkt + (int64_t)bh * N2 * kTile;
     const bf16 *kb[2], *vb[2], *ktb[2];
 
-    __shared__ int ids_lds[4][2][kWave];
-    wave_sort_ids(a.idx + ((int64_t)bh * N1 + g) * a.T, a.T, ids_lds[wave][0], ids_lds[wave][1], lane);
-    const int* ip = ids_lds[wave][1];
+    const int* ip = a.idx + ((int64_t)bh * N1 + g) * a.T;
     for (int t = 0; t < a.T / 2; t++) {
 #pragma unroll
         for (int j = 0; j < 2; j++) {
-            const int blk = clampi(__builtin_amdgcn_readfirstlane(ip[2 * t + j]), 0, N1 - 1);
+            const int blk = clampi(ip[2 * t + j], 0, N1 - 1);
             kb[j] = kr + (int64_t)blk * kTile;
             vb[j] = vr + (int64_t)blk * kTile;
             ktb[j] = kt + (int64_t)blk * kTile;
@@ -318,7 +316,7 @@ __global__ __launch_bounds__(256) void attn_kside_kernel(KSideParams p) {
         const int* work = p.work + (int64_t)bh * p.work_stride;
         const int item = (MODE == MODE_FINE) ? bx * 4 + wave : bx;
         if (item >= work[0]) return;                          // uniform over the item's waves
-        const int it = work[2 + p.n_units + item];
+        const int it = work[4 + p.n_units + item];
         const int ci = it & 0xffff;
         unit = it >> 16;
         const int chunk = (MODE == MODE_FINE) ? LLSA_CHUNK_FINE : LLSA_CHUNK_COARSE;
@@ -326,7 +324,7 @@ __global__ __launch_bounds__(256) void attn_kside_kernel(KSideParams p) {
         start = o[0] + ci * chunk;
         cnt = min(chunk, o[1] - start);
         if (MODE == MODE_SPARSE1) cnt *= kBlk;                // every parent stands for its 16 children
-        const int sb = work[2 + unit];
+        const int sb = work[4 + unit];
         if (sb >= 0) slot = (int64_t)bh * p.slot_stride + sb + ci;
         fl = p.flat + (int64_t)bh * p.flat_stride;
     }
@@ -409,41 +407,62 @@ __global__ __launch_bounds__(256) void attn_kside_kernel(KSideParams p) {
     }
 }
 
-// Finishes the units the K-side kernel did not write itself: a unit whose list was cut into
-// several chunks is the sum of its partial slots (added in chunk order, so the result does not
-// depend on scheduling); a unit nobody selected gets zeros.  One wave per unit.
-// DENSE mode: every unit has `n_chunks` partials at stride `chunk_stride` slots.
-__global__ __launch_bounds__(64) void kside_reduce_kernel(const f32x4* __restrict__ part, const int* __restrict__ off,
-                                                          const int* __restrict__ work, bf16* dk, int64_t sdkb, int64_t sdkh,
-                                                          int64_t sdkn, bf16* dv, int64_t sdvb, int64_t sdvh, int64_t sdvn,
-                                                          int H, int n_units, int chunk, int64_t work_stride,
-                                                          int64_t slot_stride, int n_chunks, int64_t chunk_stride) {
-    const int lane = threadIdx.x, unit = blockIdx.x, bh = blockIdx.y, b = bh / H, h = bh % H;
+// Finishes the units whose list was cut into several pieces: the result is the sum of the
+// unit's partial slots, added in chunk order, so it does not depend on scheduling.  One launch
+// serves the three K-side passes; one wave per unit.
+struct ReduceJob {
+    const f32x4* part;
+    const int* off;          // CSR offsets (sparse jobs) or nullptr (dense job)
+    const int* work;         // work list (sparse jobs)
+    bf16* dk; int64_t sdkb, sdkh, sdkn;
+    bf16* dv; int64_t sdvb, sdvh, sdvn;
+    int n_units, chunk, max_units;       // max_units: upper bound of units this job can have per (b,h)
+    int64_t work_stride, slot_stride;
+    int n_chunks;            // dense job: partials per unit, at stride BH * n_units slots
+};
+struct ReduceParams {
+    ReduceJob job[3];
+    int n_jobs, H;
+};
+
+__global__ __launch_bounds__(256) void kside_reduce_kernel(ReduceParams rp) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int bh = blockIdx.y, b = bh / rp.H, h = bh % rp.H;
     const int r = lane & 15, quad = lane >> 4;
+    int u = blockIdx.x * 4 + wave, j = 0;
+    while (j < rp.n_jobs && u >= rp.job[j].max_units) {
+        u -= rp.job[j].max_units;
+        j++;
+    }
+    if (j >= rp.n_jobs) return;
+    const ReduceJob& jb = rp.job[j];
+    int unit, n;
     int64_t first, stride;
-    int n;
-    if (work != nullptr) {
-        const int* o = off + (int64_t)bh * (n_units + 1) + unit;
-        const int len = o[1] - o[0];
-        n = (len + chunk - 1) / chunk;
-        if (n == 1) return;                                   // written by the K-side kernel
-        first = (int64_t)bh * slot_stride + work[(int64_t)bh * work_stride + 2 + unit];
+    if (jb.work != nullptr) {
+        const int* work = jb.work + (int64_t)bh * jb.work_stride;
+        if (u >= work[2]) return;
+        const int max_items = (int)(jb.work_stride - 4 - jb.n_units - jb.max_units);
+        unit = work[4 + jb.n_units + max_items + u];
+        const int* o = jb.off + (int64_t)bh * (jb.n_units + 1) + unit;
+        n = (o[1] - o[0] + jb.chunk - 1) / jb.chunk;
+        first = (int64_t)bh * jb.slot_stride + work[4 + unit];
         stride = 1;
     } else {
-        n = n_chunks;
-        first = (int64_t)bh * n_units + unit;
-        stride = chunk_stride;
+        unit = u;
+        n = jb.n_chunks;
+        first = (int64_t)bh * jb.n_units + unit;
+        stride = (int64_t)gridDim.y * jb.n_units;
     }
     f32x4 acc[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
     for (int c = 0; c < n; c++) {
-        const f32x4* ps = part + (first + c * stride) * (8 * kWave);
+        const f32x4* ps = jb.part + (first + c * stride) * (8 * kWave);
 #pragma unroll
         for (int i = 0; i < 8; i++) acc[i] += ps[i * kWave + lane];
     }
-    bf16* kp = dk + b * sdkb + h * sdkh + (int64_t)(unit * kBlk + r) * sdkn + quad * 4;
-    bf16* vp = dv + b * sdvb + h * sdvh + (int64_t)(unit * kBlk + r) * sdvn + quad * 4;
+    bf16* kp = jb.dk + b * jb.sdkb + h * jb.sdkh + (int64_t)(unit * kBlk + r) * jb.sdkn + quad * 4;
+    bf16* vp = jb.dv + b * jb.sdvb + h * jb.sdvh + (int64_t)(unit * kBlk + r) * jb.sdvn + quad * 4;
 #pragma unroll
     for (int dt = 0; dt < 4; dt++) {
         st8(kp + dt * 16, cvt4(acc[dt] * kScale));
@@ -550,6 +569,9 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     if (stages & LLSA_BWD_DQ)
         hipLaunchKernelGGL(attn_dq_kernel, dim3((N1 + 3) / 4, BH), dim3(256), 0, s, *a, (const float*)delta, (const bf16*)dor);
 
+    ReduceParams rp;
+    rp.n_jobs = 0;
+    rp.H = H;
     KSideParams p;
     p.qr = (const bf16*)a->qr; p.dor = dor;
     p.qt = (const bf16*)a->qt; p.dot = dot; p.lse = a->lse; p.delta = delta;
@@ -566,9 +588,12 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     if (stages & LLSA_BWD_DKV) {
         const int max_items = N1 * a->T / LLSA_CHUNK_FINE + N1;
         hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_FINE>), dim3((max_items + 3) / 4, BH), dim3(256), 0, s, p);
-        hipLaunchKernelGGL(kside_reduce_kernel, dim3(N1, BH), dim3(64), 0, s, (const f32x4*)p.part, p.off, p.work, p.dk, p.sdkb,
-                           p.sdkh, p.sdkn, p.dv, p.sdvb, p.sdvh, p.sdvn, H, N1, LLSA_CHUNK_FINE, p.work_stride, p.slot_stride,
-                           0, (int64_t)0);
+        ReduceJob& j = rp.job[rp.n_jobs++];
+        j.part = p.part; j.off = p.off; j.work = p.work;
+        j.dk = p.dk; j.sdkb = p.sdkb; j.sdkh = p.sdkh; j.sdkn = p.sdkn;
+        j.dv = p.dv; j.sdvb = p.sdvb; j.sdvh = p.sdvh; j.sdvn = p.sdvn;
+        j.n_units = N1; j.chunk = LLSA_CHUNK_FINE; j.max_units = N1 * a->T / LLSA_CHUNK_FINE + 1;
+        j.work_stride = p.work_stride; j.slot_stride = p.slot_stride; j.n_chunks = 0;
     }
 
     const int64_t s1b = (int64_t)H * N1 * 64, s1h = (int64_t)N1 * 64;
@@ -584,13 +609,16 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
         p.n_units = N2; p.w = a->cgw1;
         const int max_items = N2 * a->T2 / LLSA_CHUNK_COARSE + N2;
         hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_SPARSE1>), dim3(max_items, BH), dim3(256), 0, s, p);
-        hipLaunchKernelGGL(kside_reduce_kernel, dim3(N2, BH), dim3(64), 0, s, (const f32x4*)p.part, p.off, p.work, p.dk, p.sdkb,
-                           p.sdkh, p.sdkn, p.dv, p.sdvb, p.sdvh, p.sdvn, H, N2, LLSA_CHUNK_COARSE, p.work_stride,
-                           p.slot_stride, 0, (int64_t)0);
+        ReduceJob& j = rp.job[rp.n_jobs++];
+        j.part = p.part; j.off = p.off; j.work = p.work;
+        j.dk = p.dk; j.sdkb = p.sdkb; j.sdkh = p.sdkh; j.sdkn = p.sdkn;
+        j.dv = p.dv; j.sdvb = p.sdvb; j.sdvh = p.sdvh; j.sdvn = p.sdvn;
+        j.n_units = N2; j.chunk = LLSA_CHUNK_COARSE; j.max_units = N2 * a->T2 / LLSA_CHUNK_COARSE + 1;
+        j.work_stride = p.work_stride; j.slot_stride = p.slot_stride; j.n_chunks = 0;
     }
     // dense coarsest level: every unit (16 pooled tokens) meets every query block; the query
     // range is cut into d.chunks pieces whose partial sums are added afterwards
-    if (!(stages & LLSA_BWD_DENSE)) return launch_status("attn_bwd");
+    if (stages & LLSA_BWD_DENSE) {
     if (a->levels == 2) {
         p.kk = (const bf16*)a->pk2r; p.vv = (const bf16*)a->pv2r;
         p.dk = (bf16*)a->dpk2; p.dv = (bf16*)a->dpv2;
@@ -607,8 +635,16 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     p.part = (f32x4*)(ws + wsp.part_dense);
     p.n_units = d.n_tok / 16; p.chunk_len = d.chunk_len;
     hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_DENSE>), dim3(p.n_units, BH, d.chunks), dim3(256), 0, s, p);
-    hipLaunchKernelGGL(kside_reduce_kernel, dim3(p.n_units, BH), dim3(64), 0, s, (const f32x4*)p.part, (const int*)nullptr,
-                       (const int*)nullptr, p.dk, p.sdkb, p.sdkh, p.sdkn, p.dv, p.sdvb, p.sdvh, p.sdvn, H, p.n_units, 1,
-                       (int64_t)0, (int64_t)0, d.chunks, (int64_t)BH * p.n_units);
+    ReduceJob& j = rp.job[rp.n_jobs++];
+    j.part = p.part; j.off = nullptr; j.work = nullptr;
+    j.dk = p.dk; j.sdkb = p.sdkb; j.sdkh = p.sdkh; j.sdkn = p.sdkn;
+    j.dv = p.dv; j.sdvb = p.sdvb; j.sdvh = p.sdvh; j.sdvn = p.sdvn;
+    j.n_units = p.n_units; j.chunk = 1; j.max_units = p.n_units; j.work_stride = 0; j.slot_stride = 0; j.n_chunks = d.chunks;
+    }
+    if (rp.n_jobs > 0) {
+        int total = 0;
+        for (int i = 0; i < rp.n_jobs; i++) total += rp.job[i].max_units;
+        hipLaunchKernelGGL(kside_reduce_kernel, dim3((total + 3) / 4, BH), dim3(256), 0, s, rp);
+    }
     return launch_status("attn_bwd");
 }

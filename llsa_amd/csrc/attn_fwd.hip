@@ -130,9 +130,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(llsa_attn_fwd_args a) {
     const bf16* pvt = (const bf16*)a.pvt + (int64_t)bh * N2 * kTile;
     const bf16* pk2 = (a.levels == 2) ? (const bf16*)a.pk2r + (int64_t)bh * (N2 / kBlk) * kTile : nullptr;
     const bf16* pv2t = (a.levels == 2) ? (const bf16*)a.pv2t + (int64_t)bh * (N2 / kBlk) * kTile : nullptr;
-    __shared__ int ids_lds[4][2][kWave];
-    wave_sort_ids(a.idx + ((int64_t)bh * N1 + g) * a.T, a.T, ids_lds[wave][0], ids_lds[wave][1], lane);
-    const int* ip = ids_lds[wave][1];
+    const int* ip = a.idx + ((int64_t)bh * N1 + g) * a.T;
     const int* pip = (a.levels == 2) ? a.pidx + ((int64_t)bh * N2 + g / kBlk) * a.T2 : nullptr;
 
     // step t of the KV list: fine blocks, then (l2) the parent's level-1 pooled blocks, then
@@ -146,7 +144,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(llsa_attn_fwd_args a) {
         if (t < n_fine) {
 #pragma unroll
             for (int j = 0; j < NB; j++) {
-                const int blk = clampi(__builtin_amdgcn_readfirstlane(ip[NB * t + j]), 0, N1 - 1);
+                const int blk = clampi(ip[NB * t + j], 0, N1 - 1);
                 d.kb[j] = kr + (int64_t)blk * kTile;
                 d.vtb[j] = vt + (int64_t)blk * kTile;
             }

@@ -105,31 +105,6 @@ __device__ __forceinline__ int xcd_logical_id() {
     return xcd * q + (xcd < rem ? xcd : rem) + slot;
 }
 
-// Sorts the T (<= 64) block ids at src ascending into `out` (LDS, 64 ints; `tmp` is another 64
-// ints of LDS scratch), one wave, no workgroup barrier.  Attention is invariant to the order of
-// the selected blocks; walking them in ascending order makes sibling waves, whose selections
-// overlap heavily on spatially coherent inputs, touch the same K/V rows at about the same time,
-// so that they hit in the CU's L1 instead of going to L2 again.
-__device__ __forceinline__ void wave_sort_ids(const int* src, int T, int* tmp, int* out, int lane) {
-    int v = 0;
-    if (lane < T) {
-        v = src[lane];
-        tmp[lane] = v;
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    if (lane < T) {
-        int rank = 0;
-        for (int j = 0; j < T; j++) {
-            const int o = tmp[j];
-            rank += (o < v || (o == v && j < lane)) ? 1 : 0;
-        }
-        out[rank] = v;
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-}
-
 __device__ __forceinline__ int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
 
 }  // namespace llsa

@@ -24,15 +24,19 @@ __device__ __forceinline__ int wave_incl_scan(int v, int lane) {
 
 // Work list (optional): the K-side kernels walk each key block's segment in chunks of at most
 // `chunk` entries so that a popular key block does not serialise on one wave.  Per (b,h):
-//   work[0] = number of items, work[1] = number of partial-sum slots,
-//   work[2 + n] = first slot of key block n, or -1 when n has at most one chunk,
-//   work[2 + Kb + i] = item i = (n << 16) | chunk index   (items of one key block are adjacent)
+//   work[0] = number of items, work[1] = number of partial-sum slots, work[2] = number of key
+//   blocks with more than one chunk, work[3] unused,
+//   work[4 + n] = first slot of key block n, or -1 when n has one chunk,
+//   work[4 + Kb + i] = item i = (n << 16) | chunk index   (items of one key block are adjacent),
+//   work[4 + Kb + max_items + j] = j-th key block with more than one chunk
+// Every key block has at least one item (an unselected block's item has no entries and only
+// writes zeros), and max_items = Mb*T/chunk + Kb.
 __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int* __restrict__ idx, int* __restrict__ offsets,
                                                                       int* __restrict__ flat, int* __restrict__ work,
                                                                       int Mb, int Kb, int T, int chunk, int work_stride) {
     HIP_DYNAMIC_SHARED(int, smem)
     int* pos = smem;                               // Kb
-    int* wave_tot = smem + Kb;                     // 3 * kTrWaves (+ padding to 64)
+    int* wave_tot = smem + Kb;                     // 4 * kTrWaves
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int bh = blockIdx.x;
@@ -49,39 +53,45 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
     // exclusive scan over pos[0..Kb): each thread owns `per` consecutive counters
     const int per = (Kb + kTrThreads - 1) / kTrThreads;
     const int c0 = min(tid * per, Kb), c1 = min(c0 + per, Kb);
-    int local = 0, l_items = 0, l_slots = 0;
+    int local = 0, l_items = 0, l_slots = 0, l_multi = 0;
     for (int i = c0; i < c1; i++) {
         const int c = pos[i];
-        const int nch = (c + chunk - 1) / chunk;
+        const int nch = max(1, (c + chunk - 1) / chunk);
         local += c;
         l_items += nch;
         l_slots += (nch > 1) ? nch : 0;
+        l_multi += (nch > 1) ? 1 : 0;
     }
     const int incl = wave_incl_scan(local, lane);
     const int incl_i = wave_incl_scan(l_items, lane);
     const int incl_s = wave_incl_scan(l_slots, lane);
+    const int incl_m = wave_incl_scan(l_multi, lane);
     if (lane == kWave - 1) {
         wave_tot[wave] = incl;
         wave_tot[kTrWaves + wave] = incl_i;
         wave_tot[2 * kTrWaves + wave] = incl_s;
+        wave_tot[3 * kTrWaves + wave] = incl_m;
     }
     __syncthreads();
-    int run = incl - local, run_i = incl_i - l_items, run_s = incl_s - l_slots;
+    int run = incl - local, run_i = incl_i - l_items, run_s = incl_s - l_slots, run_m = incl_m - l_multi;
     for (int w = 0; w < wave; w++) {
         run += wave_tot[w];
         run_i += wave_tot[kTrWaves + w];
         run_s += wave_tot[2 * kTrWaves + w];
+        run_m += wave_tot[3 * kTrWaves + w];
     }
     if (work != nullptr) work += (int64_t)bh * work_stride;
+    const int max_items = E / chunk + Kb;
     for (int i = c0; i < c1; i++) {
         const int c = pos[i];
         offsets[i] = run;
         pos[i] = run;
         run += c;
         if (work != nullptr) {
-            const int nch = (c + chunk - 1) / chunk;
-            work[2 + i] = (nch > 1) ? run_s : -1;
-            for (int ci = 0; ci < nch; ci++) work[2 + Kb + run_i + ci] = (i << 16) | ci;
+            const int nch = max(1, (c + chunk - 1) / chunk);
+            work[4 + i] = (nch > 1) ? run_s : -1;
+            for (int ci = 0; ci < nch; ci++) work[4 + Kb + run_i + ci] = (i << 16) | ci;
+            if (nch > 1) work[4 + Kb + max_items + run_m++] = i;
             run_i += nch;
             run_s += (nch > 1) ? nch : 0;
         }
@@ -90,6 +100,8 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
     if (work != nullptr && tid == kTrThreads - 1) {
         work[0] = run_i;
         work[1] = run_s;
+        work[2] = run_m;
+        work[3] = 0;
     }
     __syncthreads();
 
@@ -144,7 +156,8 @@ using namespace llsa;
 
 extern "C" int64_t llsa_work_list_len(int Mb, int Kb, int T, int chunk) {
     if (Mb <= 0 || Kb <= 0 || T <= 0 || chunk <= 0) return -1;
-    return 2 + (int64_t)Kb + ((int64_t)Mb * T / chunk + Kb);
+    const int64_t e = (int64_t)Mb * T;
+    return 4 + (int64_t)Kb + (e / chunk + Kb) + (e / chunk + 1);
 }
 
 extern "C" int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, int32_t* work, int B, int H, int Mb,
@@ -155,7 +168,7 @@ extern "C" int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int3
                  "transpose_indices: work list needs chunk >= 1, Kb < 32768 and fewer than 65536 chunks per key block");
     if (chunk < 1) chunk = 1;
     const size_t lds = sizeof(int) * ((size_t)Kb + 64);
-    static_assert(3 * kTrWaves <= 64, "wave totals must fit their LDS slot");
+    static_assert(4 * kTrWaves <= 64, "wave totals must fit their LDS slot");
     LLSA_REQUIRE(lds <= 160 * 1024, "transpose_indices: Kb=%d needs %zu bytes of LDS (limit 163840)", Kb, lds);
     const size_t lds_sort = sizeof(unsigned) * 4 * ((size_t)(Mb + 31) / 32);
     LLSA_REQUIRE(lds_sort <= 64 * 1024, "transpose_indices: Mb=%d needs %zu bytes of LDS for the segment sort", Mb, lds_sort);

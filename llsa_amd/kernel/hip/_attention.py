@@ -59,8 +59,6 @@ def attn_fwd(q, k, v, pk, pv, indices, token_weight, pk2=None, pv2=None, p_indic
     _check_shapes(q, k, v, pk, pv, pk2, pv2, levels)
     B, H, N, D = q.shape
     T = indices.shape[-1]
-    if T > 64:
-        raise ValueError("topk must be <= 64")
     T2 = p_indices.shape[-1] if levels == 2 else 0
     need = dict(qr=(q, "r"), kr=(k, "r"), vt=(v, "t"), pkr=(pk, "r"), pvt=(pv, "t"))
     if levels == 2:
