@@ -456,10 +456,21 @@ __global__ __launch_bounds__(256) void kside_reduce_kernel(ReduceParams rp) {
     f32x4 acc[8];
 #pragma unroll
     for (int i = 0; i < 8; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-    for (int c = 0; c < n; c++) {
-        const f32x4* ps = jb.part + (first + c * stride) * (8 * kWave);
+    for (int c0 = 0; c0 < n; c0 += 4) {                       // four partials in flight, added in chunk order
+        f32x4 v[4][8];
 #pragma unroll
-        for (int i = 0; i < 8; i++) acc[i] += ps[i * kWave + lane];
+        for (int k = 0; k < 4; k++) {
+            const int c = min(c0 + k, n - 1);
+            const f32x4* ps = jb.part + (first + c * stride) * (8 * kWave);
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[k][i] = ps[i * kWave + lane];
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++)
+            if (c0 + k < n) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) acc[i] += v[k][i];
+            }
     }
     bf16* kp = jb.dk + b * jb.sdkb + h * jb.sdkh + (int64_t)(unit * kBlk + r) * jb.sdkn + quad * 4;
     bf16* vp = jb.dv + b * jb.sdvb + h * jb.sdvh + (int64_t)(unit * kBlk + r) * jb.sdvn + quad * 4;
