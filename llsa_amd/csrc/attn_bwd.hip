@@ -409,7 +409,7 @@ __global__ __launch_bounds__(256) void attn_kside_kernel(KSideParams p) {
 
 // Finishes the units whose list was cut into several pieces: the result is the sum of the
 // unit's partial slots, added in chunk order, so it does not depend on scheduling.  One launch
-// serves the three K-side passes; one wave per unit.
+// serves the three K-side passes.
 struct ReduceJob {
     const f32x4* part;
     const int* off;          // CSR offsets (sparse jobs) or nullptr (dense job)
@@ -426,10 +426,13 @@ struct ReduceParams {
 };
 
 __global__ __launch_bounds__(256) void kside_reduce_kernel(ReduceParams rp) {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // two workgroups per unit; every thread owns one f32x4 of the unit's 8 x 64 accumulator
+    // registers and streams that position of all partials, eight loads in flight
     const int bh = blockIdx.y, b = bh / rp.H, h = bh % rp.H;
+    const int pos = (blockIdx.x & 1) * 256 + threadIdx.x;
+    const int reg = pos >> 6, lane = pos & 63;
     const int r = lane & 15, quad = lane >> 4;
-    int u = blockIdx.x * 4 + wave, j = 0;
+    int u = blockIdx.x >> 1, j = 0;
     while (j < rp.n_jobs && u >= rp.job[j].max_units) {
         u -= rp.job[j].max_units;
         j++;
@@ -453,31 +456,23 @@ __global__ __launch_bounds__(256) void kside_reduce_kernel(ReduceParams rp) {
         first = (int64_t)bh * jb.n_units + unit;
         stride = (int64_t)gridDim.y * jb.n_units;
     }
-    f32x4 acc[8];
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    const f32x4* ps = jb.part + first * (8 * kWave) + reg * kWave + lane;
+    for (int c0 = 0; c0 < n; c0 += 8) {
+        f32x4 v[8];
 #pragma unroll
-    for (int i = 0; i < 8; i++) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-    for (int c0 = 0; c0 < n; c0 += 4) {                       // four partials in flight, added in chunk order
-        f32x4 v[4][8];
+        for (int k = 0; k < 8; k++) v[k] = ps[(int64_t)min(c0 + k, n - 1) * stride * (8 * kWave)];
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            const int c = min(c0 + k, n - 1);
-            const f32x4* ps = jb.part + (first + c * stride) * (8 * kWave);
-#pragma unroll
-            for (int i = 0; i < 8; i++) v[k][i] = ps[i * kWave + lane];
-        }
-#pragma unroll
-        for (int k = 0; k < 4; k++)
-            if (c0 + k < n) {
-#pragma unroll
-                for (int i = 0; i < 8; i++) acc[i] += v[k][i];
-            }
+        for (int k = 0; k < 8; k++)
+            if (c0 + k < n) acc += v[k];                       // chunk order: the sum does not depend on scheduling
     }
-    bf16* kp = jb.dk + b * jb.sdkb + h * jb.sdkh + (int64_t)(unit * kBlk + r) * jb.sdkn + quad * 4;
-    bf16* vp = jb.dv + b * jb.sdvb + h * jb.sdvh + (int64_t)(unit * kBlk + r) * jb.sdvn + quad * 4;
-#pragma unroll
-    for (int dt = 0; dt < 4; dt++) {
-        st8(kp + dt * 16, cvt4(acc[dt] * kScale));
-        st8(vp + dt * 16, cvt4(acc[4 + dt]));
+    const int dt = reg & 3;
+    if (reg < 4) {
+        bf16* kp = jb.dk + b * jb.sdkb + h * jb.sdkh + (int64_t)(unit * kBlk + r) * jb.sdkn + quad * 4;
+        st8(kp + dt * 16, cvt4(acc * kScale));
+    } else {
+        bf16* vp = jb.dv + b * jb.sdvb + h * jb.sdvh + (int64_t)(unit * kBlk + r) * jb.sdvn + quad * 4;
+        st8(vp + dt * 16, cvt4(acc));
     }
 }
 
@@ -655,7 +650,7 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     if (rp.n_jobs > 0) {
         int total = 0;
         for (int i = 0; i < rp.n_jobs; i++) total += rp.job[i].max_units;
-        hipLaunchKernelGGL(kside_reduce_kernel, dim3((total + 3) / 4, BH), dim3(256), 0, s, rp);
+        hipLaunchKernelGGL(kside_reduce_kernel, dim3(total * 2, BH), dim3(256), 0, s, rp);
     }
     return launch_status("attn_bwd");
 }
