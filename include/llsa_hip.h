@@ -27,7 +27,10 @@
  *        offset = ((c >> 3) * 16 + t) * 8 + (c & 7)
  *   T tile (products that contract over the block's 16 tokens: P.V, dS.K, P^T.dO, dS^T.Q)
  *        offset = (((c >> 4) * 4 + (t >> 2)) * 16 + (c & 15)) * 4 + (t & 3)
- * Tiled tensors are (B,H,n/16,1024) contiguous.  llsa_pool_pyramid_fwd writes them.
+ * Tiled tensors are (B,H,n/16,1024) contiguous.  llsa_pool_pyramid_fwd writes them.  Only the
+ * forward's P.V product reads T tiles from memory (of v and the pooled v); the backward
+ * kernels fetch R tiles only and produce the token-major orientation on chip with the
+ * transposing LDS read of gfx950.
  */
 #ifndef LLSA_HIP_H
 #define LLSA_HIP_H
@@ -162,13 +165,9 @@ typedef struct llsa_attn_bwd_args {
     const void* dout; int64_t sdob, sdoh, sdon;  /* (B,H,N,64) upstream gradient                 */
     const void* o;    int64_t sob, soh, son;     /* (B,H,N,64) forward output                     */
     const float* lse;                            /* (B,H,N)                                       */
-    const void* qr;  const void* qt;             /* R and T tiles of q   (B,H,N/16,1024)          */
-    const void* kr;  const void* kt;             /* R and T tiles of k                            */
-    const void* vr;                              /* R tiles of v                                  */
-    const void* pkr; const void* pkt;            /* R and T tiles of pk  (B,H,N/256,1024)         */
-    const void* pvr;                             /* R tiles of pv                                 */
-    const void* pk2r; const void* pk2t;          /* R and T tiles of pk2 (B,H,N/4096,1024)        */
-    const void* pv2r;                            /* R tiles of pv2                                */
+    const void* qr;  const void* kr;  const void* vr;   /* R tiles of q, k, v  (B,H,N/16,1024)    */
+    const void* pkr; const void* pvr;            /* R tiles of pk, pv   (B,H,N/256,1024)          */
+    const void* pk2r; const void* pv2r;          /* R tiles of pk2, pv2 (B,H,N/4096,1024)         */
     const int32_t* idx;  const int32_t* pidx;
     const int32_t* off;  const int32_t* flat;  const int32_t* work;    /* transposed idx  (Kb = N/16)     */
     const int32_t* poff; const int32_t* pflat; const int32_t* pwork;   /* transposed pidx (Kb = N/256)    */

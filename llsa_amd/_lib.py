@@ -41,9 +41,8 @@ class AttnBwdArgs(C.Structure):
     _fields_ = (
         [("dout", c_void_p), ("sdob", c_int64), ("sdoh", c_int64), ("sdon", c_int64)]
         + _t3("o")
-        + [("lse", c_void_p), ("qr", c_void_p), ("qt", c_void_p), ("kr", c_void_p), ("kt", c_void_p), ("vr", c_void_p),
-           ("pkr", c_void_p), ("pkt", c_void_p), ("pvr", c_void_p), ("pk2r", c_void_p), ("pk2t", c_void_p),
-           ("pv2r", c_void_p),
+        + [("lse", c_void_p), ("qr", c_void_p), ("kr", c_void_p), ("vr", c_void_p),
+           ("pkr", c_void_p), ("pvr", c_void_p), ("pk2r", c_void_p), ("pv2r", c_void_p),
            ("idx", c_void_p), ("pidx", c_void_p), ("off", c_void_p), ("flat", c_void_p), ("work", c_void_p),
            ("poff", c_void_p), ("pflat", c_void_p), ("pwork", c_void_p)]
         + [("dq", c_void_p), ("sdqb", c_int64), ("sdqh", c_int64), ("sdqn", c_int64),

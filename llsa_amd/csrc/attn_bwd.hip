@@ -19,11 +19,11 @@
 namespace llsa {
 
 // ---------------------------------------------------------------------------------------
-// delta = rowsum(O * dO) in fp32, and the R and T operand tiles of dO.
+// delta = rowsum(O * dO) in fp32, and the R operand tiles of dO.
 // Same thread mapping as the pooling kernel: 16 blocks x 8 channel chunks per workgroup.
 // ---------------------------------------------------------------------------------------
 __global__ __launch_bounds__(128) void bwd_pre_kernel(llsa_attn_bwd_args a, float* __restrict__ delta,
-                                                      bf16* __restrict__ dor, bf16* __restrict__ dot) {
+                                                      bf16* __restrict__ dor) {
     const int N1 = a.N / kBlk;
     const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
     const int t = threadIdx.x, c = t & 7, r = t >> 3;
@@ -58,27 +58,18 @@ __global__ __launch_bounds__(128) void bwd_pre_kernel(llsa_attn_bwd_args a, floa
     bf16* xr = dor + ((int64_t)bh * N1 + blk) * kTile + c * 128;
 #pragma unroll
     for (int i = 0; i < 16; i++) st16(xr + i * 8, gv[i]);
-    bf16* xt = dot + ((int64_t)bh * N1 + blk) * kTile;
-#pragma unroll
-    for (int e = 0; e < 8; e++)
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-            bf16x4 v;
-#pragma unroll
-            for (int j = 0; j < 4; j++) v[j] = gv[4 * q + j][e];
-            st8(xt + t_tile_off(4 * q, 8 * c + e), v);
-        }
 }
 
 // ---------------------------------------------------------------------------------------
 // dQ: one wave per query block, key blocks taken two at a time (32 keys = one MFMA K step)
 // ---------------------------------------------------------------------------------------
-// kb / vb / ktb: R tile of K, R tile of V, T tile of K for the two key blocks of the pair
+// kb / vb: R tiles of K and V for the two key blocks of the pair.  K is the A operand of S^T from
+// the registers and, parked in the wave's LDS `stage` (2048 elements) and read back transposed,
+// the A operand of dQ^T += K^T.dS^T.
 __device__ __forceinline__ void dq_pair(f32x4 dq[4], const bf16x8 bq[2], const bf16x8 bdo[2], float lse2, float delta,
-                                        float w, const bf16* const kb[2], const bf16* const vb[2],
-                                        const bf16* const ktb[2], int lane) {
+                                        float w, const bf16* const kb[2], const bf16* const vb[2], bf16* stage,
+                                        int lane) {
     bf16x8 kreg[2][2], vreg[2][2];
-    bf16x4 ktreg[2][4];
 #pragma unroll
     for (int j = 0; j < 2; j++) {
         kreg[j][0] = ld16(kb[j] + lane * 8);
@@ -87,9 +78,12 @@ __device__ __forceinline__ void dq_pair(f32x4 dq[4], const bf16x8 bq[2], const b
         vreg[j][1] = ld16(vb[j] + 512 + lane * 8);
     }
 #pragma unroll
-    for (int j = 0; j < 2; j++)
-#pragma unroll
-        for (int dt = 0; dt < 4; dt++) ktreg[j][dt] = ld8(ktb[j] + dt * 256 + lane * 4);
+    for (int j = 0; j < 2; j++) {
+        st16(stage + j * kTile + lane * 8, kreg[j][0]);
+        st16(stage + j * kTile + 512 + lane * 8, kreg[j][1]);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
     bf16x8 bds;
 #pragma unroll
     for (int j = 0; j < 2; j++) {
@@ -105,7 +99,10 @@ __device__ __forceinline__ void dq_pair(f32x4 dq[4], const bf16x8 bq[2], const b
         }
     }
 #pragma unroll
-    for (int dt = 0; dt < 4; dt++) dq[dt] = mfma_bf16(cat(ktreg[0][dt], ktreg[1][dt]), bds, dq[dt]);
+    for (int dt = 0; dt < 4; dt++)
+        dq[dt] = mfma_bf16(cat(lds_t_operand(stage, dt, lane), lds_t_operand(stage + kTile, dt, lane)), bds, dq[dt]);
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();              // the next pair overwrites `stage`
 }
 
 __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, const float* __restrict__ delta,
@@ -137,11 +134,11 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, cons
 
     const bf16* kr = (const bf16*)a.kr + (int64_t)bh * N1 * kTile;
     const bf16* vr = (const bf16*)a.vr + (int64_t)bh * N1 * kTile;
-    const bf16* kt = (const bf16*)a.kt + (int64_t)bh * N1 * kTile;
     const bf16* pk = (const bf16*)a.pkr + (int64_t)bh * N2 * kTile;
     const bf16* pv = (const bf16*)a.pvr + (int64_t)bh * N2 * kTile;
-    const bf16* pkt = (const bf16*)a.pkt + (int64_t)bh * N2 * kTile;
-    const bf16 *kb[2], *vb[2], *ktb[2];
+    const bf16 *kb[2], *vb[2];
+    __shared__ __align__(16) bf16 stage_all[4][2 * kTile];
+    bf16* stage = stage_all[wave];
 
     const int* ip = a.idx + ((int64_t)bh * N1 + g) * a.T;
     for (int t = 0; t < a.T / 2; t++) {
@@ -150,9 +147,8 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, cons
             const int blk = clampi(ip[2 * t + j], 0, N1 - 1);
             kb[j] = kr + (int64_t)blk * kTile;
             vb[j] = vr + (int64_t)blk * kTile;
-            ktb[j] = kt + (int64_t)blk * kTile;
         }
-        dq_pair(dq, bq, bdo, lse2, dl, 1.f, kb, vb, ktb, lane);
+        dq_pair(dq, bq, bdo, lse2, dl, 1.f, kb, vb, stage, lane);
     }
     if (a.levels == 2) {
         const int* pip = a.pidx + ((int64_t)bh * N2 + g / kBlk) * a.T2;
@@ -162,21 +158,18 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, cons
                 const int blk = clampi(pip[2 * t + j], 0, N2 - 1);
                 kb[j] = pk + (int64_t)blk * kTile;
                 vb[j] = pv + (int64_t)blk * kTile;
-                ktb[j] = pkt + (int64_t)blk * kTile;
             }
-            dq_pair(dq, bq, bdo, lse2, dl, a.w1, kb, vb, ktb, lane);
+            dq_pair(dq, bq, bdo, lse2, dl, a.w1, kb, vb, stage, lane);
         }
         const bf16* pk2 = (const bf16*)a.pk2r + (int64_t)bh * (N2 / kBlk) * kTile;
         const bf16* pv2 = (const bf16*)a.pv2r + (int64_t)bh * (N2 / kBlk) * kTile;
-        const bf16* pk2t = (const bf16*)a.pk2t + (int64_t)bh * (N2 / kBlk) * kTile;
         for (int t = 0; t < N2 / 32; t++) {
 #pragma unroll
             for (int j = 0; j < 2; j++) {
                 kb[j] = pk2 + (int64_t)(2 * t + j) * kTile;
                 vb[j] = pv2 + (int64_t)(2 * t + j) * kTile;
-                ktb[j] = pk2t + (int64_t)(2 * t + j) * kTile;
             }
-            dq_pair(dq, bq, bdo, lse2, dl, a.w2, kb, vb, ktb, lane);
+            dq_pair(dq, bq, bdo, lse2, dl, a.w2, kb, vb, stage, lane);
         }
     } else {
         for (int t = 0; t < N1 / 32; t++) {
@@ -184,9 +177,8 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, cons
             for (int j = 0; j < 2; j++) {
                 kb[j] = pk + (int64_t)(2 * t + j) * kTile;
                 vb[j] = pv + (int64_t)(2 * t + j) * kTile;
-                ktb[j] = pkt + (int64_t)(2 * t + j) * kTile;
             }
-            dq_pair(dq, bq, bdo, lse2, dl, a.w1, kb, vb, ktb, lane);
+            dq_pair(dq, bq, bdo, lse2, dl, a.w1, kb, vb, stage, lane);
         }
     }
 
@@ -221,7 +213,6 @@ enum { MODE_FINE = 0, MODE_SPARSE1 = 1, MODE_DENSE = 2 };
 
 struct KSideParams {
     const bf16* qr;  const bf16* dor;             // R tiles of q and dO, (BH, N1, 1024)
-    const bf16* qt;  const bf16* dot;             // T tiles of q and dO
     const float* lse; const float* delta;         // (BH, N)
     const bf16* kk;  const bf16* vv;              // R tiles the unit's 16 key rows come from, (BH, n_units, 1024)
     const int* off;  const int* flat;             // CSR of the list (FINE: per K block, SPARSE1: per coarse block)
@@ -236,15 +227,17 @@ struct KSideParams {
     float w;
 };
 
-// Two query blocks (g0, g1; g1 < 0: only one) against the unit's 16 key rows.  All operands of
-// both blocks are fetched first -- eight 1 KB and eight 512 B coalesced loads -- then used.
+// Two query blocks (g0, g1; g1 < 0: only one) against the unit's 16 key rows.  Q and dO are
+// fetched once, as R tiles: they are the A operands of S = Q.K^T and dP = dO.V^T straight from
+// the registers, and they are parked in a wave-private piece of LDS (`stage`, 4096 elements)
+// from which the transposing LDS read delivers them again as T operands for dV^T += dO^T.P and
+// dK^T += Q^T.dS.
 __device__ __forceinline__ void kside_pair(f32x4 dk[4], f32x4 dv[4], const bf16x8 bk[2], const bf16x8 bv[2], float w,
-                                           int g0, int g1, const bf16* qrb, const bf16* dorb, const bf16* qtb,
-                                           const bf16* dotb, const float* lseb, const float* dlb, int lane) {
+                                           int g0, int g1, const bf16* qrb, const bf16* dorb, const float* lseb,
+                                           const float* dlb, bf16* stage, int lane) {
     const int quad = lane >> 4;
     const int gg[2] = {g0, (g1 < 0) ? g0 : g1};
     bf16x8 aq[2][2], ag[2][2];
-    bf16x4 tq[2][4], tg[2][4];
     f32x4 l4[2], d4[2];
 #pragma unroll
     for (int u = 0; u < 2; u++) {
@@ -257,12 +250,14 @@ __device__ __forceinline__ void kside_pair(f32x4 dk[4], f32x4 dv[4], const bf16x
         d4[u] = *reinterpret_cast<const f32x4*>(dlb + gg[u] * kBlk + quad * 4);
     }
 #pragma unroll
-    for (int u = 0; u < 2; u++)
-#pragma unroll
-        for (int dt = 0; dt < 4; dt++) {
-            tq[u][dt] = ld8(qtb + (int64_t)gg[u] * kTile + dt * 256 + lane * 4);
-            tg[u][dt] = ld8(dotb + (int64_t)gg[u] * kTile + dt * 256 + lane * 4);
-        }
+    for (int u = 0; u < 2; u++) {
+        st16(stage + (u * 2 + 0) * kTile + lane * 8, aq[u][0]);
+        st16(stage + (u * 2 + 0) * kTile + 512 + lane * 8, aq[u][1]);
+        st16(stage + (u * 2 + 1) * kTile + lane * 8, ag[u][0]);
+        st16(stage + (u * 2 + 1) * kTile + 512 + lane * 8, ag[u][1]);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
     bf16x8 bp, bds;
 #pragma unroll
     for (int u = 0; u < 2; u++) {
@@ -282,9 +277,13 @@ __device__ __forceinline__ void kside_pair(f32x4 dk[4], f32x4 dv[4], const bf16x
     }
 #pragma unroll
     for (int dt = 0; dt < 4; dt++) {
-        dv[dt] = mfma_bf16(cat(tg[0][dt], tg[1][dt]), bp, dv[dt]);
-        dk[dt] = mfma_bf16(cat(tq[0][dt], tq[1][dt]), bds, dk[dt]);
+        const bf16x4 tg0 = lds_t_operand(stage + 1 * kTile, dt, lane), tg1 = lds_t_operand(stage + 3 * kTile, dt, lane);
+        const bf16x4 tq0 = lds_t_operand(stage + 0 * kTile, dt, lane), tq1 = lds_t_operand(stage + 2 * kTile, dt, lane);
+        dv[dt] = mfma_bf16(cat(tg0, tg1), bp, dv[dt]);
+        dk[dt] = mfma_bf16(cat(tq0, tq1), bds, dk[dt]);
     }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();              // the next pair overwrites `stage`
 }
 
 // A partial sum of one unit (16 key rows x 64 channels, dK and dV) is kept in the MFMA
@@ -294,6 +293,8 @@ __device__ __forceinline__ f32x4* part_slot(f32x4* part, int64_t slot) { return 
 template <int MODE>
 __global__ __launch_bounds__(256) void attn_kside_kernel(KSideParams p) {
     constexpr int W = (MODE == MODE_FINE) ? 1 : 4;            // waves per work item
+    // 4 waves x (2 query blocks x {Q, dO} R tiles); reused for the cross-wave reduction
+    __shared__ __align__(16) unsigned char smem_raw[4 * 4 * kTile * sizeof(bf16)];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int N1 = p.N / kBlk;
@@ -350,14 +351,13 @@ __global__ __launch_bounds__(256) void attn_kside_kernel(KSideParams p) {
         bv[1] = ld16(vp + 512);
         const bf16* qrb = p.qr + (int64_t)bh * N1 * kTile;
         const bf16* dorb = p.dor + (int64_t)bh * N1 * kTile;
-        const bf16* qtb = p.qt + (int64_t)bh * N1 * kTile;
-        const bf16* dotb = p.dot + (int64_t)bh * N1 * kTile;
         const float* lseb = p.lse + (int64_t)bh * p.N;
         const float* dlb = p.delta + (int64_t)bh * p.N;
+        bf16* stage = reinterpret_cast<bf16*>(smem_raw) + wave * (4 * kTile);
         for (int i = 2 * sub; i < cnt; i += 2 * W) {
             const int g0 = entry(i);
             const int g1 = (i + 1 < cnt) ? entry(i + 1) : -1;
-            kside_pair(dk, dv, bk, bv, p.w, g0, g1, qrb, dorb, qtb, dotb, lseb, dlb, lane);
+            kside_pair(dk, dv, bk, bv, p.w, g0, g1, qrb, dorb, lseb, dlb, stage, lane);
         }
     }
 
@@ -381,7 +381,9 @@ __global__ __launch_bounds__(256) void attn_kside_kernel(KSideParams p) {
         return;
     }
     // four waves per item: reduce through LDS, wave w finishes channel tile w
-    __shared__ f32x4 red[4][8][kWave];
+    __syncthreads();                                          // everyone is done with the staging area
+    f32x4 (*red)[8][kWave] = reinterpret_cast<f32x4 (*)[8][kWave]>(smem_raw);
+    static_assert(sizeof(smem_raw) >= 4 * 8 * kWave * sizeof(f32x4), "reduction buffer must fit the staging area");
 #pragma unroll
     for (int dt = 0; dt < 4; dt++) {
         red[wave][dt][lane] = dk[dt];
@@ -501,7 +503,7 @@ static int64_t align256(int64_t x) { return (x + 255) & ~(int64_t)255; }
 constexpr int64_t kSlotBytes = 8 * kWave * sizeof(f32x4);     // one partial: 16 rows x 64 ch x (dK, dV) fp32
 
 struct BwdWorkspace {
-    int64_t delta, dor, dot, part_fine, part_coarse, part_dense, total;
+    int64_t delta, dor, part_fine, part_coarse, part_dense, total;
     int64_t slots_fine, slots_coarse;                           // per (b,h)
 };
 
@@ -516,7 +518,6 @@ static BwdWorkspace bwd_workspace(int B, int H, int N, int T, int T2, int levels
     int64_t o = 0;
     w.delta = o;        o += align256(BH * N * 4);
     w.dor = o;          o += align256(BH * N * 64 * 2);
-    w.dot = o;          o += align256(BH * N * 64 * 2);
     w.part_fine = o;    o += align256(BH * w.slots_fine * kSlotBytes);
     w.part_coarse = o;  o += align256(BH * w.slots_coarse * kSlotBytes);
     w.part_dense = o;   o += align256((int64_t)d.chunks * BH * (d.n_tok / 16) * kSlotBytes);
@@ -537,7 +538,7 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     LLSA_REQUIRE(a != nullptr, "attn_bwd: null args");
     LLSA_REQUIRE(a->levels == 1 || a->levels == 2, "attn_bwd: levels must be 1 or 2");
     LLSA_REQUIRE(a->B > 0 && a->H > 0 && a->N > 0, "attn_bwd: bad B/H/N");
-    LLSA_REQUIRE(a->dout && a->o && a->lse && a->qr && a->qt && a->kr && a->kt && a->vr && a->pkr && a->pkt && a->pvr && a->idx &&
+    LLSA_REQUIRE(a->dout && a->o && a->lse && a->qr && a->kr && a->vr && a->pkr && a->pvr && a->idx &&
                      a->off && a->flat && a->dq && a->dk && a->dv && a->dpk && a->dpv && a->workspace,
                  "attn_bwd: null tensor");
     LLSA_REQUIRE(a->T >= 4 && a->T % 4 == 0 && a->T <= a->N / 16, "attn_bwd: topk=%d must be a multiple of 4 and <= N/16", a->T);
@@ -546,11 +547,11 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
         LLSA_REQUIRE(a->N % 1024 == 0, "attn_bwd: llsa_l1 needs N %% 1024 == 0 (N=%d)", a->N);
     } else {
         LLSA_REQUIRE(a->N % 16384 == 0, "attn_bwd: llsa_l2 needs N %% 16384 == 0 (N=%d)", a->N);
-        LLSA_REQUIRE(a->pk2r && a->pv2r && a->pk2t && a->pidx && a->poff && a->pflat && a->dpk2 && a->dpv2, "attn_bwd: level-2 tensors missing");
+        LLSA_REQUIRE(a->pk2r && a->pv2r && a->pidx && a->poff && a->pflat && a->dpk2 && a->dpv2, "attn_bwd: level-2 tensors missing");
         LLSA_REQUIRE(a->T2 >= 4 && a->T2 % 4 == 0 && a->T2 <= a->N / 256, "attn_bwd: topk2=%d must be a multiple of 4 and <= N/256", a->T2);
         LLSA_REQUIRE(a->w2 > 0.f, "attn_bwd: token_weight_2 must be > 0");
     }
-    const void* al[] = {a->dout, a->o, a->qr, a->qt, a->kr, a->kt, a->vr, a->pkr, a->pkt, a->pvr, a->pk2r, a->pk2t, a->pv2r,
+    const void* al[] = {a->dout, a->o, a->qr, a->kr, a->vr, a->pkr, a->pvr, a->pk2r, a->pv2r,
                         a->dq, a->dk, a->dv, a->dpk, a->dpv, a->dpk2, a->dpv2, a->workspace, a->freq_dq, a->lse};
     for (const void* p : al) LLSA_REQUIRE(aligned16(p), "attn_bwd: tensors must be 16-byte aligned");
     const int64_t st[] = {a->sdob, a->sdoh, a->sdon, a->sob, a->soh, a->son};
@@ -568,10 +569,9 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     char* ws = (char*)a->workspace;
     float* delta = (float*)(ws + wsp.delta);
     bf16* dor = (bf16*)(ws + wsp.dor);
-    bf16* dot = (bf16*)(ws + wsp.dot);
 
     const int stages = a->stages ? a->stages : 0x7fffffff;
-    if (stages & LLSA_BWD_PRE) hipLaunchKernelGGL(bwd_pre_kernel, dim3((N1 + 15) / 16, BH), dim3(128), 0, s, *a, delta, dor, dot);
+    if (stages & LLSA_BWD_PRE) hipLaunchKernelGGL(bwd_pre_kernel, dim3((N1 + 15) / 16, BH), dim3(128), 0, s, *a, delta, dor);
     if (stages & LLSA_BWD_DQ)
         hipLaunchKernelGGL(attn_dq_kernel, dim3((N1 + 3) / 4, BH), dim3(256), 0, s, *a, (const float*)delta, (const bf16*)dor);
 
@@ -580,7 +580,7 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     rp.H = H;
     KSideParams p;
     p.qr = (const bf16*)a->qr; p.dor = dor;
-    p.qt = (const bf16*)a->qt; p.dot = dot; p.lse = a->lse; p.delta = delta;
+    p.lse = a->lse; p.delta = delta;
     p.H = H; p.N = N; p.chunk_len = 0;
 
     // fine K/V blocks

@@ -91,6 +91,21 @@ constexpr int kTile = kBlk * kD;     // elements per block tile
 __device__ __forceinline__ int r_tile_off(int i, int c) { return ((c >> 3) * 16 + i) * 8 + (c & 7); }
 __device__ __forceinline__ int t_tile_off(int t, int c) { return (((c >> 4) * 4 + (t >> 2)) * 16 + (c & 15)) * 4 + (t & 3); }
 
+// A T operand out of an R tile that sits in LDS, with the transposing LDS read of gfx950
+// (ds_read_b64_tr_b16).  Within each group of 16 lanes, lane j supplies the address of four
+// consecutive 16-bit elements and lane i receives element i%4 of the chunks supplied by lanes
+// i/4, 4 + i/4, 8 + i/4, 12 + i/4.  Pointing lane j at (token 4*(l/16) + j/4, channels
+// 16*dt + 4*(j%4) ..+3) therefore hands lane i tokens 4*(l/16)..+3 of channel 16*dt + i: the T
+// operand.  So K/Q/dO are fetched from HBM once, as R tiles, and the second orientation is
+// made on chip instead of being read from a second copy.
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+__device__ __forceinline__ bf16x4 lds_t_operand(const bf16* r_tile_in_lds, int dt, int lane) {
+    const int j = lane & 15, q = lane >> 4;
+    const bf16* p = r_tile_in_lds + r_tile_off(4 * q + (j >> 2), 16 * dt + 4 * (j & 3));
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4*)p);
+    return __builtin_bit_cast(bf16x4, v);
+}
+
 // XCD-aware workgroup order.  The 8 XCDs of the chip each have a private L2 and receive
 // workgroups round-robin by linear id (id % 8).  Neighbouring logical work items (query or
 // key blocks that are close in Z-order) read overlapping K/V/Q rows, so they should share an

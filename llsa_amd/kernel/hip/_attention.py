@@ -92,7 +92,7 @@ def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_wei
     """Backward.  Returns (dq, dk, dv, dpk, dpv[, dpk2, dpv2]) with the reference's conventions:
     every gradient is `empty_like` of its primal; the pooled gradients are NOT yet folded
     into dk / dv (autograd, or pool_bwd_accum, does that).  `tiles` may carry operand tiles the
-    caller already has (qr, qt, kr, kt, vr, pkr, pkt, pvr, pk2r, pk2t, pv2r).  `stages` (a mask of
+    caller already has (qr, kr, vr, pkr, pvr, pk2r, pv2r).  `stages` (a mask of
     the LLSA_BWD_* bits of include/llsa_hip.h) launches only some of the kernels, for profiling."""
     levels = 1 if pk2 is None else 2
     lib = lib_for(do, q, k, v, pk, pv, pk2, pv2, o, lse)
@@ -103,10 +103,9 @@ def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_wei
     T = indices.shape[-1]
     T2 = p_indices.shape[-1] if levels == 2 else 0
     do, o = as_rows(do), as_rows(o)
-    need = dict(qr=(q, "r"), qt=(q, "t"), kr=(k, "r"), kt=(k, "t"), vr=(v, "r"), pkr=(pk, "r"), pkt=(pk, "t"),
-                pvr=(pv, "r"))
+    need = dict(qr=(q, "r"), kr=(k, "r"), vr=(v, "r"), pkr=(pk, "r"), pvr=(pv, "r"))
     if levels == 2:
-        need.update(pk2r=(pk2, "r"), pk2t=(pk2, "t"), pv2r=(pv2, "r"))
+        need.update(pk2r=(pk2, "r"), pv2r=(pv2, "r"))
     tl = _tiles(tiles, need)
     idx = indices.to(torch.int32).contiguous()
     if levels == 2:
@@ -129,7 +128,7 @@ def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_wei
     a.o, (a.sob, a.soh, a.son) = o.data_ptr(), s3(o)
     lse = lse.contiguous()
     a.lse = lse.data_ptr()
-    for n in ("qr", "qt", "kr", "kt", "vr", "pkr", "pkt", "pvr"):
+    for n in ("qr", "kr", "vr", "pkr", "pvr"):
         setattr(a, n, tl[n].data_ptr())
     a.idx, a.off, a.flat, a.work = idx.data_ptr(), off.data_ptr(), flat.data_ptr(), work.data_ptr()
     a.dq, (a.sdqb, a.sdqh, a.sdqn) = dq.data_ptr(), s3(dq)
@@ -140,7 +139,7 @@ def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_wei
     if levels == 2:
         dpk2 = torch.empty_like(pk2, memory_format=torch.contiguous_format)
         dpv2 = torch.empty_like(pv2, memory_format=torch.contiguous_format)
-        for n in ("pk2r", "pk2t", "pv2r"):
+        for n in ("pk2r", "pv2r"):
             setattr(a, n, tl[n].data_ptr())
         a.pidx, a.poff, a.pflat, a.pwork = pidx.data_ptr(), poff.data_ptr(), pflat.data_ptr(), pwork.data_ptr()
         a.dpk2, a.dpv2 = dpk2.data_ptr(), dpv2.data_ptr()

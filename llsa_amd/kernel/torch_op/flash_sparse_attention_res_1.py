@@ -53,8 +53,8 @@ class _LlsaL1Fused(Function):
             raise NotImplementedError("block_size must be 16")
         g = any(ctx.needs_input_grad[:3])
         rope = freq is not None
-        oq, ok, ov = pool_pyramid([PoolSpec(q, y1=True, xr=True, xt=g, rope=rope),
-                                   PoolSpec(k, y1=True, xr=True, xt=g, y1r=True, y1t=g, rope=rope),
+        oq, ok, ov = pool_pyramid([PoolSpec(q, y1=True, xr=True, rope=rope),
+                                   PoolSpec(k, y1=True, xr=True, y1r=True, rope=rope),
                                    PoolSpec(v, y1=True, xr=g, xt=True, y1r=g, y1t=True)], freq)
         pq, pk, pv = oq["y1"], ok["y1"], ov["y1"]
         indices = gen_sparse_indices(pq, pk, topk)
@@ -62,17 +62,16 @@ class _LlsaL1Fused(Function):
         # q / k are only shape-and-stride templates below: the kernels read the (rotated) tiles
         o, m = sparse_indices_attn_res_fwd(q, k, v, pk, pv, indices, indices.shape[-1], block_size, 4, tiles=tiles)
         if g:
-            ctx.save_for_backward(q, k, v, pk, pv, o, m, indices, freq, oq["xr"], oq["xt"], ok["xr"], ok["xt"], ov["xr"],
-                                  ok["y1r"], ok["y1t"], ov["y1r"])
+            ctx.save_for_backward(q, k, v, pk, pv, o, m, indices, freq, oq["xr"], ok["xr"], ov["xr"], ok["y1r"], ov["y1r"])
         ctx.block_size = block_size
         ctx.indices = indices
         return o
 
     @staticmethod
     def backward(ctx, do):
-        q, k, v, pk, pv, o, m, indices, freq, qr, qt, kr, kt, vr, pkr, pkt, pvr = ctx.saved_tensors
+        q, k, v, pk, pv, o, m, indices, freq, qr, kr, vr, pkr, pvr = ctx.saved_tensors
         bs = ctx.block_size
-        tiles = dict(qr=qr, qt=qt, kr=kr, kt=kt, vr=vr, pkr=pkr, pkt=pkt, pvr=pvr)
+        tiles = dict(qr=qr, kr=kr, vr=vr, pkr=pkr, pvr=pvr)
         dq, dk, dv, _, dpk, dpv = sparse_indices_attn_res_scatter_bwd_v2(
             do, q, k, v, pk, pv, o, m, indices, indices.shape[-1], bs, bs, tiles=tiles, freq_dq=freq)
         dk = pool_bwd_accum(dk, dpk, None, freq, out=dk)

@@ -31,6 +31,7 @@ struct WaveSync {
     int arrived = 0;
     unsigned gen = 0;
     uint32_t stage[kWave];
+    const void* ptr[kWave];
     bf16x8_t a[kWave], b[kWave];
 };
 std::vector<WaveSync> waves;
@@ -128,6 +129,20 @@ f32x4_t mfma_16x16x32_bf16(bf16x8_t a, bf16x8_t b, f32x4_t c) {
     }
     wave_barrier();
     return d;
+}
+
+// ds_read_b64_tr_b16: in each group of 16 lanes, lane i gets element i%4 of the 8-byte chunks
+// addressed by lanes i/4, 4 + i/4, 8 + i/4, 12 + i/4 (behaviour observed on gfx950 hardware).
+s16x4_t ds_read_tr16_b64(const void* p) {
+    WaveSync& ws = waves[cur / kWave];
+    const int l = cur % kWave;
+    ws.ptr[l] = p;
+    wave_barrier();
+    const int grp = l & ~15, i = l & 15;
+    s16x4_t r;
+    for (int e = 0; e < 4; e++) r[e] = reinterpret_cast<const short*>(ws.ptr[grp + 4 * e + i / 4])[i % 4];
+    wave_barrier();
+    return r;
 }
 
 void launch(dim3 grid, dim3 block, size_t shmem, const std::function<void()>& body) {

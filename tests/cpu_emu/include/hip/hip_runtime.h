@@ -52,6 +52,8 @@ int lane_id();
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 f32x4_t mfma_16x16x32_bf16(bf16x8_t a, bf16x8_t b, f32x4_t c);
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+s16x4_t ds_read_tr16_b64(const void* p);
 }  // namespace emu
 
 #define threadIdx emu::g_threadIdx
@@ -98,6 +100,7 @@ inline int __ffs(int x) { return __builtin_ffs(x); }
 inline int __clz(int x) { return x ? __builtin_clz((unsigned)x) : 32; }
 
 #define __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, x, y, z) emu::mfma_16x16x32_bf16((a), (b), (c))
+#define __builtin_amdgcn_ds_read_tr16_b64_v4i16(p) emu::ds_read_tr16_b64((const void*)(p))
 #define __builtin_amdgcn_exp2f(x) exp2f(x)
 #define __builtin_amdgcn_logf(x) log2f(x)
 #define __builtin_amdgcn_rcpf(x) (1.0f / (x))
