@@ -32,6 +32,14 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 
+# HBM-side bytes per launch (L2 <-> fabric reads + writes) measured with rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE on this command, each scaled by what the same counter reads for a 256 MiB elementwise
+# copy (fetch x2.000, write x1.000); the tables they come from are profiles/step_kernels_<workload>_hbm_traffic.txt
+MEASURED_TRAFFIC = {
+    "c3": {"attn_fwd": 130407581, "bwd_dq": 192478201, "bwd_dkv": 261496020, "bwd_dpkv1_sparse": 244863559,
+           "bwd_dpkv_dense": 78392634, "pool_pyramid": 103315496},
+}
+
 WORKLOADS = {
     # name: (op, B, H, N, topk1, topk2, rope)
     "c2": ("l1", 4, 6, 4096, 16, 0, False),
@@ -175,6 +183,10 @@ def main():
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-extras", action="store_true", help="skip stage profile, CPU baseline and dense SDPA")
     ap.add_argument("--unfused", action="store_true", help="use the reference's composition (separate pools, autograd adds)")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="after the timed region also launch a plain elementwise copy of 256 MiB (fp32, read 256 MiB + "
+                         "write 256 MiB) five times, so that a counter profile of this command holds a kernel of known "
+                         "HBM traffic to scale FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (one MI355X per box); --gpus must be 1", file=sys.stderr)
@@ -210,6 +222,14 @@ def main():
         step()
     torch.cuda.synchronize()
     ms = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    if args.calibrate:
+        src = torch.ones(64 * 1024 * 1024, device=dev, dtype=torch.float32)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
 
     nkv = n_kv(op, N, t1, t2)
     unit_flops = B * H * N * D * nkv                    # one "GEMM unit": 2 * this = one product
@@ -255,11 +275,12 @@ def main():
         out["stage_sum_ms"] = sum(st.values())
         dom = max(alg, key=lambda n: st[n])
         out["roofline"] = {"kernel": dom, "bound": "mfma", "achieved": kernels[dom]["tflops"], "peak": PEAK_BF16_TFLOPS,
-                           "unit": "TFLOP/s", "frac": kernels[dom]["frac_mfma_peak"], "traffic": None,
+                           "unit": "TFLOP/s", "frac": kernels[dom]["frac_mfma_peak"],
+                           "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get(dom),
                            "avg_launch_ms": st[dom], "algorithmic_gflop_per_launch": alg[dom] / 1e9}
         out["roofline_hbm"] = {"kernel": "pool_pyramid", "bound": "hbm", "achieved": kernels["pool_pyramid"]["gbs"],
                                "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": kernels["pool_pyramid"]["frac_hbm_peak"],
-                               "traffic": None}
+                               "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("pool_pyramid")}
         # dense attention on the same GPU
         try:
             import torch.nn.functional as F

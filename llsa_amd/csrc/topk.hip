@@ -143,18 +143,25 @@ __device__ __forceinline__ void wave_topk_radix(const unsigned* u, int npos, int
         uk[e] = ok[e] ? u[pos] : 0u;
         gk[e] = ok[e] ? (unsigned)gidx_of(pos) : 0xFFFFFFFFu;
     }
+    // Invalid slots hold key 0 and never equal `want` (its current bit is set), so the bit loop
+    // needs no validity mask.  `match` counts the entries that agree with the decided bits; once
+    // it equals the number still to take, all of them are winners and the remaining bits need
+    // not be looked at (tau = prefix with zero low bits then selects exactly those).
     unsigned prefix = 0;
-    int remaining = T;
-    for (int bit = 31; bit >= 0; bit--) {
+    int remaining = T, match = npos;
+    for (int bit = 31; bit >= 0 && match != remaining; bit--) {
         const unsigned msk = (bit == 31) ? 0x80000000u : ((0xFFFFFFFFu << (bit + 1)) | (1u << bit));
         const unsigned want = prefix | (1u << bit);
         int cnt1 = 0;
 #pragma unroll
-        for (int e = 0; e < E; e++) cnt1 += __popcll(__ballot(ok[e] && (uk[e] & msk) == want));
-        if (cnt1 >= remaining)
+        for (int e = 0; e < E; e++) cnt1 += __popcll(__ballot((uk[e] & msk) == want));
+        if (cnt1 >= remaining) {
             prefix = want;
-        else
+            match = cnt1;
+        } else {
             remaining -= cnt1;
+            match -= cnt1;
+        }
     }
     const unsigned tau = prefix;                              // the T-th largest score
     int n_eq = 0;
@@ -225,11 +232,12 @@ __device__ __forceinline__ void wave_topk_radix_any(const unsigned* u, int npos,
 constexpr int kRadixMaxN = 1024;      // keys per row the radix kernels keep in LDS
 
 // dense selection for n <= kRadixMaxN: 16 query rows per workgroup, all n keys scored into LDS
-__global__ __launch_bounds__(256) void topk_dense_radix_kernel(const bf16* __restrict__ pq, const bf16* __restrict__ pk,
-                                                               int* __restrict__ out, int n, int T, int round_scores) {
+// (16 waves: one row each, so the 16 selections run side by side instead of four deep)
+__global__ __launch_bounds__(1024) void topk_dense_radix_kernel(const bf16* __restrict__ pq, const bf16* __restrict__ pk,
+                                                                int* __restrict__ out, int n, int T, int round_scores) {
     HIP_DYNAMIC_SHARED(unsigned, su)                          // [16][n + 1]
-    __shared__ unsigned sel_u[4][kWave];
-    __shared__ int sel_i[4][kWave];
+    __shared__ unsigned sel_u[16][kWave];
+    __shared__ int sel_i[16][kWave];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int bh = blockIdx.y, q0 = blockIdx.x * 16;
     const int stride = n + 1;
@@ -238,26 +246,26 @@ __global__ __launch_bounds__(256) void topk_dense_radix_kernel(const bf16* __res
     bf16x8 bq[2];
     bq[0] = ld16(pqb + (lane & 15) * kD + (lane >> 4) * 8);
     bq[1] = ld16(pqb + (lane & 15) * kD + (lane >> 4) * 8 + 32);
-    for (int tile = wave; tile < n / 16; tile += 4) {
+    for (int tile = wave; tile < n / 16; tile += 16) {
         f32x4 s = score_tile(pkb + (int64_t)tile * 16 * kD, bq);
 #pragma unroll
         for (int e = 0; e < 4; e++)
             su[(lane & 15) * stride + tile * 16 + 4 * (lane >> 4) + e] = ordered_bits(round_scores ? rn_bf16(s[e]) : s[e]);
     }
     __syncthreads();
-    for (int row = wave; row < 16; row += 4)
+    for (int row = wave; row < 16; row += 16)
         wave_topk_radix_any(
             su + row * stride, n, T, [](int pos) { return pos; }, sel_u[wave], sel_i[wave],
             out + ((int64_t)bh * n + q0 + row) * T, lane);
 }
 
-__global__ __launch_bounds__(256) void topk_sparse_kernel(const bf16* __restrict__ pq, const bf16* __restrict__ pk,
-                                                          const int* __restrict__ pidx, int* __restrict__ out, int N1,
-                                                          int T, int T2) {
+__global__ __launch_bounds__(1024) void topk_sparse_kernel(const bf16* __restrict__ pq, const bf16* __restrict__ pk,
+                                                           const int* __restrict__ pidx, int* __restrict__ out, int N1,
+                                                           int T, int T2) {
     __shared__ unsigned su[16][kMaxCand + 1];
     __shared__ int cand[kMaxCand];
-    __shared__ unsigned sel_u[4][kWave];
-    __shared__ int sel_i[4][kWave];
+    __shared__ unsigned sel_u[16][kWave];
+    __shared__ int sel_i[16][kWave];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int bh = blockIdx.y, G = blockIdx.x;
@@ -265,20 +273,20 @@ __global__ __launch_bounds__(256) void topk_sparse_kernel(const bf16* __restrict
     const bf16* pqb = pq + ((int64_t)bh * N1 + G * kBlk) * kD;
     const bf16* pkb = pk + (int64_t)bh * N1 * kD;
 
-    for (int i = tid; i < C; i += 256)
+    for (int i = tid; i < C; i += 1024)
         cand[i] = clampi(pidx[((int64_t)bh * N2 + G) * T2 + i / kBlk], 0, N2 - 1) * kBlk + (i % kBlk);
     bf16x8 bq[2];
     bq[0] = ld16(pqb + (lane & 15) * kD + (lane >> 4) * 8);
     bq[1] = ld16(pqb + (lane & 15) * kD + (lane >> 4) * 8 + 32);
     __syncthreads();
 
-    for (int a = wave; a < T2; a += 4) {
+    for (int a = wave; a < T2; a += 16) {
         f32x4 s = score_tile(pkb + (int64_t)cand[a * kBlk] * kD, bq);
 #pragma unroll
         for (int e = 0; e < 4; e++) su[lane & 15][a * kBlk + 4 * (lane >> 4) + e] = ordered_bits(s[e]);
     }
     __syncthreads();
-    for (int row = wave; row < 16; row += 4)
+    for (int row = wave; row < 16; row += 16)
         wave_topk_radix_any(
             su[row], C, T, [&](int pos) { return cand[pos]; }, sel_u[wave], sel_i[wave],
             out + ((int64_t)bh * N1 + G * kBlk + row) * T, lane);
@@ -300,7 +308,7 @@ extern "C" int llsa_topk_dense(const void* pq, const void* pk, int32_t* out_idx,
             hipError_t e = hipFuncSetAttribute((const void*)topk_dense_radix_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
             if (e != hipSuccess) return fail(-101, "topk_dense: cannot raise dynamic LDS to %d bytes: %s", lds, hipGetErrorString(e));
         }
-        hipLaunchKernelGGL(topk_dense_radix_kernel, dim3(n / 16, B * H), dim3(256), sizeof(unsigned) * 16 * (n + 1),
+        hipLaunchKernelGGL(topk_dense_radix_kernel, dim3(n / 16, B * H), dim3(1024), sizeof(unsigned) * 16 * (n + 1),
                            (hipStream_t)stream, (const bf16*)pq, (const bf16*)pk, out_idx, n, T, round_scores);
     } else
         hipLaunchKernelGGL(topk_dense_kernel, dim3(n / 16, B * H), dim3(256), 0, (hipStream_t)stream, (const bf16*)pq,
@@ -315,7 +323,7 @@ extern "C" int llsa_topk_sparse(const void* pq, const void* pk, const int32_t* p
     LLSA_REQUIRE(T2 >= 1 && T2 * 16 <= kMaxCand && T2 <= N1 / 16, "topk_sparse: need 1 <= T2 <= min(%d, N1/16), got %d", kMaxCand / 16, T2);
     LLSA_REQUIRE(T >= 1 && T <= kMaxT && T <= T2 * 16, "topk_sparse: need 1 <= T <= min(%d, 16*T2), got %d", kMaxT, T);
     LLSA_REQUIRE(aligned16(pq) && aligned16(pk), "topk_sparse: inputs must be 16-byte aligned");
-    hipLaunchKernelGGL(topk_sparse_kernel, dim3(N1 / 16, B * H), dim3(256), 0, (hipStream_t)stream, (const bf16*)pq,
+    hipLaunchKernelGGL(topk_sparse_kernel, dim3(N1 / 16, B * H), dim3(1024), 0, (hipStream_t)stream, (const bf16*)pq,
                        (const bf16*)pk, parent_idx, out_idx, N1, T, T2);
     return launch_status("topk_sparse");
 }
