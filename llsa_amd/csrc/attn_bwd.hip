@@ -291,10 +291,13 @@ __device__ __forceinline__ void kside_pair(f32x4 dk[4], f32x4 dv[4], const bf16x
 __device__ __forceinline__ f32x4* part_slot(f32x4* part, int64_t slot) { return part + slot * (8 * kWave); }
 
 template <int MODE>
-__global__ __launch_bounds__(256) void attn_kside_kernel(KSideParams p) {
-    constexpr int W = (MODE == MODE_FINE) ? 1 : 4;            // waves per work item
-    // 4 waves x (2 query blocks x {Q, dO} R tiles); reused for the cross-wave reduction
-    __shared__ __align__(16) unsigned char smem_raw[4 * 4 * kTile * sizeof(bf16)];
+__global__ __launch_bounds__(MODE == MODE_FINE ? 64 : 256) void attn_kside_kernel(KSideParams p) {
+    // FINE: one wave per work item and per workgroup (items differ a lot in length; a wave that
+    // shares its workgroup with a longer one would keep its registers and LDS allocated while idle).
+    // Others: four waves per work item.
+    constexpr int W = (MODE == MODE_FINE) ? 1 : 4;            // waves per work item = waves per workgroup
+    // per wave 2 query blocks x {Q, dO} R tiles; reused for the cross-wave reduction
+    __shared__ __align__(16) unsigned char smem_raw[W * 4 * kTile * sizeof(bf16)];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int N1 = p.N / kBlk;
@@ -315,7 +318,7 @@ __global__ __launch_bounds__(256) void attn_kside_kernel(KSideParams p) {
         slot = ((int64_t)blockIdx.z * gridDim.y + bh) * p.n_units + unit;
     } else {
         const int* work = p.work + (int64_t)bh * p.work_stride;
-        const int item = (MODE == MODE_FINE) ? bx * 4 + wave : bx;
+        const int item = bx;
         if (item >= work[0]) return;                          // uniform over the item's waves
         const int it = work[4 + p.n_units + item];
         const int ci = it & 0xffff;
@@ -329,8 +332,12 @@ __global__ __launch_bounds__(256) void attn_kside_kernel(KSideParams p) {
         if (sb >= 0) slot = (int64_t)bh * p.slot_stride + sb + ci;
         fl = p.flat + (int64_t)bh * p.flat_stride;
     }
-    auto entry = [&](int i) -> int {                          // i-th query block of this item
-        if (MODE == MODE_FINE) return clampi(fl[start + i], 0, N1 - 1);
+    // The item's list entries (FINE: at most 32 query blocks) are fetched once, entry i into
+    // lane i, and handed out with readlane: the walk below then has no load that depends on a load.
+    int mine = 0;
+    if (MODE == MODE_FINE) mine = (lane < cnt) ? fl[start + lane] : 0;
+    auto entry = [&](int i) -> int {                          // i-th query block of this item (i is wave-uniform)
+        if (MODE == MODE_FINE) return clampi(__builtin_amdgcn_readlane(mine, i), 0, N1 - 1);
         if (MODE == MODE_SPARSE1) return clampi(fl[start + i / kBlk], 0, N1 / kBlk - 1) * kBlk + (i % kBlk);
         return start + i;
     };
@@ -383,7 +390,7 @@ __global__ __launch_bounds__(256) void attn_kside_kernel(KSideParams p) {
     // four waves per item: reduce through LDS, wave w finishes channel tile w
     __syncthreads();                                          // everyone is done with the staging area
     f32x4 (*red)[8][kWave] = reinterpret_cast<f32x4 (*)[8][kWave]>(smem_raw);
-    static_assert(sizeof(smem_raw) >= 4 * 8 * kWave * sizeof(f32x4), "reduction buffer must fit the staging area");
+    static_assert(MODE == MODE_FINE || sizeof(smem_raw) >= 4 * 8 * kWave * sizeof(f32x4), "reduction buffer must fit the staging area");
 #pragma unroll
     for (int dt = 0; dt < 4; dt++) {
         red[wave][dt][lane] = dk[dt];
@@ -593,7 +600,7 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     p.n_units = N1; p.w = 1.f;
     if (stages & LLSA_BWD_DKV) {
         const int max_items = N1 * a->T / LLSA_CHUNK_FINE + N1;
-        hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_FINE>), dim3((max_items + 3) / 4, BH), dim3(256), 0, s, p);
+        hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_FINE>), dim3(max_items, BH), dim3(64), 0, s, p);
         ReduceJob& j = rp.job[rp.n_jobs++];
         j.part = p.part; j.off = p.off; j.work = p.work;
         j.dk = p.dk; j.sdkb = p.sdkb; j.sdkh = p.sdkh; j.sdkn = p.sdkn;

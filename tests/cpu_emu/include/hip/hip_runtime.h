@@ -111,6 +111,7 @@ inline int __clz(int x) { return x ? __builtin_clz((unsigned)x) : 32; }
 template <typename F>
 inline hipError_t hipFuncSetAttribute(F, int, int) { return hipSuccess; }
 #define __builtin_amdgcn_readfirstlane(x) (x)
+#define __builtin_amdgcn_readlane(x, l) __shfl((x), (l))
 #define __builtin_nontemporal_store(v, p) (*(p) = (v))
 #define __builtin_nontemporal_load(p) (*(p))
 
