@@ -10,11 +10,11 @@
 // max, running sum, rescale factor) never leave the lane that needs them; a row reduction
 // is two cross-lane steps (lanes l, l^16, l^32, l^48).
 //
-// KV order per query block: T selected 16-token blocks of K/V, then (l2) the 16*T2 level-1
-// pooled tokens inside the parent's selected coarse blocks, then every token of the
-// coarsest pooled level.  Pooled segments count with weight w1 / w2: the accumulator and
-// the running sum are kept in units of the current segment's weight, converted once at
-// each segment boundary.
+// KV order per query block: (l2) the 16*T2 level-1 pooled tokens inside the parent's selected
+// coarse blocks, then every token of the coarsest pooled level, then the T selected 16-token
+// blocks of K/V (the reference walks the same set fine blocks first; the order only moves
+// roundings).  Pooled segments count with weight w1 / w2: the accumulator and the running sum
+// are kept in units of the current segment's weight, converted once at each segment boundary.
 #include "llsa_device.h"
 #include "llsa_host.h"
 #include "../../include/llsa_hip.h"
@@ -99,18 +99,84 @@ __device__ __forceinline__ void compute_step(SoftmaxState& st, const bf16x8 bq[2
             st.acc[dt] = mfma_bf16(cat(t.v[2 * c][dt], t.v[2 * c + 1][dt]), bp[c], st.acc[dt]);
 }
 
-// One wave per query block; the KV list is walked in steps of NB blocks with the loads of
-// step t+1 issued before the arithmetic of step t (two register buffers, ping-pong).
+// Operands of one step out of the workgroup's LDS copy of shared blocks (4 KB per block: R tile
+// of the keys, then T tile of the values).
+template <int NB>
+__device__ __forceinline__ void load_step_lds(KvRegs<NB>& t, const bf16* blocks, int lane) {
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        t.k[j][0] = lds_ld16(blocks + j * 2 * kTile + lane * 8);
+        t.k[j][1] = lds_ld16(blocks + j * 2 * kTile + 512 + lane * 8);
+    }
+#pragma unroll
+    for (int j = 0; j < NB; j++)
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) t.v[j][dt] = lds_ld8(blocks + j * 2 * kTile + kTile + dt * 256 + lane * 4);
+}
+
+constexpr int kGroup = 4;      // shared blocks per LDS buffer
+
+// One wave per query block, four consecutive query blocks per workgroup.
+//
+// The pooled blocks -- the level-1 pooled tokens of the parent's coarse blocks and the coarsest
+// level -- are the same for all query blocks of a 256-token parent, hence for the four waves of
+// the workgroup: they are fetched once per workgroup, kGroup at a time, straight into LDS (two
+// buffers, the next fetch in flight during the arithmetic), and every wave reads its operands
+// from there.  The T fine blocks differ from query block to query block: every wave then walks
+// its own in steps of NB blocks, the loads of step t+1 issued before the arithmetic of step t
+// (two register buffers, ping-pong).  The shared phase comes first because the compiler drains
+// the whole vector-memory queue at every wait while a copy into LDS is outstanding, which would
+// undo the register ping-pong.  This is what bounds the kernel: without the sharing every wave
+// pulls all of its 4 KB per block through the L2, and the L2's bandwidth, not the MFMA, sets the time.
 template <int NB>
 __global__ __launch_bounds__(256) void attn_fwd_kernel(llsa_attn_fwd_args a) {
+    static_assert(NB == 2, "the shared phase reads an LDS buffer as two steps of two blocks");
+    __shared__ __align__(16) bf16 sh[2][kGroup][2 * kTile];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int N1 = a.N / kBlk, N2 = N1 / kBlk;
     const int lid = xcd_logical_id();
-    const int g = (lid % (int)gridDim.x) * 4 + wave;
-    if (g >= N1) return;
+    const int g = (lid % (int)gridDim.x) * 4 + wave;          // < N1: the host checks N1 % 4 == 0
     const int bh = lid / (int)gridDim.x, b = bh / a.H, h = bh % a.H;
     const int r = lane & 15, quad = lane >> 4;
+
+    const bf16* kr = (const bf16*)a.kr + (int64_t)bh * N1 * kTile;
+    const bf16* vt = (const bf16*)a.vt + (int64_t)bh * N1 * kTile;
+    const bf16* pk = (const bf16*)a.pkr + (int64_t)bh * N2 * kTile;
+    const bf16* pvt = (const bf16*)a.pvt + (int64_t)bh * N2 * kTile;
+    const bf16* pk2 = (a.levels == 2) ? (const bf16*)a.pk2r + (int64_t)bh * (N2 / kBlk) * kTile : nullptr;
+    const bf16* pv2t = (a.levels == 2) ? (const bf16*)a.pv2t + (int64_t)bh * (N2 / kBlk) * kTile : nullptr;
+    const int* ip = a.idx + ((int64_t)bh * N1 + g) * a.T;
+    const int* pip = (a.levels == 2) ? a.pidx + ((int64_t)bh * N2 + g / kBlk) * a.T2 : nullptr;
+
+    // shared list: (l2) T2 blocks of level-1 pooled tokens, then every block of the coarsest level
+    const int n_mid = (a.levels == 2) ? a.T2 : 0;
+    const int n_dense = (a.levels == 2) ? N2 / kBlk : N1 / kBlk;
+    const int n_groups = (n_mid + n_dense) / kGroup;          // both are multiples of kGroup (host checks)
+    const int pmine = (a.levels == 2 && lane < a.T2) ? pip[lane] : 0;   // first 64 parent entries, entry i in lane i
+    const bf16* dense_k = (a.levels == 2) ? pk2 : pk;
+    const bf16* dense_vt = (a.levels == 2) ? pv2t : pvt;
+    bf16* const sh0 = &sh[0][0][0];
+    auto issue_group = [=](int grp) __attribute__((always_inline)) {   // this wave brings in block kGroup*grp + wave
+        const int sblk = kGroup * grp + wave;
+        const bf16 *kb, *vb;
+        if (sblk < n_mid) {
+            const int blk = clampi(sblk < kWave ? __builtin_amdgcn_readlane(pmine, sblk) : pip[sblk], 0, N2 - 1);
+            kb = pk + (int64_t)blk * kTile;
+            vb = pvt + (int64_t)blk * kTile;
+        } else {
+            const int u = sblk - n_mid;
+            kb = dense_k + (int64_t)u * kTile;
+            vb = dense_vt + (int64_t)u * kTile;
+        }
+        bf16* dst = sh0 + ((grp & 1) * kGroup + wave) * (2 * kTile);
+        copy16_global_to_lds(kb + lane * 8, dst);
+        copy16_global_to_lds(kb + 512 + lane * 8, dst + 512);
+        copy16_global_to_lds(vb + lane * 8, dst + kTile);
+        copy16_global_to_lds(vb + 512 + lane * 8, dst + kTile + 512);
+    };
+    issue_group(0);
+    int mine = (lane < min(kWave, a.T)) ? ip[lane] : 0;       // first 64 fine indices, entry i in lane i
 
     bf16x8 bq[2];
     {
@@ -124,72 +190,57 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(llsa_attn_fwd_args a) {
 #pragma unroll
     for (int dt = 0; dt < 4; dt++) st.acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const bf16* kr = (const bf16*)a.kr + (int64_t)bh * N1 * kTile;
-    const bf16* vt = (const bf16*)a.vt + (int64_t)bh * N1 * kTile;
-    const bf16* pk = (const bf16*)a.pkr + (int64_t)bh * N2 * kTile;
-    const bf16* pvt = (const bf16*)a.pvt + (int64_t)bh * N2 * kTile;
-    const bf16* pk2 = (a.levels == 2) ? (const bf16*)a.pk2r + (int64_t)bh * (N2 / kBlk) * kTile : nullptr;
-    const bf16* pv2t = (a.levels == 2) ? (const bf16*)a.pv2t + (int64_t)bh * (N2 / kBlk) * kTile : nullptr;
-    const int* ip = a.idx + ((int64_t)bh * N1 + g) * a.T;
-    const int* pip = (a.levels == 2) ? a.pidx + ((int64_t)bh * N2 + g / kBlk) * a.T2 : nullptr;
+    KvRegs<NB> ra, rb;
 
-    // step t of the KV list: fine blocks, then (l2) the parent's level-1 pooled blocks, then
-    // every block of the coarsest pooled level
-    const int n_fine = a.T / NB;
-    const int n_mid = (a.levels == 2) ? a.T2 / NB : 0;
-    const int n_dense = ((a.levels == 2) ? N2 / kBlk : N1 / kBlk) / NB;
-    const int n_steps = n_fine + n_mid + n_dense;
-    const float w_last = (a.levels == 2) ? a.w2 : a.w1;
-    auto describe = [&](int t, StepDesc<NB>& d) {
-        if (t < n_fine) {
+    // ---- shared blocks, out of LDS.  The barrier at the top of round grp says two things: every
+    // wave's part of group grp has landed, and every wave is done reading the other buffer
+    // (group grp - 1), which the next fetch overwrites.
+    const float w_shared_last = (a.levels == 2) ? a.w2 : a.w1;
+    for (int grp = 0; grp < n_groups; grp++) {
+        wait_vm0();
+        __syncthreads();
+        // weight(previous segment) / weight(this one); nothing is accumulated before group 0
+        const float wr = (a.levels == 2 && kGroup * grp == n_mid) ? a.w1 / a.w2 : 1.f;
+        // (LDS reads first: the compiler makes every LDS read wait for all copies into LDS that
+        // were issued before it, which would serialise the next fetch with this round's arithmetic)
+        load_step_lds(ra, &sh[grp & 1][0][0], lane);
+        load_step_lds(rb, &sh[grp & 1][NB][0], lane);
+        if (grp + 1 < n_groups) issue_group(grp + 1);
+        compute_step(st, bq, ra, wr);
+        compute_step(st, bq, rb, 1.f);
+    }
+
+    // ---- fine blocks, private to the wave.  Their indices are fetched 64 at a time, entry i into
+    // lane i, and handed out with readlane (a copy into LDS counts as a store for the compiler,
+    // after which it no longer turns uniform loads into scalar loads; a vector load inside the
+    // pipelined loop would wait for every tile load issued before it).
+    for (int c0 = 0; c0 < a.T; c0 += kWave) {
+        const int cn = min(kWave, a.T - c0);                  // a multiple of 4: an even number of steps
+        if (c0 > 0) mine = (lane < cn) ? ip[c0 + lane] : 0;
+        const int n_fine = cn / NB;
+        auto describe = [=](int t, StepDesc<NB>& d) __attribute__((always_inline)) {
 #pragma unroll
             for (int j = 0; j < NB; j++) {
-                const int blk = clampi(ip[NB * t + j], 0, N1 - 1);
+                const int blk = clampi(__builtin_amdgcn_readlane(mine, NB * t + j), 0, N1 - 1);
                 d.kb[j] = kr + (int64_t)blk * kTile;
                 d.vtb[j] = vt + (int64_t)blk * kTile;
             }
-            d.wratio = 1.f;
-        } else if (t < n_fine + n_mid) {
-            const int u = t - n_fine;
-#pragma unroll
-            for (int j = 0; j < NB; j++) {
-                const int blk = clampi(pip[NB * u + j], 0, N2 - 1);
-                d.kb[j] = pk + (int64_t)blk * kTile;
-                d.vtb[j] = pvt + (int64_t)blk * kTile;
-            }
-            d.wratio = (u == 0) ? 1.f / a.w1 : 1.f;
-        } else {
-            const int u = t - n_fine - n_mid;
-            const bf16* kk = (a.levels == 2) ? pk2 : pk;
-            const bf16* vv = (a.levels == 2) ? pv2t : pvt;
-#pragma unroll
-            for (int j = 0; j < NB; j++) {
-                d.kb[j] = kk + (int64_t)(NB * u + j) * kTile;
-                d.vtb[j] = vv + (int64_t)(NB * u + j) * kTile;
-            }
-            d.wratio = (u == 0) ? ((a.levels == 2) ? a.w1 / a.w2 : 1.f / a.w1) : 1.f;
-        }
-    };
-
-    // The prefetch is unconditional (past the end it re-reads the last step) so that the loop
-    // body is straight-line code: with the loads inside a branch the compiler has to drain the
-    // memory queue (s_waitcnt vmcnt(0)) before every step and the overlap is lost.
-    KvRegs<NB> ra, rb;
-    StepDesc<NB> d;
-    float wa, wb;
-    describe(0, d);
-    load_step(ra, d, lane);
-    wa = d.wratio;
-    for (int t = 0; t < n_steps; t += 2) {
-        describe(min(t + 1, n_steps - 1), d);
-        load_step(rb, d, lane);
-        wb = d.wratio;
-        compute_step(st, bq, ra, wa);
-        if (t + 1 >= n_steps) break;
-        describe(min(t + 2, n_steps - 1), d);
+        };
+        // The prefetch is unconditional (past the end it re-reads the last step) so that the loop
+        // body is straight-line code: with the loads inside a branch the compiler has to drain the
+        // memory queue (s_waitcnt vmcnt(0)) before every step and the overlap is lost.
+        StepDesc<NB> d;
+        describe(0, d);
         load_step(ra, d, lane);
-        wa = d.wratio;
-        compute_step(st, bq, rb, wb);
+        for (int t = 0; t < n_fine; t += 2) {
+            describe(min(t + 1, n_fine - 1), d);
+            load_step(rb, d, lane);
+            compute_step(st, bq, ra, (c0 == 0 && t == 0) ? w_shared_last : 1.f);   // fine tokens weigh 1
+            if (t + 1 >= n_fine) break;
+            describe(min(t + 2, n_fine - 1), d);
+            load_step(ra, d, lane);
+            compute_step(st, bq, rb, 1.f);
+        }
     }
 
     const float L = quad_sum(st.lsum);
@@ -197,7 +248,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(llsa_attn_fwd_args a) {
     bf16* op = (bf16*)a.o + b * a.sob + h * a.soh + (int64_t)(g * kBlk + r) * a.son + quad * 4;
 #pragma unroll
     for (int dt = 0; dt < 4; dt++) st8(op + dt * 16, cvt4(st.acc[dt] * inv));
-    if (quad == 0) a.lse[(int64_t)bh * a.N + g * kBlk + r] = (st.m2 + __builtin_amdgcn_logf(L * w_last)) * kLn2;
+    if (quad == 0) a.lse[(int64_t)bh * a.N + g * kBlk + r] = (st.m2 + __builtin_amdgcn_logf(L)) * kLn2;
 }
 
 }  // namespace llsa

@@ -106,6 +106,24 @@ __device__ __forceinline__ bf16x4 lds_t_operand(const bf16* r_tile_in_lds, int d
     return __builtin_bit_cast(bf16x4, v);
 }
 
+// Asynchronous 16-byte-per-lane copy from global memory straight into LDS (no registers):
+// lane l's 16 bytes land at lds_wave_base + 16*l, so a wave moves 1 KB that is contiguous in
+// LDS.  lds_wave_base must be the same in every lane.  The copy is tracked by the vector-memory
+// counter: wait_vm0() before the data (or a barrier that publishes it) is relied on.
+__device__ __forceinline__ void copy16_global_to_lds(const bf16* g_lane, bf16* lds_wave_base) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)g_lane,
+                                     (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
+}
+__device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0), other counters untouched
+
+// 16- and 8-byte reads that are LDS reads by construction (ds_read_b128 / ds_read_b64)
+__device__ __forceinline__ bf16x8 lds_ld16(const bf16* p) {
+    return *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>((const __attribute__((address_space(3))) bf16*)p);
+}
+__device__ __forceinline__ bf16x4 lds_ld8(const bf16* p) {
+    return *reinterpret_cast<const __attribute__((address_space(3))) bf16x4*>((const __attribute__((address_space(3))) bf16*)p);
+}
+
 // XCD-aware workgroup order.  The 8 XCDs of the chip each have a private L2 and receive
 // workgroups round-robin by linear id (id % 8).  Neighbouring logical work items (query or
 // key blocks that are close in Z-order) read overlapping K/V/Q rows, so they should share an
