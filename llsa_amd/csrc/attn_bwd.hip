@@ -61,61 +61,116 @@ __global__ __launch_bounds__(128) void bwd_pre_kernel(llsa_attn_bwd_args a, floa
 }
 
 // ---------------------------------------------------------------------------------------
-// dQ: one wave per query block, key blocks taken two at a time (32 keys = one MFMA K step)
+// dQ: one wave per query block, four consecutive query blocks per workgroup, key blocks taken
+// two at a time (32 keys = one MFMA K step).
+//
+// K and V always reach the MFMA from R tiles.  K is needed twice: as the A operand of S^T (a plain
+// 16-byte read per lane) and, read back with the transposing LDS load, as the A operand of
+// dQ^T += K^T.dS^T -- so K goes through LDS in any case, copied there straight from global memory.
+//  * pooled blocks (level-1 pooled tokens of the parent's coarse blocks, the coarsest level) are
+//    the same for the four query blocks of the workgroup: one copy per workgroup, kGroup blocks
+//    of K and V at a time, two buffers;
+//  * fine blocks are private: afterwards each wave re-uses a quarter of the same LDS as two slots
+//    for the K tiles of a pair (the copy of pair t+1 in flight during pair t), V stays in registers.
 // ---------------------------------------------------------------------------------------
-// kb / vb: R tiles of K and V for the two key blocks of the pair.  K is the A operand of S^T from
-// the registers and, parked in the wave's LDS `stage` (2048 elements) and read back transposed,
-// the A operand of dQ^T += K^T.dS^T.
-__device__ __forceinline__ void dq_pair(f32x4 dq[4], const bf16x8 bq[2], const bf16x8 bdo[2], float lse2, float delta,
-                                        float w, const bf16* const kb[2], const bf16* const vb[2], bf16* stage,
-                                        int lane) {
-    bf16x8 kreg[2][2], vreg[2][2];
+struct PairR {
+    bf16x8 k[2][2], v[2][2];       // block j, channel half
+};
+struct PairT {
+    bf16x4 t[2][4];                // block j, channel tile dt
+};
+
+__device__ __forceinline__ void read_k_r(PairR& o, const bf16* k0, const bf16* k1, int lane) {
+    o.k[0][0] = lds_ld16(k0 + lane * 8);
+    o.k[0][1] = lds_ld16(k0 + 512 + lane * 8);
+    o.k[1][0] = lds_ld16(k1 + lane * 8);
+    o.k[1][1] = lds_ld16(k1 + 512 + lane * 8);
+}
+__device__ __forceinline__ void read_v_r(PairR& o, const bf16* v0, const bf16* v1, int lane) {
+    o.v[0][0] = lds_ld16(v0 + lane * 8);
+    o.v[0][1] = lds_ld16(v0 + 512 + lane * 8);
+    o.v[1][0] = lds_ld16(v1 + lane * 8);
+    o.v[1][1] = lds_ld16(v1 + 512 + lane * 8);
+}
+__device__ __forceinline__ void read_k_t(PairT& o, const bf16* k0, const bf16* k1, int lane) {
 #pragma unroll
-    for (int j = 0; j < 2; j++) {
-        kreg[j][0] = ld16(kb[j] + lane * 8);
-        kreg[j][1] = ld16(kb[j] + 512 + lane * 8);
-        vreg[j][0] = ld16(vb[j] + lane * 8);
-        vreg[j][1] = ld16(vb[j] + 512 + lane * 8);
+    for (int dt = 0; dt < 4; dt++) {
+        o.t[0][dt] = lds_t_operand(k0, dt, lane);
+        o.t[1][dt] = lds_t_operand(k1, dt, lane);
     }
-#pragma unroll
-    for (int j = 0; j < 2; j++) {
-        st16(stage + j * kTile + lane * 8, kreg[j][0]);
-        st16(stage + j * kTile + 512 + lane * 8, kreg[j][1]);
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
+}
+// dS^T of a pair of key blocks, as the B operand of the dQ product
+__device__ __forceinline__ bf16x8 dq_scores(const PairR& p, const bf16x8 bq[2], const bf16x8 bdo[2], float lse2,
+                                            float delta, float w) {
     bf16x8 bds;
 #pragma unroll
     for (int j = 0; j < 2; j++) {
         f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
-        s = mfma_bf16(kreg[j][0], bq[0], s);
-        s = mfma_bf16(kreg[j][1], bq[1], s);
-        dp = mfma_bf16(vreg[j][0], bdo[0], dp);
-        dp = mfma_bf16(vreg[j][1], bdo[1], dp);
+        s = mfma_bf16(p.k[j][0], bq[0], s);
+        s = mfma_bf16(p.k[j][1], bq[1], s);
+        dp = mfma_bf16(p.v[j][0], bdo[0], dp);
+        dp = mfma_bf16(p.v[j][1], bdo[1], dp);
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            const float p = exp2_fast(fmaf(s[e], kScaleLog2e, -lse2)) * w;
-            bds[j * 4 + e] = (bf16)(p * (dp[e] - delta));
+            const float pe = exp2_fast(fmaf(s[e], kScaleLog2e, -lse2)) * w;
+            bds[j * 4 + e] = (bf16)(pe * (dp[e] - delta));
         }
     }
+    return bds;
+}
+__device__ __forceinline__ void dq_accum(f32x4 dq[4], const PairT& p, bf16x8 bds) {
 #pragma unroll
-    for (int dt = 0; dt < 4; dt++)
-        dq[dt] = mfma_bf16(cat(lds_t_operand(stage, dt, lane), lds_t_operand(stage + kTile, dt, lane)), bds, dq[dt]);
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_wave_barrier();              // the next pair overwrites `stage`
+    for (int dt = 0; dt < 4; dt++) dq[dt] = mfma_bf16(cat(p.t[0][dt], p.t[1][dt]), bds, dq[dt]);
 }
 
 __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, const float* __restrict__ delta,
                                                       const bf16* __restrict__ dor) {
+    __shared__ __align__(16) bf16 sh[2][kGroup][2 * kTile];   // per block: R tile of K, R tile of V
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int N1 = a.N / kBlk, N2 = N1 / kBlk;
     const int lid = xcd_logical_id();
-    const int g = (lid % (int)gridDim.x) * 4 + wave;
-    if (g >= N1) return;
+    const int g = (lid % (int)gridDim.x) * 4 + wave;          // < N1: the host checks N1 % 4 == 0
     const int bh = lid / (int)gridDim.x, b = bh / a.H, h = bh % a.H;
     const int r = lane & 15, quad = lane >> 4;
     const int tok = g * kBlk + r;
+
+    const bf16* kr = (const bf16*)a.kr + (int64_t)bh * N1 * kTile;
+    const bf16* vr = (const bf16*)a.vr + (int64_t)bh * N1 * kTile;
+    const bf16* pk = (const bf16*)a.pkr + (int64_t)bh * N2 * kTile;
+    const bf16* pv = (const bf16*)a.pvr + (int64_t)bh * N2 * kTile;
+    const int* ip = a.idx + ((int64_t)bh * N1 + g) * a.T;
+    const int* pip = (a.levels == 2) ? a.pidx + ((int64_t)bh * N2 + g / kBlk) * a.T2 : nullptr;
+
+    // shared list: (l2) T2 blocks of level-1 pooled tokens, then every block of the coarsest level
+    const int n_mid = (a.levels == 2) ? a.T2 : 0;
+    const int n_dense = (a.levels == 2) ? N2 / kBlk : N1 / kBlk;
+    const int n_groups = (n_mid + n_dense) / kGroup;
+    const int pmine = (a.levels == 2 && lane < a.T2) ? pip[lane] : 0;   // first 64 parent entries, entry i in lane i
+    const bf16* dense_k = (a.levels == 2) ? (const bf16*)a.pk2r + (int64_t)bh * (N2 / kBlk) * kTile : pk;
+    const bf16* dense_v = (a.levels == 2) ? (const bf16*)a.pv2r + (int64_t)bh * (N2 / kBlk) * kTile : pv;
+    const float w_dense = (a.levels == 2) ? a.w2 : a.w1;
+    bf16* const sh0 = &sh[0][0][0];
+    auto issue_group = [=](int grp) __attribute__((always_inline)) {   // this wave brings in block kGroup*grp + wave
+        const int sblk = kGroup * grp + wave;
+        const bf16 *kb, *vb;
+        if (sblk < n_mid) {
+            const int blk = clampi(sblk < kWave ? __builtin_amdgcn_readlane(pmine, sblk) : pip[sblk], 0, N2 - 1);
+            kb = pk + (int64_t)blk * kTile;
+            vb = pv + (int64_t)blk * kTile;
+        } else {
+            const int u = sblk - n_mid;
+            kb = dense_k + (int64_t)u * kTile;
+            vb = dense_v + (int64_t)u * kTile;
+        }
+        bf16* dst = sh0 + ((grp & 1) * kGroup + wave) * (2 * kTile);
+        copy16_global_to_lds(kb + lane * 8, dst);
+        copy16_global_to_lds(kb + 512 + lane * 8, dst + 512);
+        copy16_global_to_lds(vb + lane * 8, dst + kTile);
+        copy16_global_to_lds(vb + 512 + lane * 8, dst + kTile + 512);
+    };
+    issue_group(0);
+    int mine = (lane < min(kWave, a.T)) ? ip[lane] : 0;       // first 64 fine indices, entry i in lane i
 
     bf16x8 bq[2], bdo[2];
     {
@@ -132,53 +187,67 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, cons
 #pragma unroll
     for (int dt = 0; dt < 4; dt++) dq[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const bf16* kr = (const bf16*)a.kr + (int64_t)bh * N1 * kTile;
-    const bf16* vr = (const bf16*)a.vr + (int64_t)bh * N1 * kTile;
-    const bf16* pk = (const bf16*)a.pkr + (int64_t)bh * N2 * kTile;
-    const bf16* pv = (const bf16*)a.pvr + (int64_t)bh * N2 * kTile;
-    const bf16 *kb[2], *vb[2];
-    __shared__ __align__(16) bf16 stage_all[4][2 * kTile];
-    bf16* stage = stage_all[wave];
-
-    const int* ip = a.idx + ((int64_t)bh * N1 + g) * a.T;
-    for (int t = 0; t < a.T / 2; t++) {
-#pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const int blk = clampi(ip[2 * t + j], 0, N1 - 1);
-            kb[j] = kr + (int64_t)blk * kTile;
-            vb[j] = vr + (int64_t)blk * kTile;
-        }
-        dq_pair(dq, bq, bdo, lse2, dl, 1.f, kb, vb, stage, lane);
+    // ---- pooled blocks out of the shared copy.  The barrier at the top of round grp says: every
+    // wave's part of group grp has landed, and every wave is done reading the other buffer.  All
+    // LDS reads of a round come before the next fetch is issued (the compiler makes an LDS read
+    // wait for every copy into LDS issued before it).
+    for (int grp = 0; grp < n_groups; grp++) {
+        wait_vm0();
+        __syncthreads();
+        const float w = (kGroup * grp < n_mid) ? a.w1 : w_dense;
+        const bf16* blk = sh0 + (grp & 1) * kGroup * (2 * kTile);
+        PairR r0, r1;
+        PairT t0, t1;
+        read_k_r(r0, blk, blk + 2 * kTile, lane);
+        read_v_r(r0, blk + kTile, blk + 3 * kTile, lane);
+        read_k_t(t0, blk, blk + 2 * kTile, lane);
+        const bf16x8 ds0 = dq_scores(r0, bq, bdo, lse2, dl, w);
+        read_k_r(r1, blk + 4 * kTile, blk + 6 * kTile, lane);
+        read_v_r(r1, blk + 5 * kTile, blk + 7 * kTile, lane);
+        read_k_t(t1, blk + 4 * kTile, blk + 6 * kTile, lane);
+        if (grp + 1 < n_groups) issue_group(grp + 1);
+        dq_accum(dq, t0, ds0);
+        const bf16x8 ds1 = dq_scores(r1, bq, bdo, lse2, dl, w);
+        dq_accum(dq, t1, ds1);
     }
-    if (a.levels == 2) {
-        const int* pip = a.pidx + ((int64_t)bh * N2 + g / kBlk) * a.T2;
-        for (int t = 0; t < a.T2 / 2; t++) {
+    __syncthreads();                                          // the shared copy is dead: its LDS becomes private slots
+
+    // ---- fine blocks: K of pair t+1 is copied into the wave's other slot and V of pair t+1 loaded
+    // into registers while pair t is worked on.  Nothing may be in flight when the wave ends (a copy
+    // landing in LDS that already belongs to another workgroup), so the last pair fetches nothing.
+    bf16* const priv = sh0 + wave * (4 * kTile);              // two slots of two K tiles
+    for (int c0 = 0; c0 < a.T; c0 += kWave) {
+        const int cn = min(kWave, a.T - c0);
+        if (c0 > 0) mine = (lane < cn) ? ip[c0 + lane] : 0;
+        const int n_pairs = cn / 2;
+        PairR ra, rb;
+        auto fetch = [=](int t, PairR& dst) __attribute__((always_inline)) {
+            bf16* slot = priv + (t & 1) * (2 * kTile);
 #pragma unroll
             for (int j = 0; j < 2; j++) {
-                const int blk = clampi(pip[2 * t + j], 0, N2 - 1);
-                kb[j] = pk + (int64_t)blk * kTile;
-                vb[j] = pv + (int64_t)blk * kTile;
+                const int blk = clampi(__builtin_amdgcn_readlane(mine, 2 * t + j), 0, N1 - 1);
+                const bf16* kb = kr + (int64_t)blk * kTile;
+                const bf16* vb = vr + (int64_t)blk * kTile;
+                copy16_global_to_lds(kb + lane * 8, slot + j * kTile);
+                copy16_global_to_lds(kb + 512 + lane * 8, slot + j * kTile + 512);
+                dst.v[j][0] = ld16(vb + lane * 8);
+                dst.v[j][1] = ld16(vb + 512 + lane * 8);
             }
-            dq_pair(dq, bq, bdo, lse2, dl, a.w1, kb, vb, stage, lane);
-        }
-        const bf16* pk2 = (const bf16*)a.pk2r + (int64_t)bh * (N2 / kBlk) * kTile;
-        const bf16* pv2 = (const bf16*)a.pv2r + (int64_t)bh * (N2 / kBlk) * kTile;
-        for (int t = 0; t < N2 / 32; t++) {
-#pragma unroll
-            for (int j = 0; j < 2; j++) {
-                kb[j] = pk2 + (int64_t)(2 * t + j) * kTile;
-                vb[j] = pv2 + (int64_t)(2 * t + j) * kTile;
-            }
-            dq_pair(dq, bq, bdo, lse2, dl, a.w2, kb, vb, stage, lane);
-        }
-    } else {
-        for (int t = 0; t < N1 / 32; t++) {
-#pragma unroll
-            for (int j = 0; j < 2; j++) {
-                kb[j] = pk + (int64_t)(2 * t + j) * kTile;
-                vb[j] = pv + (int64_t)(2 * t + j) * kTile;
-            }
-            dq_pair(dq, bq, bdo, lse2, dl, a.w1, kb, vb, stage, lane);
+        };
+        auto work = [&](int t, PairR& cur, PairR& nxt) __attribute__((always_inline)) {
+            wait_vm0();
+            const bf16* slot = priv + (t & 1) * (2 * kTile);
+            PairT tt;
+            read_k_r(cur, slot, slot + kTile, lane);
+            read_k_t(tt, slot, slot + kTile, lane);
+            if (t + 1 < n_pairs) fetch(t + 1, nxt);
+            const bf16x8 ds = dq_scores(cur, bq, bdo, lse2, dl, 1.f);
+            dq_accum(dq, tt, ds);
+        };
+        fetch(0, ra);
+        for (int t = 0; t < n_pairs; t += 2) {                // n_pairs is even (T % 4 == 0)
+            work(t, ra, rb);
+            work(t + 1, rb, ra);
         }
     }
 

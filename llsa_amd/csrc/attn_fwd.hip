@@ -114,8 +114,6 @@ __device__ __forceinline__ void load_step_lds(KvRegs<NB>& t, const bf16* blocks,
         for (int dt = 0; dt < 4; dt++) t.v[j][dt] = lds_ld8(blocks + j * 2 * kTile + kTile + dt * 256 + lane * 4);
 }
 
-constexpr int kGroup = 4;      // shared blocks per LDS buffer
-
 // One wave per query block, four consecutive query blocks per workgroup.
 //
 // The pooled blocks -- the level-1 pooled tokens of the parent's coarse blocks and the coarsest

@@ -116,6 +116,8 @@ __device__ __forceinline__ void copy16_global_to_lds(const bf16* g_lane, bf16* l
 }
 __device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0), other counters untouched
 
+constexpr int kGroup = 4;      // pooled blocks per LDS buffer in the query-side attention kernels (one per wave)
+
 // 16- and 8-byte reads that are LDS reads by construction (ds_read_b128 / ds_read_b64)
 __device__ __forceinline__ bf16x8 lds_ld16(const bf16* p) {
     return *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>((const __attribute__((address_space(3))) bf16*)p);
