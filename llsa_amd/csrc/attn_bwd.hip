@@ -196,19 +196,17 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, cons
         __syncthreads();
         const float w = (kGroup * grp < n_mid) ? a.w1 : w_dense;
         const bf16* blk = sh0 + (grp & 1) * kGroup * (2 * kTile);
-        PairR r0, r1;
-        PairT t0, t1;
+        PairR r0;
+        PairT t0;
         read_k_r(r0, blk, blk + 2 * kTile, lane);
         read_v_r(r0, blk + kTile, blk + 3 * kTile, lane);
         read_k_t(t0, blk, blk + 2 * kTile, lane);
-        const bf16x8 ds0 = dq_scores(r0, bq, bdo, lse2, dl, w);
-        read_k_r(r1, blk + 4 * kTile, blk + 6 * kTile, lane);
-        read_v_r(r1, blk + 5 * kTile, blk + 7 * kTile, lane);
-        read_k_t(t1, blk + 4 * kTile, blk + 6 * kTile, lane);
+        dq_accum(dq, t0, dq_scores(r0, bq, bdo, lse2, dl, w));
+        read_k_r(r0, blk + 4 * kTile, blk + 6 * kTile, lane);
+        read_v_r(r0, blk + 5 * kTile, blk + 7 * kTile, lane);
+        read_k_t(t0, blk + 4 * kTile, blk + 6 * kTile, lane);
         if (grp + 1 < n_groups) issue_group(grp + 1);
-        dq_accum(dq, t0, ds0);
-        const bf16x8 ds1 = dq_scores(r1, bq, bdo, lse2, dl, w);
-        dq_accum(dq, t1, ds1);
+        dq_accum(dq, t0, dq_scores(r0, bq, bdo, lse2, dl, w));
     }
     __syncthreads();                                          // the shared copy is dead: its LDS becomes private slots
 
@@ -366,7 +364,10 @@ __global__ __launch_bounds__(MODE == MODE_FINE ? 64 : 256) void attn_kside_kerne
     // Others: four waves per work item.
     constexpr int W = (MODE == MODE_FINE) ? 1 : 4;            // waves per work item = waves per workgroup
     // per wave 2 query blocks x {Q, dO} R tiles; reused for the cross-wave reduction
-    __shared__ __align__(16) unsigned char smem_raw[W * 4 * kTile * sizeof(bf16)];
+#ifndef KS_PAD
+#define KS_PAD 1
+#endif
+    __shared__ __align__(16) unsigned char smem_raw[KS_PAD * W * 4 * kTile * sizeof(bf16)];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int N1 = p.N / kBlk;
