@@ -78,8 +78,9 @@ def stage_profile(op, q, k, v, do, t1, t2, freq, iters, torch):
     """Runs the kernels of one forward + backward one stage at a time, the same launches the
     fused operator makes, and times each stage with events on the launch stream."""
     from llsa_amd.kernel.hip import _attention as A
+    from llsa_amd._lib import CHUNK_COARSE, CHUNK_FINE
     from llsa_amd.kernel.hip.indices_transpose import transpose_indices
-    from llsa_amd.kernel.hip.mean_pool import PoolSpec, pool_bwd_accum, pool_pyramid
+    from llsa_amd.kernel.hip.mean_pool import PoolSpec, pool_pyramid
     from llsa_amd.kernel.hip.topk import compute_topk_indices_sparse, gen_sparse_indices
     B, H, N, D = q.shape
     l2 = op == "l2"
@@ -117,25 +118,23 @@ def stage_profile(op, q, k, v, do, t1, t2, freq, iters, torch):
     res["attn_fwd"] = timed(lambda: A.attn_fwd(q, k, v, pk, pv, idx, 16.0, tiles=tiles, **kw), iters, torch)
 
     def transposes():
-        r = transpose_indices(idx, N // 16, 32)
-        return r + transpose_indices(pidx, N // 256, 8) if l2 else r
+        r = transpose_indices(idx, N // 16, CHUNK_FINE)
+        return r + transpose_indices(pidx, N // 256, CHUNK_COARSE) if l2 else r
 
     csr = transposes()
     res["transpose_indices"] = timed(transposes, iters, torch)
     bkw = dict(kw, tiles=tiles, csr=csr)
-    run = lambda st, f=None: A.attn_bwd(do, q, k, v, pk, pv, o, lse, idx, 16.0, cgw, stages=st, freq_dq=f, **bkw)
-    run(1)
-    for name, st in (("bwd_delta_dOt", 1), ("bwd_dq", 2), ("bwd_dkv", 4), ("bwd_dpkv1_sparse", 8), ("bwd_dpkv_dense", 16)):
+    # as the fused operator calls it: pooled gradients folded into dk / dv by the fine pass
+    run = lambda st: A.attn_bwd(do, q, k, v, pk, pv, o, lse, idx, 16.0, cgw, stages=st, freq_dq=freq, fold_pooled=True,
+                                freq_dk=freq, **bkw)
+    run(2)
+    for name, st in (("bwd_dq", 2), ("bwd_dpkv1_sparse", 8), ("bwd_dpkv_dense", 16), ("bwd_dkv", 4)):
         if st == 8 and not l2:
             continue
-        # a stage run alone reads whatever workspace the allocator hands back (the block stage 1
-        # just filled); only its duration is used
-        res[name] = timed(lambda: run(st, freq if st == 2 else None), iters, torch)
-    outs = run(0, freq)
-    dk, dv, dpk, dpv = outs[1], outs[2], outs[3], outs[4]
-    dpk2, dpv2 = (outs[5], outs[6]) if l2 else (None, None)
-    res["pool_bwd_accum"] = timed(lambda: (pool_bwd_accum(dk, dpk, dpk2, freq), pool_bwd_accum(dv, dpv, dpv2, None)),
-                                  iters, torch)
+        # a stage run alone reads whatever workspace the allocator hands back (the block the dq stage
+        # just filled with delta and the dO tiles); only its duration is used.  The K-side stages
+        # include the reduction of their partial sums.
+        res[name] = timed(lambda: run(st), iters, torch)
     return res
 
 
@@ -257,10 +256,9 @@ def main():
         else:
             alg["bwd_dpkv_dense"] = 4.0 * B * H * N * D * (N // 16)
         el = 2 * B * H * N * D
-        hbm = {"pool_pyramid": 3 * el * (1 + 1 / 16 + (1 / 256 if op == "l2" else 0)),
-               "pool_bwd_accum": 2 * 2 * el, "bwd_delta_dOt": 2 * el + 4 * B * H * N}
-        # (the pooling and delta kernels also write the operand tiles the attention kernels read;
-        # those bytes are layout work of this implementation and are not counted as algorithmic)
+        hbm = {"pool_pyramid": 3 * el * (1 + 1 / 16 + (1 / 256 if op == "l2" else 0))}
+        # (the pooling kernel also writes the operand tiles the attention kernels read; those bytes
+        # are layout work of this implementation and are not counted as algorithmic)
         kernels = {}
         for name, t in st.items():
             e = {"ms": t}

@@ -149,7 +149,7 @@ int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, 
  * (B,H,llsa_work_list_len(Mb,Kb,T,chunk)) int32; llsa_attn_bwd needs chunk = LLSA_CHUNK_FINE
  * for idx and chunk = LLSA_CHUNK_COARSE for pidx. */
 int64_t llsa_work_list_len(int Mb, int Kb, int T, int chunk);
-#define LLSA_CHUNK_FINE 32
+#define LLSA_CHUNK_FINE 64
 #define LLSA_CHUNK_COARSE 8
 
 /* ------------------------------------------------------------------------------------------
@@ -178,14 +178,21 @@ typedef struct llsa_attn_bwd_args {
     void* dpk2; void* dpv2;                      /* (B,H,N/256,64) contiguous out (levels == 2)   */
     void* workspace; int64_t workspace_bytes;    /* see llsa_attn_bwd_workspace_bytes             */
     const void* freq_dq;                         /* (N,64) or NULL: rotate dq back (fused rope)   */
+    const void* freq_dk;                         /* (N,64) or NULL: rotate dk back; needs fold_pooled */
     int32_t B, H, N, T, T2, levels;
     float w1, w2, cgw1;
     int32_t stages;                              /* 0 = everything; else a mask of LLSA_BWD_* to
                                                     launch only those kernels (profiling)        */
+    int32_t fold_pooled;                         /* 0: dk, dv are the fine-token gradients only, as the
+                                                    reference's kernels return them (mean_pool1d's backward
+                                                    and autograd add dpk.. afterwards).  1: dk, dv also
+                                                    receive the pooled gradients of their blocks, with the
+                                                    same bf16 roundings (= llsa_pool_bwd_accum), and dk is
+                                                    rotated back with freq_dk                          */
 } llsa_attn_bwd_args;
 
-#define LLSA_BWD_PRE 1      /* delta + block-transposed dO (everything below needs it)           */
-#define LLSA_BWD_DQ 2
+#define LLSA_BWD_DQ 2       /* dq; also delta = rowsum(o * dout) and the R tiles of dout, which the
+                               stages below read from the workspace                              */
 #define LLSA_BWD_DKV 4      /* dK/dV of the fine tokens                                          */
 #define LLSA_BWD_DPKV1 8    /* sparse level-1 pooled gradients (levels == 2)                     */
 #define LLSA_BWD_DENSE 16   /* dense coarsest pooled gradients (partials + reduction)            */

@@ -49,9 +49,9 @@ class AttnBwdArgs(C.Structure):
            ("dk", c_void_p), ("sdkb", c_int64), ("sdkh", c_int64), ("sdkn", c_int64),
            ("dv", c_void_p), ("sdvb", c_int64), ("sdvh", c_int64), ("sdvn", c_int64)]
         + [("dpk", c_void_p), ("dpv", c_void_p), ("dpk2", c_void_p), ("dpv2", c_void_p),
-           ("workspace", c_void_p), ("workspace_bytes", c_int64), ("freq_dq", c_void_p),
+           ("workspace", c_void_p), ("workspace_bytes", c_int64), ("freq_dq", c_void_p), ("freq_dk", c_void_p),
            ("B", c_int32), ("H", c_int32), ("N", c_int32), ("T", c_int32), ("T2", c_int32), ("levels", c_int32),
-           ("w1", c_float), ("w2", c_float), ("cgw1", c_float), ("stages", c_int32)])
+           ("w1", c_float), ("w2", c_float), ("cgw1", c_float), ("stages", c_int32), ("fold_pooled", c_int32)])
 
 
 P64 = C.POINTER(c_int64)
@@ -75,7 +75,7 @@ _SIGNATURES = {
 }
 
 EXPORTS = tuple(_SIGNATURES)
-CHUNK_FINE, CHUNK_COARSE = 32, 8          # LLSA_CHUNK_FINE / LLSA_CHUNK_COARSE of include/llsa_hip.h
+CHUNK_FINE, CHUNK_COARSE = 64, 8          # LLSA_CHUNK_FINE / LLSA_CHUNK_COARSE of include/llsa_hip.h
 
 
 class LlsaError(RuntimeError):

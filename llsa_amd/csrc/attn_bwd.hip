@@ -19,48 +19,6 @@
 namespace llsa {
 
 // ---------------------------------------------------------------------------------------
-// delta = rowsum(O * dO) in fp32, and the R operand tiles of dO.
-// Same thread mapping as the pooling kernel: 16 blocks x 8 channel chunks per workgroup.
-// ---------------------------------------------------------------------------------------
-__global__ __launch_bounds__(128) void bwd_pre_kernel(llsa_attn_bwd_args a, float* __restrict__ delta,
-                                                      bf16* __restrict__ dor) {
-    const int N1 = a.N / kBlk;
-    const int bh = blockIdx.y, b = bh / a.H, h = bh % a.H;
-    const int t = threadIdx.x, c = t & 7, r = t >> 3;
-    const int blk = blockIdx.x * 16 + r;
-    if (blk >= N1) return;                      // no barrier below
-    const bf16* op = (const bf16*)a.o + b * a.sob + h * a.soh + (int64_t)blk * kBlk * a.son + c * 8;
-    const bf16* gp = (const bf16*)a.dout + b * a.sdob + h * a.sdoh + (int64_t)blk * kBlk * a.sdon + c * 8;
-    bf16x8 gv[16];
-    float part[16];
-#pragma unroll
-    for (int i = 0; i < 16; i++) {
-        gv[i] = ld16(gp + i * a.sdon);
-        const bf16x8 ov = ld16(op + i * a.son);
-        float s = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; e++) s += (float)ov[e] * (float)gv[i][e];
-        part[i] = s;
-    }
-#pragma unroll
-    for (int i = 0; i < 16; i++) {
-        float s = part[i];
-        s += __shfl_xor(s, 1);
-        s += __shfl_xor(s, 2);
-        s += __shfl_xor(s, 4);
-        part[i] = s;
-    }
-    if (c == 0) {
-        float* dp = delta + (int64_t)bh * a.N + blk * kBlk;
-#pragma unroll
-        for (int i = 0; i < 16; i++) dp[i] = part[i];
-    }
-    bf16* xr = dor + ((int64_t)bh * N1 + blk) * kTile + c * 128;
-#pragma unroll
-    for (int i = 0; i < 16; i++) st16(xr + i * 8, gv[i]);
-}
-
-// ---------------------------------------------------------------------------------------
 // dQ: one wave per query block, four consecutive query blocks per workgroup, key blocks taken
 // two at a time (32 keys = one MFMA K step).
 //
@@ -123,8 +81,8 @@ __device__ __forceinline__ void dq_accum(f32x4 dq[4], const PairT& p, bf16x8 bds
     for (int dt = 0; dt < 4; dt++) dq[dt] = mfma_bf16(cat(p.t[0][dt], p.t[1][dt]), bds, dq[dt]);
 }
 
-__global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, const float* __restrict__ delta,
-                                                      const bf16* __restrict__ dor) {
+__global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, float* __restrict__ delta,
+                                                      bf16* __restrict__ dor) {
     __shared__ __align__(16) bf16 sh[2][kGroup][2 * kTile];   // per block: R tile of K, R tile of V
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -172,17 +130,33 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, cons
     issue_group(0);
     int mine = (lane < min(kWave, a.T)) ? ip[lane] : 0;       // first 64 fine indices, entry i in lane i
 
+    // dO comes straight from the caller's tensor, already in the register layout of an R operand
+    // (lane l: row l%16, channels 8*(l/16)..+7 and 32 + 8*(l/16)..+7).  The wave also does the
+    // pre-pass the K-side kernels need: delta = rowsum(O * dO) in fp32 (the reference sums in the
+    // tensor dtype, sparse_attention_res_1.py:153-177) and dO as an R tile.
     bf16x8 bq[2], bdo[2];
+    float dl;
     {
         const bf16* qp = (const bf16*)a.qr + ((int64_t)bh * N1 + g) * kTile + lane * 8;
-        const bf16* gp = dor + ((int64_t)bh * N1 + g) * kTile + lane * 8;
         bq[0] = ld16(qp);
         bq[1] = ld16(qp + 512);
+        const bf16* gp = (const bf16*)a.dout + b * a.sdob + h * a.sdoh + (int64_t)tok * a.sdon + quad * 8;
+        const bf16* op = (const bf16*)a.o + b * a.sob + h * a.soh + (int64_t)tok * a.son + quad * 8;
         bdo[0] = ld16(gp);
-        bdo[1] = ld16(gp + 512);
+        bdo[1] = ld16(gp + 32);
+        const bf16x8 o0 = ld16(op), o1 = ld16(op + 32);
+        float acc = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc += (float)o0[e] * (float)bdo[0][e];
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc += (float)o1[e] * (float)bdo[1][e];
+        dl = quad_sum(acc);
+        bf16* tile = dor + ((int64_t)bh * N1 + g) * kTile + lane * 8;
+        st16(tile, bdo[0]);
+        st16(tile + 512, bdo[1]);
+        if (quad == 0) delta[(int64_t)bh * a.N + tok] = dl;
     }
     const float lse2 = a.lse[(int64_t)bh * a.N + tok] * kLog2e;
-    const float dl = delta[(int64_t)bh * a.N + tok];
     f32x4 dq[4];
 #pragma unroll
     for (int dt = 0; dt < 4; dt++) dq[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -254,19 +228,7 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, cons
 #pragma unroll
     for (int dt = 0; dt < 4; dt++) {
         bf16x4 o = cvt4(dq[dt] * kScale);
-        if (fq != nullptr) {                    // rotate the gradient back: [sin, cos] pairs
-#pragma clang fp contract(off)
-            const bf16x4 f = ld8(fq + dt * 16);
-            bf16x4 y;
-#pragma unroll
-            for (int j = 0; j < 2; j++) {
-                const float s = (float)f[2 * j], c = (float)f[2 * j + 1];
-                const float ge = (float)o[2 * j], go = (float)o[2 * j + 1];
-                y[2 * j] = (bf16)(rn_bf16(c * ge) + rn_bf16(s * go));
-                y[2 * j + 1] = (bf16)(rn_bf16(-s * ge) + rn_bf16(c * go));
-            }
-            o = y;
-        }
+        if (fq != nullptr) o = rope_bwd4(o, ld8(fq + dt * 16));   // rotate the gradient back
         st8(op + dt * 16, o);
     }
 }
@@ -277,6 +239,41 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, cons
 // blocks; the unit's waves walk the list two query blocks at a time.
 // ---------------------------------------------------------------------------------------
 enum { MODE_FINE = 0, MODE_SPARSE1 = 1, MODE_DENSE = 2 };
+
+// Optional last step of the fine dK / dV: add the pooled gradients the token's block received
+// (what the backward of the two mean pools and autograd's accumulation do in the reference:
+// every sum and every division by 16 rounded to bf16) and rotate dK back through the RoPE.
+struct PoolFold {
+    const bf16* g1k; const bf16* g1v;             // level-1 pooled gradients (BH, N/16, 64); nullptr: no folding
+    const bf16* g2k; const bf16* g2v;             // level-2 pooled gradients (BH, N/256, 64) or nullptr
+    const bf16* freq;                             // (N, 64) or nullptr
+};
+// x: four channels of one token; g / gg: the same channels of its block's level-1 / level-2 pooled
+// gradient; f: their [sin, cos] entries.  Mirrors pool_bwd_accum_kernel.
+__device__ __forceinline__ bf16x4 fold_math(bf16x4 x, bf16x4 g, bool has_gg, bf16x4 gg, bool has_f, bf16x4 f) {
+#pragma clang fp contract(off)
+    if (has_gg) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) g[e] = (bf16)((float)g[e] + rn_bf16((float)gg[e] * 0.0625f));
+    }
+#pragma unroll
+    for (int e = 0; e < 4; e++) x[e] = (bf16)((float)x[e] + rn_bf16((float)g[e] * 0.0625f));
+    return has_f ? rope_bwd4(x, f) : x;
+}
+// x: channels c0..c0+3 of token `tok` of (b,h) `bh`; which = 0 for dK, 1 for dV
+__device__ __forceinline__ bf16x4 fold_pooled(bf16x4 x, const PoolFold& f, int which, int64_t bh, int N, int tok, int c0) {
+    const bf16* g1 = which ? f.g1v : f.g1k;
+    const bf16* g2 = which ? f.g2v : f.g2k;
+    const int N1 = N / kBlk;
+    const bf16x4 g = ld8(g1 + (bh * N1 + tok / kBlk) * kD + c0);
+    bf16x4 gg = g, fr = g;
+    if (g2 != nullptr) gg = ld8(g2 + (bh * (N1 / kBlk) + tok / (kBlk * kBlk)) * kD + c0);
+    const bool rot = which == 0 && f.freq != nullptr;
+    if (rot) fr = ld8(f.freq + (int64_t)tok * kD + c0);
+    return fold_math(x, g, g2 != nullptr, gg, rot, fr);
+}
+constexpr int kFoldRows = 4 * kD;                 // LDS copy of a unit's fold operands: 4 pooled rows, then 16 freq rows
+constexpr int kFoldElems = kFoldRows + kBlk * kD;
 
 struct KSideParams {
     const bf16* qr;  const bf16* dor;             // R tiles of q and dO, (BH, N1, 1024)
@@ -292,6 +289,7 @@ struct KSideParams {
     int64_t work_stride;                          // ints of `work` per (b,h)
     int64_t slot_stride;                          // partial slots per (b,h)
     float w;
+    PoolFold fold;                                // FINE only
 };
 
 // Two query blocks (g0, g1; g1 < 0: only one) against the unit's 16 key rows.  Q and dO are
@@ -364,10 +362,8 @@ __global__ __launch_bounds__(MODE == MODE_FINE ? 64 : 256) void attn_kside_kerne
     // Others: four waves per work item.
     constexpr int W = (MODE == MODE_FINE) ? 1 : 4;            // waves per work item = waves per workgroup
     // per wave 2 query blocks x {Q, dO} R tiles; reused for the cross-wave reduction
-#ifndef KS_PAD
-#define KS_PAD 1
-#endif
-    __shared__ __align__(16) unsigned char smem_raw[KS_PAD * W * 4 * kTile * sizeof(bf16)];
+    __shared__ __align__(16) unsigned char smem_raw[W * 4 * kTile * sizeof(bf16)];
+    __shared__ __align__(16) bf16 fold_buf[MODE == MODE_FINE ? kFoldElems : 8];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int N1 = p.N / kBlk;
@@ -401,6 +397,23 @@ __global__ __launch_bounds__(MODE == MODE_FINE ? 64 : 256) void attn_kside_kerne
         const int sb = work[4 + unit];
         if (sb >= 0) slot = (int64_t)bh * p.slot_stride + sb + ci;
         fl = p.flat + (int64_t)bh * p.flat_stride;
+    }
+    // What the fold on the way out needs (the unit's pooled-gradient rows, its tokens' RoPE entries)
+    // is copied into LDS now, without registers, so that no load waits at the end of the wave.
+    const bool folding = MODE == MODE_FINE && p.fold.g1k != nullptr && slot < 0;
+    if (folding) {
+        const int row = lane >> 3, piece = lane & 7;          // rows: dpk, dpv, dpk2, dpv2 of the unit; 8 x 16 bytes each
+        const bool two = p.fold.g2k != nullptr;
+        if (lane < (two ? 32 : 16)) {
+            const bf16* src = (row & 1) ? ((row & 2) ? p.fold.g2v : p.fold.g1v) : ((row & 2) ? p.fold.g2k : p.fold.g1k);
+            src += ((int64_t)bh * ((row & 2) ? N1 / kBlk : N1) + ((row & 2) ? unit / kBlk : unit)) * kD;
+            copy16_global_to_lds(src + piece * 8, fold_buf);
+        }
+        if (p.fold.freq != nullptr) {
+            const bf16* fr = p.fold.freq + (int64_t)unit * kBlk * kD;
+            copy16_global_to_lds(fr + lane * 8, fold_buf + kFoldRows);
+            copy16_global_to_lds(fr + 512 + lane * 8, fold_buf + kFoldRows + 512);
+        }
     }
     // The item's list entries (FINE: at most 32 query blocks) are fetched once, entry i into
     // lane i, and handed out with readlane: the walk below then has no load that depends on a load.
@@ -450,10 +463,19 @@ __global__ __launch_bounds__(MODE == MODE_FINE ? 64 : 256) void attn_kside_kerne
         }
         bf16* kp = p.dk + b * p.sdkb + h * p.sdkh + (int64_t)(unit * kBlk + r) * p.sdkn + quad * 4;
         bf16* vp = p.dv + b * p.sdvb + h * p.sdvh + (int64_t)(unit * kBlk + r) * p.sdvn + quad * 4;
+        if (folding) wait_vm0();                              // the copies into fold_buf (long since done)
 #pragma unroll
         for (int dt = 0; dt < 4; dt++) {
-            st8(kp + dt * 16, cvt4(dk[dt] * kScale));
-            st8(vp + dt * 16, cvt4(dv[dt]));
+            bf16x4 ok = cvt4(dk[dt] * kScale), ov = cvt4(dv[dt]);
+            if (folding) {
+                const int c0 = dt * 16 + quad * 4;
+                const bool two = p.fold.g2k != nullptr, rot = p.fold.freq != nullptr;
+                ok = fold_math(ok, lds_ld8(fold_buf + c0), two, lds_ld8(fold_buf + 2 * kD + c0), rot,
+                               lds_ld8(fold_buf + kFoldRows + r * kD + c0));
+                ov = fold_math(ov, lds_ld8(fold_buf + kD + c0), two, lds_ld8(fold_buf + 3 * kD + c0), false, ov);
+            }
+            st8(kp + dt * 16, ok);
+            st8(vp + dt * 16, ov);
         }
         return;
     }
@@ -498,60 +520,83 @@ struct ReduceJob {
     int n_units, chunk, max_units;       // max_units: upper bound of units this job can have per (b,h)
     int64_t work_stride, slot_stride;
     int n_chunks;            // dense job: partials per unit, at stride BH * n_units slots
+    PoolFold fold;           // fine job only
 };
 struct ReduceParams {
     ReduceJob job[3];
-    int n_jobs, H;
+    int n_jobs, H, N;
 };
 
+constexpr int kReduceSlots = 256;    // unit positions per job and (b,h) that are walked in parallel
+__host__ __device__ inline int reduce_slots(int max_units) { return max_units < kReduceSlots ? max_units : kReduceSlots; }
+
 __global__ __launch_bounds__(256) void kside_reduce_kernel(ReduceParams rp) {
-    // two workgroups per unit; every thread owns one f32x4 of the unit's 8 x 64 accumulator
-    // registers and streams that position of all partials, eight loads in flight
+    // Two workgroups per unit; every thread owns one f32x4 of the unit's 8 x 64 accumulator
+    // registers and streams that position of all partials, sixteen loads in flight.  Every job has
+    // its own range of workgroup pairs (reduce_slots of them), which walk the job's units with that
+    // stride: the number of units with several pieces is known only on the device and usually
+    // small, and a grid sized for the worst case would be mostly workgroups that start, look and leave.
     const int bh = blockIdx.y, b = bh / rp.H, h = bh % rp.H;
     const int pos = (blockIdx.x & 1) * 256 + threadIdx.x;
     const int reg = pos >> 6, lane = pos & 63;
     const int r = lane & 15, quad = lane >> 4;
-    int u = blockIdx.x >> 1, j = 0;
-    while (j < rp.n_jobs && u >= rp.job[j].max_units) {
-        u -= rp.job[j].max_units;
+    const int dt = reg & 3;
+    const int which = reg >> 2;                               // 0: dK, 1: dV
+    int u0 = blockIdx.x >> 1, j = 0;
+    while (j < rp.n_jobs && u0 >= reduce_slots(rp.job[j].max_units)) {
+        u0 -= reduce_slots(rp.job[j].max_units);
         j++;
     }
     if (j >= rp.n_jobs) return;
     const ReduceJob& jb = rp.job[j];
-    int unit, n;
-    int64_t first, stride;
-    if (jb.work != nullptr) {
-        const int* work = jb.work + (int64_t)bh * jb.work_stride;
-        if (u >= work[2]) return;
-        const int max_items = (int)(jb.work_stride - 4 - jb.n_units - jb.max_units);
-        unit = work[4 + jb.n_units + max_items + u];
-        const int* o = jb.off + (int64_t)bh * (jb.n_units + 1) + unit;
-        n = (o[1] - o[0] + jb.chunk - 1) / jb.chunk;
-        first = (int64_t)bh * jb.slot_stride + work[4 + unit];
-        stride = 1;
-    } else {
-        unit = u;
-        n = jb.n_chunks;
-        first = (int64_t)bh * jb.n_units + unit;
-        stride = (int64_t)gridDim.y * jb.n_units;
+    const int step = reduce_slots(jb.max_units);
+    const int* work = jb.work ? jb.work + (int64_t)bh * jb.work_stride : nullptr;
+    const int max_items = (int)(jb.work_stride - 4 - jb.n_units - 4 * jb.max_units);
+    // the unit's record is fetched together with the count it is checked against (u0 is always
+    // inside the list's storage): one memory round trip instead of two
+    const int* multi = work ? work + 4 + jb.n_units + max_items : nullptr;
+    int rec_unit = 0, rec_first = 0, rec_n = 0;
+    if (work != nullptr) {
+        rec_unit = multi[4 * u0];
+        rec_first = multi[4 * u0 + 1];
+        rec_n = multi[4 * u0 + 2];
     }
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    const f32x4* ps = jb.part + first * (8 * kWave) + reg * kWave + lane;
-    for (int c0 = 0; c0 < n; c0 += 8) {
-        f32x4 v[8];
+    const int count = work ? min(work[2], jb.max_units) : jb.n_units;
+    for (int u = u0; u < count; u += step) {
+        int unit, n;
+        int64_t first, stride;
+        if (work != nullptr) {
+            if (u != u0) {
+                rec_unit = multi[4 * u];
+                rec_first = multi[4 * u + 1];
+                rec_n = multi[4 * u + 2];
+            }
+            unit = rec_unit;
+            n = rec_n;
+            first = (int64_t)bh * jb.slot_stride + rec_first;
+            stride = 1;
+        } else {
+            unit = u;
+            n = jb.n_chunks;
+            first = (int64_t)bh * jb.n_units + unit;
+            stride = (int64_t)gridDim.y * jb.n_units;
+        }
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+        const f32x4* ps = jb.part + first * (8 * kWave) + reg * kWave + lane;
+        for (int c0 = 0; c0 < n; c0 += 16) {
+            f32x4 v[16];
 #pragma unroll
-        for (int k = 0; k < 8; k++) v[k] = ps[(int64_t)min(c0 + k, n - 1) * stride * (8 * kWave)];
+            for (int k = 0; k < 16; k++) v[k] = ps[(int64_t)min(c0 + k, n - 1) * stride * (8 * kWave)];
 #pragma unroll
-        for (int k = 0; k < 8; k++)
-            if (c0 + k < n) acc += v[k];                       // chunk order: the sum does not depend on scheduling
-    }
-    const int dt = reg & 3;
-    if (reg < 4) {
-        bf16* kp = jb.dk + b * jb.sdkb + h * jb.sdkh + (int64_t)(unit * kBlk + r) * jb.sdkn + quad * 4;
-        st8(kp + dt * 16, cvt4(acc * kScale));
-    } else {
-        bf16* vp = jb.dv + b * jb.sdvb + h * jb.sdvh + (int64_t)(unit * kBlk + r) * jb.sdvn + quad * 4;
-        st8(vp + dt * 16, cvt4(acc));
+            for (int k = 0; k < 16; k++)
+                if (c0 + k < n) acc += v[k];                   // chunk order: the sum does not depend on scheduling
+        }
+        bf16x4 out = cvt4(which ? acc : acc * kScale);
+        if (jb.fold.g1k != nullptr)
+            out = fold_pooled(out, jb.fold, which, bh, rp.N, unit * kBlk + r, dt * 16 + quad * 4);
+        bf16* dst = which ? jb.dv + b * jb.sdvb + h * jb.sdvh + (int64_t)(unit * kBlk + r) * jb.sdvn
+                          : jb.dk + b * jb.sdkb + h * jb.sdkh + (int64_t)(unit * kBlk + r) * jb.sdkn;
+        st8(dst + quad * 4 + dt * 16, out);
     }
 }
 
@@ -646,43 +691,61 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     char* ws = (char*)a->workspace;
     float* delta = (float*)(ws + wsp.delta);
     bf16* dor = (bf16*)(ws + wsp.dor);
+    const bool fold = a->fold_pooled != 0;
+    LLSA_REQUIRE(fold || a->freq_dk == nullptr, "attn_bwd: freq_dk needs fold_pooled");
 
     const int stages = a->stages ? a->stages : 0x7fffffff;
-    if (stages & LLSA_BWD_PRE) hipLaunchKernelGGL(bwd_pre_kernel, dim3((N1 + 15) / 16, BH), dim3(128), 0, s, *a, delta, dor);
     if (stages & LLSA_BWD_DQ)
-        hipLaunchKernelGGL(attn_dq_kernel, dim3((N1 + 3) / 4, BH), dim3(256), 0, s, *a, (const float*)delta, (const bf16*)dor);
+        hipLaunchKernelGGL(attn_dq_kernel, dim3((N1 + 3) / 4, BH), dim3(256), 0, s, *a, delta, dor);
 
     ReduceParams rp;
     rp.n_jobs = 0;
     rp.H = H;
-    KSideParams p;
-    p.qr = (const bf16*)a->qr; p.dor = dor;
-    p.lse = a->lse; p.delta = delta;
-    p.H = H; p.N = N; p.chunk_len = 0;
-
-    // fine K/V blocks
-    p.kk = (const bf16*)a->kr; p.vv = (const bf16*)a->vr;
-    p.off = a->off; p.flat = a->flat; p.flat_stride = (int64_t)N1 * a->T;
-    p.work = a->work; p.work_stride = llsa_work_list_len(N1, N1, a->T, LLSA_CHUNK_FINE);
-    p.part = (f32x4*)(ws + wsp.part_fine); p.slot_stride = wsp.slots_fine;
-    p.dk = (bf16*)a->dk; p.sdkb = a->sdkb; p.sdkh = a->sdkh; p.sdkn = a->sdkn;
-    p.dv = (bf16*)a->dv; p.sdvb = a->sdvb; p.sdvh = a->sdvh; p.sdvn = a->sdvn;
-    p.n_units = N1; p.w = 1.f;
-    if (stages & LLSA_BWD_DKV) {
-        const int max_items = N1 * a->T / LLSA_CHUNK_FINE + N1;
-        hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_FINE>), dim3(max_items, BH), dim3(64), 0, s, p);
+    rp.N = N;
+    auto add_job = [&](const KSideParams& p, int chunk, int max_units, int n_chunks) {
         ReduceJob& j = rp.job[rp.n_jobs++];
         j.part = p.part; j.off = p.off; j.work = p.work;
         j.dk = p.dk; j.sdkb = p.sdkb; j.sdkh = p.sdkh; j.sdkn = p.sdkn;
         j.dv = p.dv; j.sdvb = p.sdvb; j.sdvh = p.sdvh; j.sdvn = p.sdvn;
-        j.n_units = N1; j.chunk = LLSA_CHUNK_FINE; j.max_units = N1 * a->T / LLSA_CHUNK_FINE + 1;
-        j.work_stride = p.work_stride; j.slot_stride = p.slot_stride; j.n_chunks = 0;
-    }
-
+        j.n_units = p.n_units; j.chunk = chunk; j.max_units = max_units;
+        j.work_stride = p.work_stride; j.slot_stride = p.slot_stride; j.n_chunks = n_chunks;
+        j.fold = p.fold;
+    };
+    auto run_reduce = [&]() {
+        if (rp.n_jobs == 0) return;
+        int slots = 0;
+        for (int i = 0; i < rp.n_jobs; i++) slots += reduce_slots(rp.job[i].max_units);
+        hipLaunchKernelGGL(kside_reduce_kernel, dim3(slots * 2, BH), dim3(256), 0, s, rp);
+        rp.n_jobs = 0;
+    };
+    KSideParams base;
+    base.qr = (const bf16*)a->qr; base.dor = dor;
+    base.lse = a->lse; base.delta = delta;
+    base.H = H; base.N = N; base.chunk_len = 0;
+    base.fold = PoolFold{nullptr, nullptr, nullptr, nullptr, nullptr};
     const int64_t s1b = (int64_t)H * N1 * 64, s1h = (int64_t)N1 * 64;
     const int64_t s2b = (int64_t)H * N2 * 64, s2h = (int64_t)N2 * 64;
-    if (a->levels == 2 && (stages & LLSA_BWD_DPKV1)) {
-        // level-1 pooled tokens, through the transposed coarse index
+
+    auto run_fine = [&]() {                                   // dK / dV of the fine tokens
+        if (!(stages & LLSA_BWD_DKV)) return;
+        KSideParams p = base;
+        p.kk = (const bf16*)a->kr; p.vv = (const bf16*)a->vr;
+        p.off = a->off; p.flat = a->flat; p.flat_stride = (int64_t)N1 * a->T;
+        p.work = a->work; p.work_stride = llsa_work_list_len(N1, N1, a->T, LLSA_CHUNK_FINE);
+        p.part = (f32x4*)(ws + wsp.part_fine); p.slot_stride = wsp.slots_fine;
+        p.dk = (bf16*)a->dk; p.sdkb = a->sdkb; p.sdkh = a->sdkh; p.sdkn = a->sdkn;
+        p.dv = (bf16*)a->dv; p.sdvb = a->sdvb; p.sdvh = a->sdvh; p.sdvn = a->sdvn;
+        p.n_units = N1; p.w = 1.f;
+        if (fold)
+            p.fold = PoolFold{(const bf16*)a->dpk, (const bf16*)a->dpv, (a->levels == 2) ? (const bf16*)a->dpk2 : nullptr,
+                              (a->levels == 2) ? (const bf16*)a->dpv2 : nullptr, (const bf16*)a->freq_dk};
+        const int max_items = N1 * a->T / LLSA_CHUNK_FINE + N1;
+        hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_FINE>), dim3(max_items, BH), dim3(64), 0, s, p);
+        add_job(p, LLSA_CHUNK_FINE, N1 * a->T / LLSA_CHUNK_FINE + 1, 0);
+    };
+    auto run_sparse1 = [&]() {                                // level-1 pooled tokens, through the transposed coarse index
+        if (a->levels != 2 || !(stages & LLSA_BWD_DPKV1)) return;
+        KSideParams p = base;
         p.kk = (const bf16*)a->pkr; p.vv = (const bf16*)a->pvr;
         p.off = a->poff; p.flat = a->pflat; p.flat_stride = (int64_t)N2 * a->T2;
         p.work = a->pwork; p.work_stride = llsa_work_list_len(N2, N2, a->T2, LLSA_CHUNK_COARSE);
@@ -692,42 +755,44 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
         p.n_units = N2; p.w = a->cgw1;
         const int max_items = N2 * a->T2 / LLSA_CHUNK_COARSE + N2;
         hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_SPARSE1>), dim3(max_items, BH), dim3(256), 0, s, p);
-        ReduceJob& j = rp.job[rp.n_jobs++];
-        j.part = p.part; j.off = p.off; j.work = p.work;
-        j.dk = p.dk; j.sdkb = p.sdkb; j.sdkh = p.sdkh; j.sdkn = p.sdkn;
-        j.dv = p.dv; j.sdvb = p.sdvb; j.sdvh = p.sdvh; j.sdvn = p.sdvn;
-        j.n_units = N2; j.chunk = LLSA_CHUNK_COARSE; j.max_units = N2 * a->T2 / LLSA_CHUNK_COARSE + 1;
-        j.work_stride = p.work_stride; j.slot_stride = p.slot_stride; j.n_chunks = 0;
-    }
+        add_job(p, LLSA_CHUNK_COARSE, N2 * a->T2 / LLSA_CHUNK_COARSE + 1, 0);
+    };
     // dense coarsest level: every unit (16 pooled tokens) meets every query block; the query
     // range is cut into d.chunks pieces whose partial sums are added afterwards
-    if (stages & LLSA_BWD_DENSE) {
-    if (a->levels == 2) {
-        p.kk = (const bf16*)a->pk2r; p.vv = (const bf16*)a->pv2r;
-        p.dk = (bf16*)a->dpk2; p.dv = (bf16*)a->dpv2;
-        p.sdkb = p.sdvb = s2b; p.sdkh = p.sdvh = s2h;
-        p.w = a->w2;
+    auto run_dense = [&]() {
+        if (!(stages & LLSA_BWD_DENSE)) return;
+        KSideParams p = base;
+        if (a->levels == 2) {
+            p.kk = (const bf16*)a->pk2r; p.vv = (const bf16*)a->pv2r;
+            p.dk = (bf16*)a->dpk2; p.dv = (bf16*)a->dpv2;
+            p.sdkb = p.sdvb = s2b; p.sdkh = p.sdvh = s2h;
+            p.w = a->w2;
+        } else {
+            p.kk = (const bf16*)a->pkr; p.vv = (const bf16*)a->pvr;
+            p.dk = (bf16*)a->dpk; p.dv = (bf16*)a->dpv;
+            p.sdkb = p.sdvb = s1b; p.sdkh = p.sdvh = s1h;
+            p.w = a->cgw1;
+        }
+        p.sdkn = p.sdvn = 64;
+        p.off = nullptr; p.flat = nullptr; p.flat_stride = 0; p.work = nullptr; p.work_stride = 0; p.slot_stride = 0;
+        p.part = (f32x4*)(ws + wsp.part_dense);
+        p.n_units = d.n_tok / 16; p.chunk_len = d.chunk_len;
+        hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_DENSE>), dim3(p.n_units, BH, d.chunks), dim3(256), 0, s, p);
+        add_job(p, 1, p.n_units, d.chunks);
+    };
+
+    if (fold) {
+        // the fine pass adds the finished pooled gradients on its way out, so they come first
+        run_sparse1();
+        run_dense();
+        run_reduce();
+        run_fine();
+        run_reduce();
     } else {
-        p.kk = (const bf16*)a->pkr; p.vv = (const bf16*)a->pvr;
-        p.dk = (bf16*)a->dpk; p.dv = (bf16*)a->dpv;
-        p.sdkb = p.sdvb = s1b; p.sdkh = p.sdvh = s1h;
-        p.w = a->cgw1;
-    }
-    p.sdkn = p.sdvn = 64;
-    p.off = nullptr; p.flat = nullptr; p.flat_stride = 0; p.work = nullptr; p.work_stride = 0; p.slot_stride = 0;
-    p.part = (f32x4*)(ws + wsp.part_dense);
-    p.n_units = d.n_tok / 16; p.chunk_len = d.chunk_len;
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_DENSE>), dim3(p.n_units, BH, d.chunks), dim3(256), 0, s, p);
-    ReduceJob& j = rp.job[rp.n_jobs++];
-    j.part = p.part; j.off = nullptr; j.work = nullptr;
-    j.dk = p.dk; j.sdkb = p.sdkb; j.sdkh = p.sdkh; j.sdkn = p.sdkn;
-    j.dv = p.dv; j.sdvb = p.sdvb; j.sdvh = p.sdvh; j.sdvn = p.sdvn;
-    j.n_units = p.n_units; j.chunk = 1; j.max_units = p.n_units; j.work_stride = 0; j.slot_stride = 0; j.n_chunks = d.chunks;
-    }
-    if (rp.n_jobs > 0) {
-        int total = 0;
-        for (int i = 0; i < rp.n_jobs; i++) total += rp.job[i].max_units;
-        hipLaunchKernelGGL(kside_reduce_kernel, dim3(total * 2, BH), dim3(256), 0, s, rp);
+        run_fine();
+        run_sparse1();
+        run_dense();
+        run_reduce();
     }
     return launch_status("attn_bwd");
 }

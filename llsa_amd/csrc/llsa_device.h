@@ -116,6 +116,21 @@ __device__ __forceinline__ void copy16_global_to_lds(const bf16* g_lane, bf16* l
 }
 __device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0), other counters untouched
 
+// Rotates a gradient back through the 2-D RoPE: 4 consecutive channels = two (even, odd) pairs, f
+// holds their [sin, cos] entries.  Every product and sum is rounded to bf16 like the forward rotation.
+__device__ __forceinline__ bf16x4 rope_bwd4(bf16x4 o, bf16x4 f) {
+#pragma clang fp contract(off)
+    bf16x4 y;
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const float s = (float)f[2 * j], c = (float)f[2 * j + 1];
+        const float ge = (float)o[2 * j], go = (float)o[2 * j + 1];
+        y[2 * j] = (bf16)(rn_bf16(c * ge) + rn_bf16(s * go));
+        y[2 * j + 1] = (bf16)(rn_bf16(-s * ge) + rn_bf16(c * go));
+    }
+    return y;
+}
+
 constexpr int kGroup = 4;      // pooled blocks per LDS buffer in the query-side attention kernels (one per wave)
 
 // 16- and 8-byte reads that are LDS reads by construction (ds_read_b128 / ds_read_b64)

@@ -28,7 +28,8 @@ __device__ __forceinline__ int wave_incl_scan(int v, int lane) {
 //   blocks with more than one chunk, work[3] unused,
 //   work[4 + n] = first slot of key block n, or -1 when n has one chunk,
 //   work[4 + Kb + i] = item i = (n << 16) | chunk index   (items of one key block are adjacent),
-//   work[4 + Kb + max_items + j] = j-th key block with more than one chunk
+//   work[4 + Kb + max_items + 4j .. +3] = j-th key block with more than one chunk: {n, first slot,
+//   number of chunks, 0} (16-byte aligned when the list itself is: one load tells the reduction all)
 // Every key block has at least one item (an unselected block's item has no entries and only
 // writes zeros), and max_items = Mb*T/chunk + Kb.
 __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int* __restrict__ idx, int* __restrict__ offsets,
@@ -91,7 +92,13 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
             const int nch = max(1, (c + chunk - 1) / chunk);
             work[4 + i] = (nch > 1) ? run_s : -1;
             for (int ci = 0; ci < nch; ci++) work[4 + Kb + run_i + ci] = (i << 16) | ci;
-            if (nch > 1) work[4 + Kb + max_items + run_m++] = i;
+            if (nch > 1) {
+                int* m = work + 4 + Kb + max_items + 4 * run_m++;
+                m[0] = i;
+                m[1] = run_s;
+                m[2] = nch;
+                m[3] = 0;
+            }
             run_i += nch;
             run_s += (nch > 1) ? nch : 0;
         }
@@ -157,7 +164,7 @@ using namespace llsa;
 extern "C" int64_t llsa_work_list_len(int Mb, int Kb, int T, int chunk) {
     if (Mb <= 0 || Kb <= 0 || T <= 0 || chunk <= 0) return -1;
     const int64_t e = (int64_t)Mb * T;
-    return 4 + (int64_t)Kb + (e / chunk + Kb) + (e / chunk + 1);
+    return 4 + (int64_t)Kb + (e / chunk + Kb) + 4 * (e / chunk + 1);
 }
 
 extern "C" int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, int32_t* work, int B, int H, int Mb,

@@ -88,10 +88,11 @@ def rows_ok8(t):
 
 def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_weight, pk2=None, pv2=None,
              p_indices=None, token_weight_2=1.0, tiles=None, freq_dq: Optional[torch.Tensor] = None, stages: int = 0,
-             csr=None):
+             csr=None, fold_pooled: bool = False, freq_dk: Optional[torch.Tensor] = None):
     """Backward.  Returns (dq, dk, dv, dpk, dpv[, dpk2, dpv2]) with the reference's conventions:
     every gradient is `empty_like` of its primal; the pooled gradients are NOT yet folded
-    into dk / dv (autograd, or pool_bwd_accum, does that).  `tiles` may carry operand tiles the
+    into dk / dv (autograd, or pool_bwd_accum, does that) unless `fold_pooled` is set, in which case
+    the fine pass adds them on its way out (same roundings) and rotates dk back with `freq_dk`.  `tiles` may carry operand tiles the
     caller already has (qr, kr, vr, pkr, pvr, pk2r, pv2r).  `stages` (a mask of
     the LLSA_BWD_* bits of include/llsa_hip.h) launches only some of the kernels, for profiling."""
     levels = 1 if pk2 is None else 2
@@ -151,6 +152,11 @@ def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_wei
         a.freq_dq = freq_dq.data_ptr()
     a.B, a.H, a.N, a.T, a.T2, a.levels = B, H, N, T, T2, levels
     a.w1, a.w2, a.cgw1 = float(token_weight), float(token_weight_2), float(coarse_grad_weight)
+    if freq_dk is not None:
+        require_bf16(freq_dk)
+        freq_dk = freq_dk.contiguous()
+        a.freq_dk = freq_dk.data_ptr()
     a.stages = stages
+    a.fold_pooled = int(bool(fold_pooled))
     lib.check(lib.attn_bwd(C.byref(a), stream_of(lib, q)), "attn_bwd")
     return tuple(outs)

@@ -12,7 +12,7 @@ from __future__ import annotations
 import torch
 from torch.autograd import Function
 
-from ..hip.mean_pool import PoolSpec, mean_pool1d, pool_bwd_accum, pool_pyramid
+from ..hip.mean_pool import PoolSpec, mean_pool1d, pool_pyramid
 from ..hip.sparse_attention_res_1 import sparse_indices_attn_res_fwd, sparse_indices_attn_res_scatter_bwd_v2
 from ..hip.topk import gen_sparse_indices
 
@@ -73,9 +73,8 @@ class _LlsaL1Fused(Function):
         bs = ctx.block_size
         tiles = dict(qr=qr, kr=kr, vr=vr, pkr=pkr, pvr=pvr)
         dq, dk, dv, _, dpk, dpv = sparse_indices_attn_res_scatter_bwd_v2(
-            do, q, k, v, pk, pv, o, m, indices, indices.shape[-1], bs, bs, tiles=tiles, freq_dq=freq)
-        dk = pool_bwd_accum(dk, dpk, None, freq, out=dk)
-        dv = pool_bwd_accum(dv, dpv, None, None, out=dv)
+            do, q, k, v, pk, pv, o, m, indices, indices.shape[-1], bs, bs, tiles=tiles, freq_dq=freq,
+            fold_pooled=True, freq_dk=freq)       # dk, dv arrive with the pooled gradients folded in
         return dq, dk, dv, None, None, None
 
 

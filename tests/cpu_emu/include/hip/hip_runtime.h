@@ -108,7 +108,8 @@ inline int __clz(int x) { return x ? __builtin_clz((unsigned)x) : 32; }
 #define __builtin_amdgcn_wave_barrier() emu::wave_sync()
 #define __builtin_amdgcn_global_load_lds(g, l, size, off, aux) \
     __builtin_memcpy((char*)(l) + (size) * emu::lane_id(), (const char*)(g), (size))
-#define __builtin_amdgcn_s_waitcnt(x) ((void)0)
+// the wave-wide effect of a wait (all lanes' copies into LDS have landed) needs a rendezvous of the lanes here
+#define __builtin_amdgcn_s_waitcnt(x) emu::wave_sync()
 #define __builtin_amdgcn_fence(order, scope) ((void)0)
 #define hipFuncAttributeMaxDynamicSharedMemorySize 0
 template <typename F>

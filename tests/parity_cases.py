@@ -242,6 +242,8 @@ def check_attn_l1(dev, B=1, H=2, N=1024, T=8, strided=False, smooth=False, weigh
     ref = O.attn_bwd_l1(doc, qc, kc, vc, pk, pv, o.cpu(), lse.cpu(), idx, weight)
     for name, a, b in zip(("dq", "dk", "dv", "dpk", "dpv"), got, ref):
         close(name, a, b)
+    _check_fold(dev, got, lambda **kw: attn_bwd(do, q, k, v, pk.to(dev), pv.to(dev), o, lse, idx.int().to(dev), weight, 1.0,
+                                                **kw), N)
 
 
 def check_attn_l2(dev, B=1, H=1, N=16384, T=8, T2=4, smooth=False, hot=None):
@@ -266,6 +268,25 @@ def check_attn_l2(dev, B=1, H=1, N=16384, T=8, T2=4, smooth=False, hot=None):
     ref = O.attn_bwd_l2(doc, qc, kc, vc, pk, pv, pk2, pv2, o.cpu(), lse.cpu(), idx, pidx)
     for name, a, b in zip(("dq", "dk", "dv", "dpk", "dpv", "dpk2", "dpv2"), got, ref):
         close(name, a, b)
+    _check_fold(dev, got, lambda **kw: attn_bwd(do, q, k, v, d(pk), d(pv), o, lse, d(idx), 16.0, 16.0, pk2=d(pk2), pv2=d(pv2),
+                                                p_indices=d(pidx.int()), token_weight_2=256.0, **kw), N)
+
+
+def _check_fold(dev, plain, run, N):
+    """fold_pooled=True must give, bit for bit, what pool_bwd_accum makes of the unfolded outputs
+    (with the same RoPE rotate-back of dk), and leave the other outputs unchanged."""
+    import math
+    from llsa_amd.kernel.hip.mean_pool import pool_bwd_accum
+    side = 1 << math.ceil(math.log2(N) / 2)                   # any (N, 64) sin/cos table will do here
+    freq = O.rope_table(side, dtype=torch.bfloat16)[:N].contiguous().to(dev)
+    folded = run(fold_pooled=True, freq_dk=freq)
+    dpk2, dpv2 = (plain[5], plain[6]) if len(plain) > 5 else (None, None)
+    want_dk = pool_bwd_accum(plain[1], plain[3], dpk2, freq)
+    want_dv = pool_bwd_accum(plain[2], plain[4], dpv2, None)
+    assert torch.equal(folded[1].cpu(), want_dk.cpu()), "folded dk differs from pool_bwd_accum"
+    assert torch.equal(folded[2].cpu(), want_dv.cpu()), "folded dv differs from pool_bwd_accum"
+    for i in (0,) + tuple(range(3, len(plain))):
+        assert torch.equal(folded[i].cpu(), plain[i].cpu()), f"output {i} changed with fold_pooled"
 
 
 def check_attn_reduces_to_sdpa(dev, B=1, H=2, N=1024):
