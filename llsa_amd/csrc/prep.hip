@@ -52,14 +52,37 @@ struct PoolParams {
     int H;
 };
 
+// The operand tiles of the workgroup's 16 blocks are one contiguous 32 KB piece of the tile
+// array.  A thread's registers hold 256-byte pieces of it that are 256 bytes apart from its
+// neighbours' (R) or 8-byte pieces scattered over a whole tile (T); stored straight from the
+// registers every store instruction would touch 64 different cache lines with 16 or 8 bytes
+// each.  They go through LDS instead (16-byte units, block stride 136 units, padded so that both
+// sides spread over the banks) and leave as full-width stores: thread t of the workgroup writes
+// the 16 bytes at (k * 128 + t) * 16 for k = 0..15.
+constexpr int kStageBlk = 136;                    // 16-byte units per block in the staging buffer (128 + padding)
+
+__device__ __forceinline__ void stage_out(bf16* stage, bf16* tiles32k, int t, int n_valid_blocks, bool r_layout) {
+    __syncthreads();                              // the staging buffer is filled
+#pragma unroll
+    for (int k = 0; k < 16; k++) {
+        if (k < n_valid_blocks) {
+            const int u = r_layout ? (t >> 4) * 17 + (t & 15) : t + (t >> 4);
+            st16(tiles32k + (k * 128 + t) * 8, ld16(stage + (k * kStageBlk + u) * 8));
+        }
+    }
+    __syncthreads();                              // and may be refilled
+}
+
 __global__ __launch_bounds__(128) void pool_pyramid_kernel(PoolParams p) {
+    __shared__ __align__(16) bf16 stage[16 * kStageBlk * 8];
     const llsa_pool_item& it = p.it[blockIdx.z];
     const int n1 = it.n / kBlk;
-    if ((int)blockIdx.x * 16 >= n1) return;
+    if ((int)blockIdx.x * 16 >= n1) return;       // uniform over the workgroup
     const int bh = blockIdx.y, b = bh / p.H, h = bh % p.H;
     const int t = threadIdx.x, c = t & 7, r = t >> 3;
     const int blk = blockIdx.x * 16 + r;
     const bool valid = blk < n1;
+    const int n_valid = min(16, n1 - (int)blockIdx.x * 16);
 
     bf16x8 xv[16];
     bf16x8 y = zero8();
@@ -89,28 +112,36 @@ __global__ __launch_bounds__(128) void pool_pyramid_kernel(PoolParams p) {
             for (int e = 0; e < 8; e++) y[e] = (bf16)(acc[e] * 0.0625f);
             if (it.y1 != nullptr) st16((bf16*)it.y1 + ((int64_t)bh * n1 + blk) * kD + c * 8, y);
         }
-        if (it.xr != nullptr) {          // R tile: chunk c of row i at (c * 16 + i) * 8
-            bf16* xr = (bf16*)it.xr + ((int64_t)bh * n1 + blk) * kTile + c * 128;
+    }
+    if (it.xr != nullptr) {              // R tile: chunk c of row i is 16-byte unit c * 16 + i of the block
+        if (valid) {
 #pragma unroll
-            for (int i = 0; i < 16; i++) st16(xr + i * 8, xv[i]);
+            for (int i = 0; i < 16; i++) st16(stage + (r * kStageBlk + c * 17 + i) * 8, xv[i]);
         }
-        if (it.xt != nullptr) {          // T tile: channel 8c+e, tokens 4q..4q+3 at t_tile_off(4q, 8c+e)
-            bf16* xt = (bf16*)it.xt + ((int64_t)bh * n1 + blk) * kTile;
+        stage_out(stage, (bf16*)it.xr + ((int64_t)bh * n1 + blockIdx.x * 16) * kTile, t, n_valid, true);
+    }
+    if (it.xt != nullptr) {              // T tile: channels 8c+e, 8c+e+1 of tokens 4q..4q+3 are one 16-byte unit
+        if (valid) {
 #pragma unroll
-            for (int e = 0; e < 8; e++)
+            for (int q = 0; q < 4; q++)
 #pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    bf16x4 v;
+                for (int ep = 0; ep < 4; ep++) {
+                    bf16x8 v;
 #pragma unroll
-                    for (int j = 0; j < 4; j++) v[j] = xv[4 * q + j][e];
-                    st8(xt + t_tile_off(4 * q, 8 * c + e), v);
+                    for (int j = 0; j < 4; j++) {
+                        v[j] = xv[4 * q + j][2 * ep];
+                        v[4 + j] = xv[4 * q + j][2 * ep + 1];
+                    }
+                    const int u = t_tile_off(4 * q, 8 * c + 2 * ep) / 8;      // 16-byte unit inside the tile
+                    st16(stage + (r * kStageBlk + u + (u >> 4)) * 8, v);
                 }
         }
+        stage_out(stage, (bf16*)it.xt + ((int64_t)bh * n1 + blockIdx.x * 16) * kTile, t, n_valid, false);
     }
     if (it.y2 == nullptr && it.y1r == nullptr && it.y1t == nullptr) return;      // uniform over the workgroup
 
     // the 16 pooled rows of this workgroup are one block of the next level
-    __shared__ bf16 sm[16][kD];
+    bf16 (*sm)[kD] = reinterpret_cast<bf16 (*)[kD]>(stage);
     st16(&sm[r][c * 8], y);
     __syncthreads();
     const int n2 = it.n / (kBlk * kBlk);
