@@ -48,7 +48,19 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
 
     for (int i = tid; i < Kb; i += kTrThreads) pos[i] = 0;
     __syncthreads();
-    for (int e = tid; e < E; e += kTrThreads) atomicAdd(&pos[clampi(idx[e], 0, Kb - 1)], 1);
+    // entries are taken 16 per thread at a time, all 16 loads issued before the first is used
+    constexpr int kBatch = 16;
+    for (int e0 = 0; e0 < E; e0 += kBatch * kTrThreads) {
+        int v[kBatch];
+#pragma unroll
+        for (int k = 0; k < kBatch; k++) {
+            const int e = e0 + k * kTrThreads + tid;
+            v[k] = (e < E) ? idx[e] : -1;
+        }
+#pragma unroll
+        for (int k = 0; k < kBatch; k++)
+            if (e0 + k * kTrThreads + tid < E) atomicAdd(&pos[clampi(v[k], 0, Kb - 1)], 1);
+    }
     __syncthreads();
 
     // exclusive scan over pos[0..Kb): each thread owns `per` consecutive counters
@@ -112,9 +124,18 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
     }
     __syncthreads();
 
-    for (int e = tid; e < E; e += kTrThreads) {
-        const int slot = atomicAdd(&pos[clampi(idx[e], 0, Kb - 1)], 1);
-        flat[slot] = e / T;
+    for (int e0 = 0; e0 < E; e0 += kBatch * kTrThreads) {
+        int v[kBatch];
+#pragma unroll
+        for (int k = 0; k < kBatch; k++) {
+            const int e = e0 + k * kTrThreads + tid;
+            v[k] = (e < E) ? idx[e] : -1;
+        }
+#pragma unroll
+        for (int k = 0; k < kBatch; k++) {
+            const int e = e0 + k * kTrThreads + tid;
+            if (e < E) flat[atomicAdd(&pos[clampi(v[k], 0, Kb - 1)], 1)] = e / T;
+        }
     }
     // pos[n] is now the END of segment n; the segments are sorted by sort_segments_kernel
 }
