@@ -383,19 +383,19 @@ __global__ __launch_bounds__(MODE == MODE_FINE ? 64 : 256) void attn_kside_kerne
         cnt = min(p.chunk_len, N1 - start);
         slot = ((int64_t)blockIdx.z * gridDim.y + bh) * p.n_units + unit;
     } else {
+        // the item's record is fetched together with the count it is checked against (the grid never
+        // exceeds the list's storage): the wave knows its key rows and entries after one round trip
         const int* work = p.work + (int64_t)bh * p.work_stride;
         const int item = bx;
-        if (item >= work[0]) return;                          // uniform over the item's waves
-        const int it = work[4 + p.n_units + item];
-        const int ci = it & 0xffff;
-        unit = it >> 16;
-        const int chunk = (MODE == MODE_FINE) ? LLSA_CHUNK_FINE : LLSA_CHUNK_COARSE;
-        const int* o = p.off + (int64_t)bh * (p.n_units + 1) + unit;
-        start = o[0] + ci * chunk;
-        cnt = min(chunk, o[1] - start);
+        const int n_items = work[0];
+        const int* rec = work + 4 + 4 * item;
+        unit = rec[0];
+        start = rec[1];
+        cnt = rec[2];
+        const int sl = rec[3];
+        if (item >= n_items) return;                          // uniform over the item's waves
         if (MODE == MODE_SPARSE1) cnt *= kBlk;                // every parent stands for its 16 children
-        const int sb = work[4 + unit];
-        if (sb >= 0) slot = (int64_t)bh * p.slot_stride + sb + ci;
+        if (sl >= 0) slot = (int64_t)bh * p.slot_stride + sl;
         fl = p.flat + (int64_t)bh * p.flat_stride;
     }
     // What the fold on the way out needs (the unit's pooled-gradient rows, its tokens' RoPE entries)
@@ -551,10 +551,10 @@ __global__ __launch_bounds__(256) void kside_reduce_kernel(ReduceParams rp) {
     const ReduceJob& jb = rp.job[j];
     const int step = reduce_slots(jb.max_units);
     const int* work = jb.work ? jb.work + (int64_t)bh * jb.work_stride : nullptr;
-    const int max_items = (int)(jb.work_stride - 4 - jb.n_units - 4 * jb.max_units);
+    const int max_items = (int)(jb.work_stride - 4 - 4 * jb.max_units) / 4;
     // the unit's record is fetched together with the count it is checked against (u0 is always
     // inside the list's storage): one memory round trip instead of two
-    const int* multi = work ? work + 4 + jb.n_units + max_items : nullptr;
+    const int* multi = work ? work + 4 + 4 * max_items : nullptr;
     int rec_unit = 0, rec_first = 0, rec_n = 0;
     if (work != nullptr) {
         rec_unit = multi[4 * u0];

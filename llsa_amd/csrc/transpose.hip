@@ -23,13 +23,13 @@ __device__ __forceinline__ int wave_incl_scan(int v, int lane) {
 }
 
 // Work list (optional): the K-side kernels walk each key block's segment in chunks of at most
-// `chunk` entries so that a popular key block does not serialise on one wave.  Per (b,h):
+// `chunk` entries so that a popular key block does not serialise on one wave.  Per (b,h), all
+// records 4 ints (16-byte aligned when the list is, so that one load fetches a record):
 //   work[0] = number of items, work[1] = number of partial-sum slots, work[2] = number of key
 //   blocks with more than one chunk, work[3] unused,
-//   work[4 + n] = first slot of key block n, or -1 when n has one chunk,
-//   work[4 + Kb + i] = item i = (n << 16) | chunk index   (items of one key block are adjacent),
-//   work[4 + Kb + max_items + 4j .. +3] = j-th key block with more than one chunk: {n, first slot,
-//   number of chunks, 0} (16-byte aligned when the list itself is: one load tells the reduction all)
+//   work[4 + 4i ..]             item i = {key block n, first entry in flat, entries, partial-sum slot
+//                               or -1 when n has one chunk}      (items of one key block are adjacent),
+//   work[4 + 4 max_items + 4j ..] j-th key block with more than one chunk = {n, first slot, chunks, 0}.
 // Every key block has at least one item (an unselected block's item has no entries and only
 // writes zeros), and max_items = Mb*T/chunk + Kb.
 __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int* __restrict__ idx, int* __restrict__ offsets,
@@ -102,10 +102,15 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
         run += c;
         if (work != nullptr) {
             const int nch = max(1, (c + chunk - 1) / chunk);
-            work[4 + i] = (nch > 1) ? run_s : -1;
-            for (int ci = 0; ci < nch; ci++) work[4 + Kb + run_i + ci] = (i << 16) | ci;
+            for (int ci = 0; ci < nch; ci++) {
+                int* it = work + 4 + 4 * (run_i + ci);
+                it[0] = i;
+                it[1] = run - c + ci * chunk;                  // (run already points past this segment)
+                it[2] = min(chunk, c - ci * chunk);
+                it[3] = (nch > 1) ? run_s + ci : -1;
+            }
             if (nch > 1) {
-                int* m = work + 4 + Kb + max_items + 4 * run_m++;
+                int* m = work + 4 + 4 * max_items + 4 * run_m++;
                 m[0] = i;
                 m[1] = run_s;
                 m[2] = nch;
@@ -185,15 +190,14 @@ using namespace llsa;
 extern "C" int64_t llsa_work_list_len(int Mb, int Kb, int T, int chunk) {
     if (Mb <= 0 || Kb <= 0 || T <= 0 || chunk <= 0) return -1;
     const int64_t e = (int64_t)Mb * T;
-    return 4 + (int64_t)Kb + (e / chunk + Kb) + 4 * (e / chunk + 1);
+    return 4 + 4 * (e / chunk + Kb) + 4 * (e / chunk + 1);
 }
 
 extern "C" int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, int32_t* work, int B, int H, int Mb,
                                       int Kb, int T, int chunk, void* stream) {
     LLSA_REQUIRE(idx && offsets && flat, "transpose_indices: null argument");
     LLSA_REQUIRE(B > 0 && H > 0 && Mb > 0 && Kb > 0 && T > 0, "transpose_indices: bad shape");
-    LLSA_REQUIRE(work == nullptr || (chunk >= 1 && Kb < 32768 && (int64_t)Mb * T / chunk + 1 < 65536),
-                 "transpose_indices: work list needs chunk >= 1, Kb < 32768 and fewer than 65536 chunks per key block");
+    LLSA_REQUIRE(work == nullptr || chunk >= 1, "transpose_indices: work list needs chunk >= 1");
     if (chunk < 1) chunk = 1;
     const size_t lds = sizeof(int) * ((size_t)Kb + 64);
     static_assert(4 * kTrWaves <= 64, "wave totals must fit their LDS slot");
