@@ -22,9 +22,11 @@ def lib_for(*tensors: torch.Tensor) -> Lib:
 
 
 def stream_of(lib: Lib, t: torch.Tensor):
+    """The raw handle of the current stream of t's device (None for the CPU emulation of the tests)."""
     if not lib.device_library:
         return None
-    return C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)
+    idx = t.device.index
+    return C.c_void_p(torch._C._cuda_getCurrentRawStream(torch.cuda.current_device() if idx is None else idx))
 
 
 def ptr(t):

@@ -12,6 +12,7 @@ from __future__ import annotations
 import torch
 from torch.autograd import Function
 
+from ..hip.indices_transpose import BackwardLists
 from ..hip.mean_pool import PoolSpec, mean_pool1d, pool_pyramid
 from ..hip.sparse_attention_res_1 import sparse_indices_attn_res_fwd, sparse_indices_attn_res_scatter_bwd_v2
 from ..hip.topk import gen_sparse_indices
@@ -60,21 +61,23 @@ class _LlsaL1Fused(Function):
         indices = gen_sparse_indices(pq, pk, topk)
         tiles = dict(qr=oq["xr"], kr=ok["xr"], vt=ov["xt"], pkr=ok["y1r"], pvt=ov["y1t"])
         # q / k are only shape-and-stride templates below: the kernels read the (rotated) tiles
+        lists = BackwardLists(indices) if g else None                 # on a second stream, beside the attention kernel
         o, m = sparse_indices_attn_res_fwd(q, k, v, pk, pv, indices, indices.shape[-1], block_size, 4, tiles=tiles)
         if g:
-            ctx.save_for_backward(q, k, v, pk, pv, o, m, indices, freq, oq["xr"], ok["xr"], ov["xr"], ok["y1r"], ov["y1r"])
+            ctx.save_for_backward(q, k, v, pk, pv, o, m, indices, freq, oq["xr"], ok["xr"], ov["xr"], ok["y1r"], ov["y1r"],
+                                  *lists.join())
         ctx.block_size = block_size
         ctx.indices = indices
         return o
 
     @staticmethod
     def backward(ctx, do):
-        q, k, v, pk, pv, o, m, indices, freq, qr, kr, vr, pkr, pvr = ctx.saved_tensors
+        q, k, v, pk, pv, o, m, indices, freq, qr, kr, vr, pkr, pvr, *csr = ctx.saved_tensors
         bs = ctx.block_size
         tiles = dict(qr=qr, kr=kr, vr=vr, pkr=pkr, pvr=pvr)
         dq, dk, dv, _, dpk, dpv = sparse_indices_attn_res_scatter_bwd_v2(
             do, q, k, v, pk, pv, o, m, indices, indices.shape[-1], bs, bs, tiles=tiles, freq_dq=freq,
-            fold_pooled=True, freq_dk=freq)       # dk, dv arrive with the pooled gradients folded in
+            fold_pooled=True, freq_dk=freq, csr=csr)       # dk, dv arrive with the pooled gradients folded in
         return dq, dk, dv, None, None, None
 
 
