@@ -355,21 +355,16 @@ __device__ __forceinline__ void kside_pair(f32x4 dk[4], f32x4 dv[4], const bf16x
 // accumulator layout: 8 f32x4 registers per lane (4 channel tiles of dK, then 4 of dV).
 __device__ __forceinline__ f32x4* part_slot(f32x4* part, int64_t slot) { return part + slot * (8 * kWave); }
 
+#ifndef KS_IPW
+#define KS_IPW 1
+#endif
 template <int MODE>
-__global__ __launch_bounds__(MODE == MODE_FINE ? 64 : 256) void attn_kside_kernel(KSideParams p) {
-    // FINE: one wave per work item and per workgroup (items differ a lot in length; a wave that
-    // shares its workgroup with a longer one would keep its registers and LDS allocated while idle).
-    // Others: four waves per work item.
+__device__ __forceinline__ void kside_item(const KSideParams& p, int bx, int bh, unsigned char* smem_raw, bf16* fold_buf) {
     constexpr int W = (MODE == MODE_FINE) ? 1 : 4;            // waves per work item = waves per workgroup
-    // per wave 2 query blocks x {Q, dO} R tiles; reused for the cross-wave reduction
-    __shared__ __align__(16) unsigned char smem_raw[W * 4 * kTile * sizeof(bf16)];
-    __shared__ __align__(16) bf16 fold_buf[MODE == MODE_FINE ? kFoldElems : 8];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int N1 = p.N / kBlk;
-    const int lid = xcd_logical_id();
-    const int bx = lid % (int)gridDim.x;
-    const int bh = lid / (int)gridDim.x, b = bh / p.H, h = bh % p.H;
+    const int b = bh / p.H, h = bh % p.H;
     const int r = lane & 15, quad = lane >> 4;
     const int sub = (MODE == MODE_FINE) ? 0 : wave;
 
@@ -482,7 +477,7 @@ __global__ __launch_bounds__(MODE == MODE_FINE ? 64 : 256) void attn_kside_kerne
     // four waves per item: reduce through LDS, wave w finishes channel tile w
     __syncthreads();                                          // everyone is done with the staging area
     f32x4 (*red)[8][kWave] = reinterpret_cast<f32x4 (*)[8][kWave]>(smem_raw);
-    static_assert(MODE == MODE_FINE || sizeof(smem_raw) >= 4 * 8 * kWave * sizeof(f32x4), "reduction buffer must fit the staging area");
+    static_assert(MODE == MODE_FINE || W * 4 * kTile * sizeof(bf16) >= 4 * 8 * kWave * sizeof(f32x4), "reduction buffer must fit the staging area");
 #pragma unroll
     for (int dt = 0; dt < 4; dt++) {
         red[wave][dt][lane] = dk[dt];
@@ -505,6 +500,29 @@ __global__ __launch_bounds__(MODE == MODE_FINE ? 64 : 256) void attn_kside_kerne
         bf16* vp = p.dv + b * p.sdvb + h * p.sdvh + (int64_t)(unit * kBlk + r) * p.sdvn + quad * 4 + dt * 16;
         st8(kp, cvt4(sk * kScale));
         st8(vp, cvt4(sv));
+    }
+}
+
+template <int MODE>
+__global__ __launch_bounds__(MODE == MODE_FINE ? 64 : 256) void attn_kside_kernel(KSideParams p) {
+    // FINE: one wave per work item and per workgroup (items differ a lot in length; a wave that
+    // shares its workgroup with a longer one would keep its registers and LDS allocated while idle).
+    // Others: four waves per work item.
+    constexpr int W = (MODE == MODE_FINE) ? 1 : 4;
+    // per wave 2 query blocks x {Q, dO} R tiles; reused for the cross-wave reduction
+    __shared__ __align__(16) unsigned char smem_raw[W * 4 * kTile * sizeof(bf16)];
+    __shared__ __align__(16) bf16 fold_buf[MODE == MODE_FINE ? kFoldElems : 8];
+    const int lid = xcd_logical_id();
+    const int bx = lid % (int)gridDim.x;
+    const int bh = lid / (int)gridDim.x;
+    if (MODE == MODE_FINE) {
+        for (int rep = 0; rep < KS_IPW; rep++) {
+            kside_item<MODE>(p, bx * KS_IPW + rep, bh, smem_raw, fold_buf);
+            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+        }
+    } else {
+        kside_item<MODE>(p, bx, bh, smem_raw, fold_buf);
     }
 }
 
@@ -740,7 +758,7 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
             p.fold = PoolFold{(const bf16*)a->dpk, (const bf16*)a->dpv, (a->levels == 2) ? (const bf16*)a->dpk2 : nullptr,
                               (a->levels == 2) ? (const bf16*)a->dpv2 : nullptr, (const bf16*)a->freq_dk};
         const int max_items = N1 * a->T / LLSA_CHUNK_FINE + N1;
-        hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_FINE>), dim3(max_items, BH), dim3(64), 0, s, p);
+        hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_FINE>), dim3((max_items + KS_IPW - 1) / KS_IPW, BH), dim3(64), 0, s, p);
         add_job(p, LLSA_CHUNK_FINE, N1 * a->T / LLSA_CHUNK_FINE + 1, 0);
     };
     auto run_sparse1 = [&]() {                                // level-1 pooled tokens, through the transposed coarse index

@@ -31,13 +31,15 @@ __device__ __forceinline__ int wave_incl_scan(int v, int lane) {
 //                               or -1 when n has one chunk}      (items of one key block are adjacent),
 //   work[4 + 4 max_items + 4j ..] j-th key block with more than one chunk = {n, first slot, chunks, 0}.
 // Every key block has at least one item (an unselected block's item has no entries and only
-// writes zeros), and max_items = Mb*T/chunk + Kb.
+// writes zeros), and max_items = Mb*T/chunk + Kb.  Items with more than chunk/2 entries come first
+// in the list: a wave walks its item serially, so the long ones have to start early or the kernel
+// ends with a few waves still working.
 __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int* __restrict__ idx, int* __restrict__ offsets,
                                                                       int* __restrict__ flat, int* __restrict__ work,
                                                                       int Mb, int Kb, int T, int chunk, int work_stride) {
     HIP_DYNAMIC_SHARED(int, smem)
     int* pos = smem;                               // Kb
-    int* wave_tot = smem + Kb;                     // 4 * kTrWaves
+    int* wave_tot = smem + Kb;                     // 5 * kTrWaves
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int bh = blockIdx.x;
@@ -66,12 +68,16 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
     // exclusive scan over pos[0..Kb): each thread owns `per` consecutive counters
     const int per = (Kb + kTrThreads - 1) / kTrThreads;
     const int c0 = min(tid * per, Kb), c1 = min(c0 + per, Kb);
-    int local = 0, l_items = 0, l_slots = 0, l_multi = 0;
+    // l_items: short items, l_long: long items (more than chunk/2 entries)
+    const int long_min = chunk / 2 + 1;
+    int local = 0, l_items = 0, l_slots = 0, l_multi = 0, l_long = 0;
     for (int i = c0; i < c1; i++) {
         const int c = pos[i];
         const int nch = max(1, (c + chunk - 1) / chunk);
+        const int n_long = (nch - 1) + ((c - (nch - 1) * chunk >= long_min) ? 1 : 0);   // all chunks but the last are full
         local += c;
-        l_items += nch;
+        l_long += n_long;
+        l_items += nch - n_long;
         l_slots += (nch > 1) ? nch : 0;
         l_multi += (nch > 1) ? 1 : 0;
     }
@@ -79,20 +85,28 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
     const int incl_i = wave_incl_scan(l_items, lane);
     const int incl_s = wave_incl_scan(l_slots, lane);
     const int incl_m = wave_incl_scan(l_multi, lane);
+    const int incl_l = wave_incl_scan(l_long, lane);
     if (lane == kWave - 1) {
         wave_tot[wave] = incl;
         wave_tot[kTrWaves + wave] = incl_i;
         wave_tot[2 * kTrWaves + wave] = incl_s;
         wave_tot[3 * kTrWaves + wave] = incl_m;
+        wave_tot[4 * kTrWaves + wave] = incl_l;
     }
     __syncthreads();
-    int run = incl - local, run_i = incl_i - l_items, run_s = incl_s - l_slots, run_m = incl_m - l_multi;
-    for (int w = 0; w < wave; w++) {
-        run += wave_tot[w];
-        run_i += wave_tot[kTrWaves + w];
-        run_s += wave_tot[2 * kTrWaves + w];
-        run_m += wave_tot[3 * kTrWaves + w];
+    int run = incl - local, run_i = incl_i - l_items, run_s = incl_s - l_slots, run_m = incl_m - l_multi, run_l = incl_l - l_long;
+    int total_long = 0;
+    for (int w = 0; w < kTrWaves; w++) {
+        total_long += wave_tot[4 * kTrWaves + w];
+        if (w < wave) {
+            run += wave_tot[w];
+            run_i += wave_tot[kTrWaves + w];
+            run_s += wave_tot[2 * kTrWaves + w];
+            run_m += wave_tot[3 * kTrWaves + w];
+            run_l += wave_tot[4 * kTrWaves + w];
+        }
     }
+    run_i += total_long;                                      // short items follow the long ones
     if (work != nullptr) work += (int64_t)bh * work_stride;
     const int max_items = E / chunk + Kb;
     for (int i = c0; i < c1; i++) {
@@ -103,10 +117,11 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
         if (work != nullptr) {
             const int nch = max(1, (c + chunk - 1) / chunk);
             for (int ci = 0; ci < nch; ci++) {
-                int* it = work + 4 + 4 * (run_i + ci);
+                const int n_ent = min(chunk, c - ci * chunk);
+                int* it = work + 4 + 4 * ((n_ent >= long_min) ? run_l++ : run_i++);
                 it[0] = i;
                 it[1] = run - c + ci * chunk;                  // (run already points past this segment)
-                it[2] = min(chunk, c - ci * chunk);
+                it[2] = n_ent;
                 it[3] = (nch > 1) ? run_s + ci : -1;
             }
             if (nch > 1) {
@@ -116,13 +131,12 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
                 m[2] = nch;
                 m[3] = 0;
             }
-            run_i += nch;
             run_s += (nch > 1) ? nch : 0;
         }
     }
     if (tid == 0) offsets[Kb] = E;
     if (work != nullptr && tid == kTrThreads - 1) {
-        work[0] = run_i;
+        work[0] = run_i;                                      // (the last thread's short items end the list)
         work[1] = run_s;
         work[2] = run_m;
         work[3] = 0;
@@ -199,8 +213,8 @@ extern "C" int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int3
     LLSA_REQUIRE(B > 0 && H > 0 && Mb > 0 && Kb > 0 && T > 0, "transpose_indices: bad shape");
     LLSA_REQUIRE(work == nullptr || chunk >= 1, "transpose_indices: work list needs chunk >= 1");
     if (chunk < 1) chunk = 1;
-    const size_t lds = sizeof(int) * ((size_t)Kb + 64);
-    static_assert(4 * kTrWaves <= 64, "wave totals must fit their LDS slot");
+    const size_t lds = sizeof(int) * ((size_t)Kb + 128);
+    static_assert(5 * kTrWaves <= 128, "wave totals must fit their LDS slot");
     LLSA_REQUIRE(lds <= 160 * 1024, "transpose_indices: Kb=%d needs %zu bytes of LDS (limit 163840)", Kb, lds);
     const size_t lds_sort = sizeof(unsigned) * 4 * ((size_t)(Mb + 31) / 32);
     LLSA_REQUIRE(lds_sort <= 64 * 1024, "transpose_indices: Mb=%d needs %zu bytes of LDS for the segment sort", Mb, lds_sort);
