@@ -526,6 +526,122 @@ __global__ __launch_bounds__(MODE == MODE_FINE ? 64 : 256) void attn_kside_kerne
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// Dense coarsest level.  Every unit (16 pooled tokens) meets every query block, so the Q / dO
+// tiles are the same for all units: a workgroup takes four units (one per wave) and one piece
+// of the query range, and the tiles of each pair of query blocks are copied into LDS once for
+// the four of them (two 8 KB buffers: the copy of pair t+1 runs during the arithmetic of pair t).
+// Each wave ends with the partial sum of its unit over this piece of the range.
+// ---------------------------------------------------------------------------------------
+constexpr int kDenseUnits = 4;                    // units (= waves) per workgroup
+
+__global__ __launch_bounds__(64 * kDenseUnits) void attn_kside_dense_kernel(KSideParams p) {
+    __shared__ __align__(16) bf16 sh[2][4 * kTile];           // per pair: Q0, dO0, Q1, dO1 as R tiles
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int quad = lane >> 4;
+    const int N1 = p.N / kBlk;
+    const int bh = blockIdx.y;
+    const int unit = blockIdx.x * kDenseUnits + wave;         // < n_units: the host checks n_units % kDenseUnits == 0
+    const int start = blockIdx.z * p.chunk_len;
+    const int n_pairs = min(p.chunk_len, N1 - start) / 2;     // chunk_len and N1 are even
+    const bf16* qrb = p.qr + ((int64_t)bh * N1 + start) * kTile;
+    const bf16* dorb = p.dor + ((int64_t)bh * N1 + start) * kTile;
+    const float* lseb = p.lse + (int64_t)bh * p.N + start * kBlk;
+    const float* dlb = p.delta + (int64_t)bh * p.N + start * kBlk;
+
+    // wave w copies tile w of the pair's four (query block w/2; Q for even w, dO for odd w)
+    auto issue = [=](int t) __attribute__((always_inline)) {
+        const bf16* src = ((wave & 1) ? dorb : qrb) + (int64_t)(2 * t + (wave >> 1)) * kTile;
+        bf16* dst = &sh[t & 1][wave * kTile];
+        copy16_global_to_lds(src + lane * 8, dst);
+        copy16_global_to_lds(src + 512 + lane * 8, dst + 512);
+    };
+    struct Stats { f32x4 l[2], d[2]; };
+    auto load_stats = [=](int t, Stats& st) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            st.l[u] = *reinterpret_cast<const f32x4*>(lseb + (2 * t + u) * kBlk + quad * 4);
+            st.d[u] = *reinterpret_cast<const f32x4*>(dlb + (2 * t + u) * kBlk + quad * 4);
+        }
+    };
+    if (n_pairs > 0) issue(0);
+    bf16x8 bk[2], bv[2];
+    {
+        const bf16* kp = p.kk + ((int64_t)bh * p.n_units + unit) * kTile + lane * 8;
+        const bf16* vp = p.vv + ((int64_t)bh * p.n_units + unit) * kTile + lane * 8;
+        bk[0] = ld16(kp);
+        bk[1] = ld16(kp + 512);
+        bv[0] = ld16(vp);
+        bv[1] = ld16(vp + 512);
+    }
+    Stats sa, sb;
+    if (n_pairs > 0) load_stats(0, sa);
+    f32x4 dk[4], dv[4];
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++) {
+        dk[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        dv[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    }
+    // One round per pair.  The barrier at its top says: the pair's tiles have landed (every wave
+    // waited for its own copies) and everybody is done reading the other buffer.  All LDS reads of
+    // the round come before the next copies are issued (the compiler makes an LDS read wait for
+    // every copy into LDS issued before it).
+    auto round = [&](int t, const Stats& cur, Stats& nxt) __attribute__((always_inline)) {
+        wait_vm0();
+        __syncthreads();
+        const bf16* b = &sh[t & 1][0];
+        bf16x8 aq[2][2], ag[2][2];
+        bf16x4 tq[2][4], tg[2][4];
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            aq[u][0] = lds_ld16(b + (2 * u) * kTile + lane * 8);
+            aq[u][1] = lds_ld16(b + (2 * u) * kTile + 512 + lane * 8);
+            ag[u][0] = lds_ld16(b + (2 * u + 1) * kTile + lane * 8);
+            ag[u][1] = lds_ld16(b + (2 * u + 1) * kTile + 512 + lane * 8);
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) {
+                tq[u][dt] = lds_t_operand(b + (2 * u) * kTile, dt, lane);
+                tg[u][dt] = lds_t_operand(b + (2 * u + 1) * kTile, dt, lane);
+            }
+        }
+        if (t + 1 < n_pairs) {
+            issue(t + 1);
+            load_stats(t + 1, nxt);
+        }
+        bf16x8 bp, bds;
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
+            s = mfma_bf16(aq[u][0], bk[0], s);
+            s = mfma_bf16(aq[u][1], bk[1], s);
+            dp = mfma_bf16(ag[u][0], bv[0], dp);
+            dp = mfma_bf16(ag[u][1], bv[1], dp);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const float pe = exp2_fast(fmaf(s[e], kScaleLog2e, -cur.l[u][e] * kLog2e)) * p.w;
+                bp[u * 4 + e] = (bf16)pe;
+                bds[u * 4 + e] = (bf16)(pe * (dp[e] - cur.d[u][e]));
+            }
+        }
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+            dv[dt] = mfma_bf16(cat(tg[0][dt], tg[1][dt]), bp, dv[dt]);
+            dk[dt] = mfma_bf16(cat(tq[0][dt], tq[1][dt]), bds, dk[dt]);
+        }
+    };
+    for (int t = 0; t < n_pairs; t += 2) {
+        round(t, sa, sb);
+        if (t + 1 < n_pairs) round(t + 1, sb, sa);
+    }
+    f32x4* ps = part_slot(p.part, ((int64_t)blockIdx.z * gridDim.y + bh) * p.n_units + unit);
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++) {
+        ps[dt * kWave + lane] = dk[dt];
+        ps[(4 + dt) * kWave + lane] = dv[dt];
+    }
+}
+
 // Finishes the units whose list was cut into several pieces: the result is the sum of the
 // unit's partial slots, added in chunk order, so it does not depend on scheduling.  One launch
 // serves the three K-side passes.
@@ -628,8 +744,8 @@ static DensePlan dense_plan(int B, int H, int N, int levels) {
     const int N1 = N / 16;
     DensePlan d;
     d.n_tok = (levels == 2) ? N1 / 16 : N1;
-    const int units = (d.n_tok / 16) * B * H;
-    int chunks = (1024 + units - 1) / units;
+    const int groups = (d.n_tok / 16 / 4) * B * H;            // workgroups per piece of the query range (4 units each)
+    int chunks = (512 + groups - 1) / groups;                 // aim at two workgroups per CU
     if (chunks > N1 / 16) chunks = N1 / 16;
     if (chunks < 1) chunks = 1;
     int len = (N1 + chunks - 1) / chunks;
@@ -795,7 +911,7 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
         p.off = nullptr; p.flat = nullptr; p.flat_stride = 0; p.work = nullptr; p.work_stride = 0; p.slot_stride = 0;
         p.part = (f32x4*)(ws + wsp.part_dense);
         p.n_units = d.n_tok / 16; p.chunk_len = d.chunk_len;
-        hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_DENSE>), dim3(p.n_units, BH, d.chunks), dim3(256), 0, s, p);
+        hipLaunchKernelGGL(attn_kside_dense_kernel, dim3(p.n_units / kDenseUnits, BH, d.chunks), dim3(64 * kDenseUnits), 0, s, p);
         add_job(p, 1, p.n_units, d.chunks);
     };
 
