@@ -182,6 +182,9 @@ def main():
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
     ap.add_argument("--no-extras", action="store_true", help="skip stage profile, CPU baseline and dense SDPA")
     ap.add_argument("--unfused", action="store_true", help="use the reference's composition (separate pools, autograd adds)")
+    ap.add_argument("--graph", action="store_true",
+                    help="also capture the step in one HIP graph (llsa_amd.GraphedStep) and time its replay; "
+                         "reported as ms_per_step_graph next to the eager figure, which stays `value`")
     ap.add_argument("--calibrate", action="store_true",
                     help="after the timed region also launch a plain elementwise copy of 256 MiB (fp32, read 256 MiB + "
                          "write 256 MiB) five times, so that a counter profile of this command holds a kernel of known "
@@ -204,23 +207,34 @@ def main():
     freq = rope_table(math.isqrt(N), dtype=torch.bfloat16).to(dev) if rope else None
     q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
 
-    def step():
-        q.grad = k.grad = v.grad = None
+    def fwd(q_, k_, v_):
         if args.unfused:
-            qq, kk = (llsa_amd.my_rope_fn(q, freq), llsa_amd.my_rope_fn(k, freq)) if rope else (q, k)
-            o = llsa_amd.llsa_l2_unfused(qq, kk, v, t1, t2, 16) if op == "l2" else llsa_amd.llsa_l1_unfused(qq, kk, v, t1, 16)
-        else:
-            o = llsa_amd.llsa_l2(q, k, v, t1, t2, 16, rope=freq) if op == "l2" else llsa_amd.llsa_l1(q, k, v, t1, 16, rope=freq)
-        o.backward(do)
+            qq, kk = (llsa_amd.my_rope_fn(q_, freq), llsa_amd.my_rope_fn(k_, freq)) if rope else (q_, k_)
+            return llsa_amd.llsa_l2_unfused(qq, kk, v_, t1, t2, 16) if op == "l2" else llsa_amd.llsa_l1_unfused(qq, kk, v_, t1, 16)
+        return llsa_amd.llsa_l2(q_, k_, v_, t1, t2, 16, rope=freq) if op == "l2" else llsa_amd.llsa_l1(q_, k_, v_, t1, 16, rope=freq)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    def eager_step():
+        q.grad = k.grad = v.grad = None
+        fwd(q, k, v).backward(do)
+
+    def time_steps(step):
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            step()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # `value` is the step as a user's training loop issues it: ~25 launches from Python.  With --graph
+    # the same step is also replayed from one captured HIP graph (one call per step; the host time of
+    # the separate launches is about what the kernels take at these sizes).
+    ms = time_steps(eager_step)
+    ms_graph = None
+    if args.graph:
+        graphed = llsa_amd.GraphedStep(fwd, [q, k, v], do)
+        ms_graph = time_steps(graphed.replay)
 
     if args.calibrate:
         src = torch.ones(64 * 1024 * 1024, device=dev, dtype=torch.float32)
@@ -243,6 +257,7 @@ def main():
                                + (" (unfused composition)" if args.unfused else ""),
                    "n_kv_per_query": nkv, "algorithmic_gflop": flops / 1e9},
         "frac_of_bf16_mfma_peak": flops / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+        "ms_per_step_graph": ms_graph,
     }
 
     if not args.no_extras:
