@@ -36,8 +36,8 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 # WRITE_SIZE on this command, each scaled by what the same counter reads for a 256 MiB elementwise
 # copy (fetch x2.000, write x1.000); the tables they come from are profiles/step_kernels_<workload>_hbm_traffic.txt
 MEASURED_TRAFFIC = {
-    "c3": {"attn_fwd": 130407581, "bwd_dq": 192478201, "bwd_dkv": 261496020, "bwd_dpkv1_sparse": 244863559,
-           "bwd_dpkv_dense": 78392634, "pool_pyramid": 103315496},
+    "c3": {"attn_fwd": 129255961, "bwd_dq": 250116299, "bwd_dkv": 307471105, "bwd_dpkv1_sparse": 243579460,
+           "bwd_dpkv_dense": 78511042, "pool_pyramid": 95455683},
 }
 
 WORKLOADS = {
@@ -128,13 +128,17 @@ def stage_profile(op, q, k, v, do, t1, t2, freq, iters, torch):
     run = lambda st: A.attn_bwd(do, q, k, v, pk, pv, o, lse, idx, 16.0, cgw, stages=st, freq_dq=freq, fold_pooled=True,
                                 freq_dk=freq, **bkw)
     run(2)
-    for name, st in (("bwd_dq", 2), ("bwd_dpkv1_sparse", 8), ("bwd_dpkv_dense", 16), ("bwd_dkv", 4)):
-        if st == 8 and not l2:
+    NO_REDUCE = 32
+    for name, st in (("bwd_dq", 2), ("bwd_dpkv1_sparse", 8 | NO_REDUCE), ("bwd_dpkv_dense", 16 | NO_REDUCE),
+                     ("bwd_dkv", 4 | NO_REDUCE)):
+        if (st & 8) and not l2:
             continue
         # a stage run alone reads whatever workspace the allocator hands back (the block the dq stage
-        # just filled with delta and the dO tiles); only its duration is used.  The K-side stages
-        # include the reduction of their partial sums.
+        # just filled with delta and the dO tiles); only its duration is used
         res[name] = timed(lambda: run(st), iters, torch)
+    # the two launches that add up the partial sums of the K-side passes
+    res["bwd_reduce"] = timed(lambda: run(4 | 8 | 16), iters, torch) - res["bwd_dkv"] - res["bwd_dpkv_dense"] \
+        - res.get("bwd_dpkv1_sparse", 0.0)
     return res
 
 

@@ -196,6 +196,8 @@ typedef struct llsa_attn_bwd_args {
 #define LLSA_BWD_DKV 4      /* dK/dV of the fine tokens                                          */
 #define LLSA_BWD_DPKV1 8    /* sparse level-1 pooled gradients (levels == 2)                     */
 #define LLSA_BWD_DENSE 16   /* dense coarsest pooled gradients (partials + reduction)            */
+#define LLSA_BWD_NO_REDUCE 32 /* with an explicit mask: leave out the reductions of partial sums (results
+                                 are then incomplete; for timing the K-side kernels alone)          */
 
 int64_t llsa_attn_bwd_workspace_bytes(int B, int H, int N, int T, int T2, int levels);
 int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream);

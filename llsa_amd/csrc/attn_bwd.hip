@@ -236,9 +236,10 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, floa
 // ---------------------------------------------------------------------------------------
 // K-side gradients.  A "unit" is 16 key rows (a fine K block, 16 level-1 pooled tokens of one
 // coarse block, or 16 tokens of the dense coarsest level) together with a list of query
-// blocks; the unit's waves walk the list two query blocks at a time.
+// blocks; the unit's waves walk the list two query blocks at a time.  attn_kside_kernel serves
+// the two list-driven passes, attn_kside_dense_kernel the dense one.
 // ---------------------------------------------------------------------------------------
-enum { MODE_FINE = 0, MODE_SPARSE1 = 1, MODE_DENSE = 2 };
+enum { MODE_FINE = 0, MODE_SPARSE1 = 1 };       // (the dense coarsest level has a kernel of its own)
 
 // Optional last step of the fine dK / dV: add the pooled gradients the token's block received
 // (what the backward of the two mean pools and autograd's accumulation do in the reference:
@@ -372,12 +373,7 @@ __device__ __forceinline__ void kside_item(const KSideParams& p, int bx, int bh,
     int unit, start, cnt;
     int64_t slot = -1;                                        // >= 0: write an fp32 partial
     const int* fl = nullptr;
-    if (MODE == MODE_DENSE) {
-        unit = bx;
-        start = blockIdx.z * p.chunk_len;
-        cnt = min(p.chunk_len, N1 - start);
-        slot = ((int64_t)blockIdx.z * gridDim.y + bh) * p.n_units + unit;
-    } else {
+    {
         // the item's record is fetched together with the count it is checked against (the grid never
         // exceeds the list's storage): the wave knows its key rows and entries after one round trip
         const int* work = p.work + (int64_t)bh * p.work_stride;
@@ -416,8 +412,7 @@ __device__ __forceinline__ void kside_item(const KSideParams& p, int bx, int bh,
     if (MODE == MODE_FINE) mine = (lane < cnt) ? fl[start + lane] : 0;
     auto entry = [&](int i) -> int {                          // i-th query block of this item (i is wave-uniform)
         if (MODE == MODE_FINE) return clampi(__builtin_amdgcn_readlane(mine, i), 0, N1 - 1);
-        if (MODE == MODE_SPARSE1) return clampi(fl[start + i / kBlk], 0, N1 / kBlk - 1) * kBlk + (i % kBlk);
-        return start + i;
+        return clampi(fl[start + i / kBlk], 0, N1 / kBlk - 1) * kBlk + (i % kBlk);
     };
 
     f32x4 dk[4], dv[4];
@@ -828,7 +823,7 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     const bool fold = a->fold_pooled != 0;
     LLSA_REQUIRE(fold || a->freq_dk == nullptr, "attn_bwd: freq_dk needs fold_pooled");
 
-    const int stages = a->stages ? a->stages : 0x7fffffff;
+    const int stages = a->stages ? a->stages : (0x7fffffff & ~LLSA_BWD_NO_REDUCE);
     if (stages & LLSA_BWD_DQ)
         hipLaunchKernelGGL(attn_dq_kernel, dim3((N1 + 3) / 4, BH), dim3(256), 0, s, *a, delta, dor);
 
@@ -846,6 +841,7 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
         j.fold = p.fold;
     };
     auto run_reduce = [&]() {
+        if (stages & LLSA_BWD_NO_REDUCE) rp.n_jobs = 0;       // (profiling: time the K-side kernels alone)
         if (rp.n_jobs == 0) return;
         int slots = 0;
         for (int i = 0; i < rp.n_jobs; i++) slots += reduce_slots(rp.job[i].max_units);
