@@ -56,25 +56,27 @@ struct PoolParams {
 // array.  A thread's registers hold 256-byte pieces of it that are 256 bytes apart from its
 // neighbours' (R) or 8-byte pieces scattered over a whole tile (T); stored straight from the
 // registers every store instruction would touch 64 different cache lines with 16 or 8 bytes
-// each.  They go through LDS instead (16-byte units, block stride 136 units, padded so that both
-// sides spread over the banks) and leave as full-width stores: thread t of the workgroup writes
-// the 16 bytes at (k * 128 + t) * 16 for k = 0..15.
-constexpr int kStageBlk = 136;                    // 16-byte units per block in the staging buffer (128 + padding)
+// each.  They go through LDS instead and leave as full-width stores: thread t of the workgroup
+// writes the 16 bytes at (k * 128 + t) * 16 for k = 0..15.  The staging buffer holds the 16-byte
+// units of a block in tile order with their low index bits XOR-ed so that both sides spread over
+// the banks without padding: exactly 32 KB, five workgroups per CU.
+__device__ __forceinline__ int swz_r(int u, int blk) { return u ^ ((u >> 4) ^ (blk & 15)); }   // u = chunk * 16 + row
+__device__ __forceinline__ int swz_t(int u) { return u ^ (u >> 5); }                           // u = unit of the T tile
 
 __device__ __forceinline__ void stage_out(bf16* stage, bf16* tiles32k, int t, int n_valid_blocks, bool r_layout) {
     __syncthreads();                              // the staging buffer is filled
 #pragma unroll
     for (int k = 0; k < 16; k++) {
         if (k < n_valid_blocks) {
-            const int u = r_layout ? (t >> 4) * 17 + (t & 15) : t + (t >> 4);
-            st16(tiles32k + (k * 128 + t) * 8, ld16(stage + (k * kStageBlk + u) * 8));
+            const int u = r_layout ? swz_r(t, k) : swz_t(t);
+            st16(tiles32k + (k * 128 + t) * 8, ld16(stage + (k * 128 + u) * 8));
         }
     }
     __syncthreads();                              // and may be refilled
 }
 
 __global__ __launch_bounds__(128) void pool_pyramid_kernel(PoolParams p) {
-    __shared__ __align__(16) bf16 stage[16 * kStageBlk * 8];
+    __shared__ __align__(16) bf16 stage[16 * 128 * 8];
     const llsa_pool_item& it = p.it[blockIdx.z];
     const int n1 = it.n / kBlk;
     if ((int)blockIdx.x * 16 >= n1) return;       // uniform over the workgroup
@@ -116,7 +118,7 @@ __global__ __launch_bounds__(128) void pool_pyramid_kernel(PoolParams p) {
     if (it.xr != nullptr) {              // R tile: chunk c of row i is 16-byte unit c * 16 + i of the block
         if (valid) {
 #pragma unroll
-            for (int i = 0; i < 16; i++) st16(stage + (r * kStageBlk + c * 17 + i) * 8, xv[i]);
+            for (int i = 0; i < 16; i++) st16(stage + (r * 128 + swz_r(c * 16 + i, r)) * 8, xv[i]);
         }
         stage_out(stage, (bf16*)it.xr + ((int64_t)bh * n1 + blockIdx.x * 16) * kTile, t, n_valid, true);
     }
@@ -133,7 +135,7 @@ __global__ __launch_bounds__(128) void pool_pyramid_kernel(PoolParams p) {
                         v[4 + j] = xv[4 * q + j][2 * ep + 1];
                     }
                     const int u = t_tile_off(4 * q, 8 * c + 2 * ep) / 8;      // 16-byte unit inside the tile
-                    st16(stage + (r * kStageBlk + u + (u >> 4)) * 8, v);
+                    st16(stage + (r * 128 + swz_t(u)) * 8, v);
                 }
         }
         stage_out(stage, (bf16*)it.xt + ((int64_t)bh * n1 + blockIdx.x * 16) * kTile, t, n_valid, false);
