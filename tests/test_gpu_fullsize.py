@@ -1,0 +1,68 @@
+"""The benchmark configurations at their full sizes.
+
+C2 and C3 are small enough for the CPU oracle, slice by slice.  At N = 65536 and 262144 the
+oracle would take minutes, so the operator is checked through properties that do not depend on
+the size (the selection depends on q and k only, so it is the same on both sides of each):
+  * constant V            -> O is that constant (the weights of fine and pooled tokens sum to 1)
+  * linearity in V        -> O(a V1 + b V2) = a O(V1) + b O(V2)
+  * column sums           -> sum over tokens of dV = sum over tokens of dO, channel by channel
+                             (every query's weights sum to 1; a pooled token hands 1/16 to each child)
+  * scale invariance      -> sum(q * dq) = sum(k * dk): scores see q and k only through q.k
+"""
+import math
+
+import pytest
+import torch
+
+import parity_cases as P
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available()
+    from llsa_amd._lib import get_lib
+    get_lib()
+    return torch.device("cuda:0")
+
+
+def test_c2_full_size_against_oracle(dev):
+    P.check_op_l1(dev, B=4, H=6, N=4096, T=16, fused=True, rope=False, smooth=True)
+
+
+def test_c3_full_size_against_oracle(dev):
+    P.check_op_l2(dev, B=2, H=6, N=16384, T=16, T2=16, fused=True, rope=True, smooth=True)
+
+
+def _rel(a, b):
+    return ((a.double() - b.double()).norm() / b.double().norm().clamp_min(1e-30)).item()
+
+
+@pytest.mark.parametrize("N,H", [(65536, 2), (262144, 1)])
+def test_large_n_properties(dev, N, H):
+    import llsa_amd
+    from llsa_amd.utils.rope_table import rope_table
+    q, k, v, do = P.smooth_inputs(1, H, N, 64, dev)
+    freq = rope_table(math.isqrt(N), dtype=torch.bfloat16).to(dev)
+    op = lambda q_, k_, v_: llsa_amd.llsa_l2(q_, k_, v_, 16, 16, 16, rope=freq)
+
+    with torch.no_grad():
+        const = torch.full_like(v, 0.625)
+        assert (op(q, k, const).float() - 0.625).abs().max().item() < 4e-3, "constant V must come out unchanged"
+        v2 = P.smooth_inputs(1, H, N, 64, dev, seeds=(5, 6, 7, 8))[2]
+        o1, o2 = op(q, k, v).float(), op(q, k, v2).float()
+        mix = (0.5 * v.float() - 0.25 * v2.float()).bfloat16()
+        want = 0.5 * o1 - 0.25 * o2
+        assert _rel(op(q, k, mix).float(), want) < 1e-2, "O must be linear in V"
+
+    q, k, v = (t.detach().requires_grad_(True) for t in (q, k, v))
+    op(q, k, v).backward(do)
+    torch.cuda.synchronize()
+    assert all(torch.isfinite(t.grad).all() for t in (q, k, v))
+    col_dv, col_do = v.grad.double().sum(dim=2), do.double().sum(dim=2)
+    assert _rel(col_dv, col_do) < 1e-2, f"column sums of dV and dO differ: {_rel(col_dv, col_do):.3e}"
+    # the gradients are bf16 and both sums cancel heavily, so compare them on the scale of their terms
+    qdq, kdk = (q.detach().double() * q.grad.double()).sum(), (k.detach().double() * k.grad.double()).sum()
+    scale = (q.detach().double() * q.grad.double()).abs().sum()
+    assert abs(qdq - kdk) / scale < 2e-3, f"sum(q dq) = {qdq:.6e} but sum(k dk) = {kdk:.6e} (terms sum to {scale:.3e})"
