@@ -1,0 +1,267 @@
+"""llsa_l1 / llsa_l2 as ONE autograd node with a lean host side.
+
+The reference composes the operator from nine Python launchers (six mean pools, two selections,
+the attention) and autograd adds the pooled gradients afterwards.  The kernels of this package
+fuse most of that work, and at the sizes of interest they finish a whole forward + backward in
+a few hundred microseconds -- less than it costs Python to allocate ~40 tensors and to fill the
+argument structures through the general-purpose wrappers.  This module is the same sequence of
+C-ABI calls as those wrappers make, with one arena per data type instead of a tensor per
+intermediate and raw pointer arithmetic instead of views:
+
+    forward   pool_pyramid_fwd (q, k, v: pooled rows, RoPE, operand tiles) [+ level-2 tiles]
+              topk_dense [+ topk_sparse]
+              transpose_indices x levels  (second stream, beside the attention kernel)
+              attn_fwd
+    backward  attn_bwd with fold_pooled = 1  (dq, dk, dv complete, rotated back)
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+from torch.autograd import Function
+
+from ..._lib import CHUNK_COARSE, CHUNK_FINE, AttnBwdArgs, AttnFwdArgs, PoolItem, current_lib
+
+_side = {}          # device -> (second stream, event)
+
+
+def _rows_ok(t):
+    return t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in t.stride()[:-1])
+
+
+def _align(n, a):
+    return (n + a - 1) // a * a
+
+
+class _Layout:
+    """Offsets (in elements) of everything the forward produces, inside one bf16 arena and one
+    int32 arena; every section is contiguous (B*H, ...) and starts 256-byte aligned."""
+
+    def __init__(self, lib, B, H, N, levels, T, T2, grad):
+        BH = B * H
+        n1, n2 = N // 16, N // 256
+        self.n1, self.n2 = n1, n2
+        o = 0
+
+        def take(rows_per_bh, width, on=True):
+            nonlocal o
+            if not on:
+                return None
+            at = o
+            o = _align(o + BH * rows_per_bh * width, 128)
+            return at
+
+        l2 = levels == 2
+        self.pq, self.pk, self.pv = take(n1, 64), take(n1, 64), take(n1, 64)
+        self.pq2, self.pk2, self.pv2 = take(n2, 64, l2), take(n2, 64, l2), take(n2, 64, l2)
+        self.qr, self.kr, self.vr, self.vt = take(n1, 1024), take(n1, 1024), take(n1, 1024, grad), take(n1, 1024)
+        self.pkr, self.pvr, self.pvt = take(n2, 1024), take(n2, 1024, grad), take(n2, 1024)
+        n3 = max(n2 // 16, 1)
+        self.pk2r, self.pv2r, self.pv2t = take(n3, 1024, l2), take(n3, 1024, l2 and grad), take(n3, 1024, l2)
+        self.n_bf16 = o
+
+        o = 0
+
+        def take_i(per_bh, on=True):
+            nonlocal o
+            if not on:
+                return None
+            at = o
+            o = _align(o + BH * per_bh, 64)
+            return at
+
+        self.wl_f = lib.work_list_len(n1, n1, T, CHUNK_FINE)
+        self.wl_c = lib.work_list_len(n2, n2, T2, CHUNK_COARSE) if l2 else 0
+        self.idx, self.pidx = take_i(n1 * T), take_i(n2 * T2, l2)
+        self.off, self.flat, self.work = take_i(n1 + 1, grad), take_i(n1 * T, grad), take_i(self.wl_f, grad)
+        self.poff, self.pflat, self.pwork = (take_i(n2 + 1, grad and l2), take_i(n2 * T2, grad and l2),
+                                             take_i(self.wl_c, grad and l2))
+        self.n_i32 = o
+        # backward arena (bytes): pooled gradients, then the kernels' workspace
+        self.ws_bytes = lib.attn_bwd_workspace_bytes(B, H, N, T, T2, levels)
+        self.dpk = 0
+        self.dpv = _align(BH * n1 * 128, 256)
+        self.dpk2 = self.dpv + _align(BH * n1 * 128, 256)
+        self.dpv2 = self.dpk2 + _align(BH * n2 * 128, 256)
+        self.ws = self.dpv2 + _align(BH * n2 * 128, 256)
+        self.n_bwd = self.ws + self.ws_bytes
+
+
+_layouts = {}
+
+
+def _layout(lib, B, H, N, levels, T, T2, grad):
+    key = (id(lib), B, H, N, levels, T, T2, grad)
+    lay = _layouts.get(key)
+    if lay is None:
+        if len(_layouts) > 64:
+            _layouts.clear()
+        lay = _layouts[key] = _Layout(lib, B, H, N, levels, T, T2, grad)
+    return lay
+
+
+def _stream(lib, t):
+    if not lib.device_library:
+        return None
+    idx = t.device.index
+    return C.c_void_p(torch._C._cuda_getCurrentRawStream(torch.cuda.current_device() if idx is None else idx))
+
+
+def _check(lib, rc, what):
+    if rc != 0:
+        lib.check(rc, what)
+
+
+class LlsaFused(Function):
+    """forward(q, k, v, levels, topk1, topk2, block_size, freq) -> o"""
+
+    @staticmethod
+    def forward(ctx, q, k, v, levels, topk1, topk2, block_size, freq):
+        lib = current_lib()
+        if block_size != 16:
+            raise NotImplementedError("block_size must be 16")
+        for t in (q, k, v):
+            if lib.device_library and not t.is_cuda:
+                raise RuntimeError("llsa_amd runs on an AMD GPU only (got a CPU tensor); there is no CPU implementation")
+            if t.dtype != torch.bfloat16:
+                raise NotImplementedError(f"llsa_amd attention kernels are bf16 only (got {t.dtype})")
+        if q.dim() != 4 or q.shape[-1] != 64:
+            raise NotImplementedError(f"llsa_amd attention kernels need (B,H,N,64) tensors (got {tuple(q.shape)})")
+        if k.shape != q.shape or v.shape != q.shape:
+            raise ValueError("self-attention only: q, k, v must have the same shape")
+        B, H, N, _ = q.shape
+        mult = 1024 if levels == 1 else 16384
+        if N % mult != 0:
+            raise ValueError(f"llsa_l{levels} needs a token count that is a multiple of {mult} (got {N})")
+        n1, n2 = N // 16, N // 256
+        T = min(topk1, n1)
+        T2 = min(topk2, n2) if levels == 2 else 0
+        rope = freq is not None
+        if rope:
+            if freq.dtype != torch.bfloat16 or tuple(freq.shape) != (N, 64):
+                raise ValueError("rope table must be bf16 (N, 64)")
+            freq = freq.contiguous()
+        grad = any(ctx.needs_input_grad[:3])
+        q, k, v = (t if _rows_ok(t) else t.contiguous() for t in (q, k, v))
+        lay = _layout(lib, B, H, N, levels, T, T2, grad)
+        dev = q.device
+        A = torch.empty(lay.n_bf16, device=dev, dtype=torch.bfloat16)
+        I = torch.empty(lay.n_i32, device=dev, dtype=torch.int32)
+        o = torch.empty_like(q) if all(s % 4 == 0 for s in q.stride()[:-1]) else torch.empty(q.shape, device=dev, dtype=q.dtype)
+        lse = torch.empty(B, H, N, device=dev, dtype=torch.float32)
+        a0, i0 = A.data_ptr(), I.data_ptr()
+        pa = lambda off: None if off is None else a0 + 2 * off
+        pi = lambda off: None if off is None else i0 + 4 * off
+        stream = _stream(lib, q)
+        l2 = levels == 2
+
+        items = (PoolItem * 3)(
+            PoolItem(q.data_ptr(), q.stride(0), q.stride(1), q.stride(2), N, int(rope), pa(lay.pq), pa(lay.pq2), pa(lay.qr),
+                     None, None, None, None),
+            PoolItem(k.data_ptr(), k.stride(0), k.stride(1), k.stride(2), N, int(rope), pa(lay.pk), pa(lay.pk2), pa(lay.kr),
+                     None, pa(lay.pkr), None, None),
+            PoolItem(v.data_ptr(), v.stride(0), v.stride(1), v.stride(2), N, 0, pa(lay.pv), pa(lay.pv2), pa(lay.vr),
+                     pa(lay.vt), pa(lay.pvr), pa(lay.pvt), None))
+        _check(lib, lib.pool_pyramid_fwd(items, 3, freq.data_ptr() if rope else None, B, H, stream), "pool_pyramid")
+        if l2:
+            s2 = (H * n2 * 64, n2 * 64, 64)
+            items2 = (PoolItem * 2)(
+                PoolItem(pa(lay.pk2), *s2, n2, 0, None, None, pa(lay.pk2r), None, None, None, None),
+                PoolItem(pa(lay.pv2), *s2, n2, 0, None, None, pa(lay.pv2r), pa(lay.pv2t), None, None, None))
+            _check(lib, lib.pool_pyramid_fwd(items2, 2, None, B, H, stream), "pool_pyramid (level-2 tiles)")
+            _check(lib, lib.topk_dense(pa(lay.pq2), pa(lay.pk2), pi(lay.pidx), B, H, n2, T2, 1, stream), "gen_sparse_indices")
+            _check(lib, lib.topk_sparse(pa(lay.pq), pa(lay.pk), pi(lay.pidx), pi(lay.idx), B, H, n1, T, T2, stream),
+                   "compute_topk_indices_sparse")
+        else:
+            _check(lib, lib.topk_dense(pa(lay.pq), pa(lay.pk), pi(lay.idx), B, H, n1, T, 1, stream), "gen_sparse_indices")
+
+        event = None
+        if grad:        # the lists of the backward: on a second stream, beside the attention kernel
+            s_lists = stream
+            if lib.device_library:
+                cur = torch.cuda.current_stream(dev)
+                side, event = _side.get(dev, (None, None))
+                if side is None:
+                    side, event = _side[dev] = (torch.cuda.Stream(device=dev), torch.cuda.Event())
+                side.wait_stream(cur)
+                s_lists = C.c_void_p(side.cuda_stream)
+            _check(lib, lib.transpose_indices(pi(lay.idx), pi(lay.off), pi(lay.flat), pi(lay.work), B, H, n1, n1, T, CHUNK_FINE,
+                                              s_lists), "transpose_indices")
+            if l2:
+                _check(lib, lib.transpose_indices(pi(lay.pidx), pi(lay.poff), pi(lay.pflat), pi(lay.pwork), B, H, n2, n2, T2,
+                                                  CHUNK_COARSE, s_lists), "transpose_indices (coarse)")
+            if event is not None:
+                event.record(side)
+
+        f = AttnFwdArgs()
+        f.qr, f.kr, f.vt, f.pkr, f.pvt = pa(lay.qr), pa(lay.kr), pa(lay.vt), pa(lay.pkr), pa(lay.pvt)
+        f.pk2r, f.pv2t, f.pidx = pa(lay.pk2r), pa(lay.pv2t), pi(lay.pidx)
+        f.idx = pi(lay.idx)
+        f.o, f.sob, f.soh, f.son = o.data_ptr(), o.stride(0), o.stride(1), o.stride(2)
+        f.lse = lse.data_ptr()
+        f.B, f.H, f.N, f.T, f.T2, f.levels = B, H, N, T, T2, levels
+        f.w1, f.w2 = 16.0, 256.0
+        _check(lib, lib.attn_fwd(C.byref(f), stream), "attn_fwd")
+        if event is not None:
+            cur.wait_event(event)
+
+        if grad:
+            ctx.save_for_backward(A, I, o, lse, freq)
+            ctx.meta = (lib, lay, B, H, N, T, T2, levels, q.shape, q.stride(), k.stride(), v.stride())
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        A, I, o, lse, freq = ctx.saved_tensors
+        lib, lay, B, H, N, T, T2, levels, shape, sq, sk, sv = ctx.meta
+        dev = o.device
+        if not _rows_ok(do):
+            do = do.contiguous()
+
+        def like(strides):      # gradients have the layout of their primals when the 8-byte stores allow it
+            if all(s % 4 == 0 for s in strides[:-1]) and strides[-1] == 1:
+                return torch.empty_strided(shape, strides, device=dev, dtype=torch.bfloat16)
+            return torch.empty(shape, device=dev, dtype=torch.bfloat16)
+
+        dq, dk, dv = like(sq), like(sk), like(sv)
+        W = torch.empty(lay.n_bwd, device=dev, dtype=torch.uint8)
+        a0, i0, w0 = A.data_ptr(), I.data_ptr(), W.data_ptr()
+        pa = lambda off: None if off is None else a0 + 2 * off
+        pi = lambda off: None if off is None else i0 + 4 * off
+        a = AttnBwdArgs()
+        a.dout, a.sdob, a.sdoh, a.sdon = do.data_ptr(), do.stride(0), do.stride(1), do.stride(2)
+        a.o, a.sob, a.soh, a.son = o.data_ptr(), o.stride(0), o.stride(1), o.stride(2)
+        a.lse = lse.data_ptr()
+        a.qr, a.kr, a.vr, a.pkr, a.pvr = pa(lay.qr), pa(lay.kr), pa(lay.vr), pa(lay.pkr), pa(lay.pvr)
+        a.pk2r, a.pv2r = pa(lay.pk2r), pa(lay.pv2r)
+        a.idx, a.pidx = pi(lay.idx), pi(lay.pidx)
+        a.off, a.flat, a.work = pi(lay.off), pi(lay.flat), pi(lay.work)
+        a.poff, a.pflat, a.pwork = pi(lay.poff), pi(lay.pflat), pi(lay.pwork)
+        a.dq, a.sdqb, a.sdqh, a.sdqn = dq.data_ptr(), dq.stride(0), dq.stride(1), dq.stride(2)
+        a.dk, a.sdkb, a.sdkh, a.sdkn = dk.data_ptr(), dk.stride(0), dk.stride(1), dk.stride(2)
+        a.dv, a.sdvb, a.sdvh, a.sdvn = dv.data_ptr(), dv.stride(0), dv.stride(1), dv.stride(2)
+        a.dpk, a.dpv = w0 + lay.dpk, w0 + lay.dpv
+        if levels == 2:
+            a.dpk2, a.dpv2 = w0 + lay.dpk2, w0 + lay.dpv2
+        a.workspace, a.workspace_bytes = w0 + lay.ws, lay.ws_bytes
+        if freq is not None:
+            a.freq_dq = a.freq_dk = freq.data_ptr()
+        a.B, a.H, a.N, a.T, a.T2, a.levels = B, H, N, T, T2, levels
+        # llsa_l1 keeps the reference's quirk: its pooled path is differentiated with weight 1
+        # (sparse_attention_res_1.py:388-389) although the forward uses token_weight
+        a.w1, a.w2, a.cgw1 = 16.0, 256.0, (16.0 if levels == 2 else 1.0)
+        a.stages, a.fold_pooled = 0, 1
+        _check(lib, lib.attn_bwd(C.byref(a), _stream(lib, o)), "attn_bwd")
+        return dq, dk, dv, None, None, None, None, None
+
+
+def selection(out):
+    """The blocks the forward that produced `out` chose: (indices (B,H,N/16,T), p_indices
+    (B,H,N/256,T2) or None), int32 views of the arena its autograd node holds."""
+    node = out.grad_fn
+    I = node.saved_tensors[1]
+    _, lay, B, H, N, T, T2, levels = node.meta[:8]
+    idx = I[lay.idx:lay.idx + B * H * lay.n1 * T].view(B, H, lay.n1, T)
+    pidx = I[lay.pidx:lay.pidx + B * H * lay.n2 * T2].view(B, H, lay.n2, T2) if levels == 2 else None
+    return idx, pidx

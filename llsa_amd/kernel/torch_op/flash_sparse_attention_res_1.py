@@ -12,8 +12,8 @@ from __future__ import annotations
 import torch
 from torch.autograd import Function
 
-from ..hip.indices_transpose import BackwardLists
-from ..hip.mean_pool import PoolSpec, mean_pool1d, pool_pyramid
+from ..hip.mean_pool import mean_pool1d
+from ._fused import LlsaFused
 from ..hip.sparse_attention_res_1 import sparse_indices_attn_res_fwd, sparse_indices_attn_res_scatter_bwd_v2
 from ..hip.topk import gen_sparse_indices
 
@@ -42,48 +42,9 @@ class FlashSparseResidualAttentionL1(Function):
 flash_sparse_residual_attention_l1_op = FlashSparseResidualAttentionL1.apply
 
 
-class _LlsaL1Fused(Function):
-    """llsa_l1 as one autograd node: pooling pyramid (+RoPE, + the operand tiles the kernels
-    read) in one pass, selection, attention; the backward folds the pooled gradients into
-    dk / dv (what mean_pool's backward and autograd's accumulation do in the reference) and
-    rotates dq / dk back."""
-
-    @staticmethod
-    def forward(ctx, q, k, v, topk, block_size, freq):
-        if block_size != 16:
-            raise NotImplementedError("block_size must be 16")
-        g = any(ctx.needs_input_grad[:3])
-        rope = freq is not None
-        oq, ok, ov = pool_pyramid([PoolSpec(q, y1=True, xr=True, rope=rope),
-                                   PoolSpec(k, y1=True, xr=True, y1r=True, rope=rope),
-                                   PoolSpec(v, y1=True, xr=g, xt=True, y1r=g, y1t=True)], freq)
-        pq, pk, pv = oq["y1"], ok["y1"], ov["y1"]
-        indices = gen_sparse_indices(pq, pk, topk)
-        tiles = dict(qr=oq["xr"], kr=ok["xr"], vt=ov["xt"], pkr=ok["y1r"], pvt=ov["y1t"])
-        # q / k are only shape-and-stride templates below: the kernels read the (rotated) tiles
-        lists = BackwardLists(indices) if g else None                 # on a second stream, beside the attention kernel
-        o, m = sparse_indices_attn_res_fwd(q, k, v, pk, pv, indices, indices.shape[-1], block_size, 4, tiles=tiles)
-        if g:
-            ctx.save_for_backward(q, k, v, pk, pv, o, m, indices, freq, oq["xr"], ok["xr"], ov["xr"], ok["y1r"], ov["y1r"],
-                                  *lists.join())
-        ctx.block_size = block_size
-        ctx.indices = indices
-        return o
-
-    @staticmethod
-    def backward(ctx, do):
-        q, k, v, pk, pv, o, m, indices, freq, qr, kr, vr, pkr, pvr, *csr = ctx.saved_tensors
-        bs = ctx.block_size
-        tiles = dict(qr=qr, kr=kr, vr=vr, pkr=pkr, pvr=pvr)
-        dq, dk, dv, _, dpk, dpv = sparse_indices_attn_res_scatter_bwd_v2(
-            do, q, k, v, pk, pv, o, m, indices, indices.shape[-1], bs, bs, tiles=tiles, freq_dq=freq,
-            fold_pooled=True, freq_dk=freq, csr=csr)       # dk, dv arrive with the pooled gradients folded in
-        return dq, dk, dv, None, None, None
-
-
 def llsa_l1(q, k, v, topk=8, block_size=16, rope=None):
     """flash_sparse_attention_res_1.py:41-47."""
-    return _LlsaL1Fused.apply(q, k, v, topk, block_size, rope)
+    return LlsaFused.apply(q, k, v, 1, topk, 0, block_size, rope)
 
 
 def llsa_l1_unfused(q, k, v, topk=8, block_size=16):

@@ -327,6 +327,7 @@ def check_op_l1(dev, B=1, H=2, N=1024, T=8, fused=True, rope=False, strided=Fals
     indices the device selected (selection itself is checked separately)."""
     from llsa_amd.kernel.hip.rope import my_rope_fn
     from llsa_amd.kernel.torch_op import flash_sparse_attention_res_1 as M
+    from llsa_amd.kernel.torch_op._fused import selection
     from llsa_amd.utils.rope_table import rope_table
     q, k, v, do = smooth_inputs(B, H, N, 64, dev) if smooth else randn_inputs(B, H, N, 64, dev, seed=19, strided=strided)
     freq = rope_table(int(math.isqrt(N)), dtype=torch.bfloat16).to(dev) if rope else None
@@ -335,7 +336,7 @@ def check_op_l1(dev, B=1, H=2, N=1024, T=8, fused=True, rope=False, strided=Fals
     def run(q_, k_, v_):
         if fused:
             out = M.llsa_l1(q_, k_, v_, T, 16, rope=freq)
-            captured["idx"] = out.grad_fn.indices
+            captured["idx"] = selection(out)[0]
             return out
         if rope:
             q_, k_ = my_rope_fn(q_, freq), my_rope_fn(k_, freq)
@@ -366,6 +367,7 @@ def check_op_l1(dev, B=1, H=2, N=1024, T=8, fused=True, rope=False, strided=Fals
 def check_op_l2(dev, B=1, H=1, N=16384, T=8, T2=4, fused=True, rope=False, smooth=False):
     from llsa_amd.kernel.hip.rope import my_rope_fn
     from llsa_amd.kernel.torch_op import flash_sparse_attention_res_2 as M
+    from llsa_amd.kernel.torch_op._fused import selection
     from llsa_amd.utils.rope_table import rope_table
     q, k, v, do = smooth_inputs(B, H, N, 64, dev) if smooth else randn_inputs(B, H, N, 64, dev, seed=20)
     freq = rope_table(int(math.isqrt(N)), dtype=torch.bfloat16).to(dev) if rope else None
@@ -374,7 +376,7 @@ def check_op_l2(dev, B=1, H=1, N=16384, T=8, T2=4, fused=True, rope=False, smoot
     def run(q_, k_, v_):
         if fused:
             out = M.llsa_l2(q_, k_, v_, T, T2, 16, rope=freq)
-            captured["idx"], captured["pidx"] = out.grad_fn.indices, out.grad_fn.p_indices
+            captured["idx"], captured["pidx"] = selection(out)
             return out
         if rope:
             q_, k_ = my_rope_fn(q_, freq), my_rope_fn(k_, freq)
