@@ -259,7 +259,8 @@ __global__ __launch_bounds__(1024) void topk_dense_radix_kernel(const bf16* __re
             out + ((int64_t)bh * n + q0 + row) * T, lane);
 }
 
-__global__ __launch_bounds__(1024) void topk_sparse_kernel(const bf16* __restrict__ pq, const bf16* __restrict__ pk,
+constexpr int kSparseWaves = 8;       // two rows per wave: four workgroups fit a CU and the grid is one round
+__global__ __launch_bounds__(64 * kSparseWaves) void topk_sparse_kernel(const bf16* __restrict__ pq, const bf16* __restrict__ pk,
                                                            const int* __restrict__ pidx, int* __restrict__ out, int N1,
                                                            int T, int T2) {
     __shared__ unsigned su[16][kMaxCand + 1];
@@ -273,20 +274,20 @@ __global__ __launch_bounds__(1024) void topk_sparse_kernel(const bf16* __restric
     const bf16* pqb = pq + ((int64_t)bh * N1 + G * kBlk) * kD;
     const bf16* pkb = pk + (int64_t)bh * N1 * kD;
 
-    for (int i = tid; i < C; i += 1024)
+    for (int i = tid; i < C; i += 64 * kSparseWaves)
         cand[i] = clampi(pidx[((int64_t)bh * N2 + G) * T2 + i / kBlk], 0, N2 - 1) * kBlk + (i % kBlk);
     bf16x8 bq[2];
     bq[0] = ld16(pqb + (lane & 15) * kD + (lane >> 4) * 8);
     bq[1] = ld16(pqb + (lane & 15) * kD + (lane >> 4) * 8 + 32);
     __syncthreads();
 
-    for (int a = wave; a < T2; a += 16) {
+    for (int a = wave; a < T2; a += kSparseWaves) {
         f32x4 s = score_tile(pkb + (int64_t)cand[a * kBlk] * kD, bq);
 #pragma unroll
         for (int e = 0; e < 4; e++) su[lane & 15][a * kBlk + 4 * (lane >> 4) + e] = ordered_bits(s[e]);
     }
     __syncthreads();
-    for (int row = wave; row < 16; row += 16)
+    for (int row = wave; row < 16; row += kSparseWaves)
         wave_topk_radix_any(
             su[row], C, T, [&](int pos) { return cand[pos]; }, sel_u[wave], sel_i[wave],
             out + ((int64_t)bh * N1 + G * kBlk + row) * T, lane);
@@ -323,7 +324,7 @@ extern "C" int llsa_topk_sparse(const void* pq, const void* pk, const int32_t* p
     LLSA_REQUIRE(T2 >= 1 && T2 * 16 <= kMaxCand && T2 <= N1 / 16, "topk_sparse: need 1 <= T2 <= min(%d, N1/16), got %d", kMaxCand / 16, T2);
     LLSA_REQUIRE(T >= 1 && T <= kMaxT && T <= T2 * 16, "topk_sparse: need 1 <= T <= min(%d, 16*T2), got %d", kMaxT, T);
     LLSA_REQUIRE(aligned16(pq) && aligned16(pk), "topk_sparse: inputs must be 16-byte aligned");
-    hipLaunchKernelGGL(topk_sparse_kernel, dim3(N1 / 16, B * H), dim3(1024), 0, (hipStream_t)stream, (const bf16*)pq,
+    hipLaunchKernelGGL(topk_sparse_kernel, dim3(N1 / 16, B * H), dim3(64 * kSparseWaves), 0, (hipStream_t)stream, (const bf16*)pq,
                        (const bf16*)pk, parent_idx, out_idx, N1, T, T2);
     return launch_status("topk_sparse");
 }
