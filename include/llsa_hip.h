@@ -146,8 +146,13 @@ int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, 
  * given: every key block's segment is cut into chunks of at most `chunk` entries, one work item
  * per chunk, so that a key block selected by very many query blocks is spread over many waves
  * (the reference walks each segment serially, sparse_attention_res_1.py:300-322).  `work` is
- * (B,H,llsa_work_list_len(Mb,Kb,T,chunk)) int32; llsa_attn_bwd needs chunk = LLSA_CHUNK_FINE
- * for idx and chunk = LLSA_CHUNK_COARSE for pidx. */
+ * (B,H,llsa_work_list_len(Mb,Kb,T,chunk)) int32, 16-byte aligned; llsa_attn_bwd needs
+ * chunk = LLSA_CHUNK_FINE for idx and chunk = LLSA_CHUNK_COARSE for pidx.  Per (b,h), in int32:
+ *   [0] items, [1] partial-sum slots, [2] key blocks with more than one chunk, [3] 0
+ *   [4 + 4i ..]              item i = {key block, first entry in flat, entries, partial-sum slot or -1};
+ *                            items with more than chunk/2 entries come first
+ *   [4 + 4*max_items + 4j ..] j-th key block with more than one chunk = {key block, first slot, chunks, 0}
+ * with max_items = Mb*T/chunk + Kb; every key block has at least one item. */
 int64_t llsa_work_list_len(int Mb, int Kb, int T, int chunk);
 #define LLSA_CHUNK_FINE 64
 #define LLSA_CHUNK_COARSE 8
