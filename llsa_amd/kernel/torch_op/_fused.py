@@ -23,7 +23,7 @@ from torch.autograd import Function
 
 from ..._lib import CHUNK_COARSE, CHUNK_FINE, AttnBwdArgs, AttnFwdArgs, PoolItem, current_lib
 
-_side = {}          # device -> (second stream, event)
+_side = {}          # device -> (second stream, two events)
 
 
 def _rows_ok(t):
@@ -176,23 +176,17 @@ class LlsaFused(Function):
         else:
             _check(lib, lib.topk_dense(pa(lay.pq), pa(lay.pk), pi(lay.idx), B, H, n1, T, 1, stream), "gen_sparse_indices")
 
-        event = None
-        if grad:        # the lists of the backward: on a second stream, beside the attention kernel
-            s_lists = stream
-            if lib.device_library:
-                cur = torch.cuda.current_stream(dev)
-                side, event = _side.get(dev, (None, None))
-                if side is None:
-                    side, event = _side[dev] = (torch.cuda.Stream(device=dev), torch.cuda.Event())
-                side.wait_stream(cur)
-                s_lists = C.c_void_p(side.cuda_stream)
-            _check(lib, lib.transpose_indices(pi(lay.idx), pi(lay.off), pi(lay.flat), pi(lay.work), B, H, n1, n1, T, CHUNK_FINE,
-                                              s_lists), "transpose_indices")
-            if l2:
-                _check(lib, lib.transpose_indices(pi(lay.pidx), pi(lay.poff), pi(lay.pflat), pi(lay.pwork), B, H, n2, n2, T2,
-                                                  CHUNK_COARSE, s_lists), "transpose_indices (coarse)")
-            if event is not None:
-                event.record(side)
+        # The lists of the backward go to a second stream, beside the attention kernel.  The attention
+        # kernel is issued first (the GPU is waiting for it); an event recorded before it lets the
+        # second stream start as soon as the selection is done.
+        cur = side = None
+        if grad and lib.device_library:
+            cur = torch.cuda.current_stream(dev)
+            pack = _side.get(dev)
+            if pack is None:
+                pack = _side[dev] = (torch.cuda.Stream(device=dev), torch.cuda.Event(), torch.cuda.Event())
+            side, ev_idx, ev_lists = pack
+            ev_idx.record(cur)
 
         f = AttnFwdArgs()
         f.qr, f.kr, f.vt, f.pkr, f.pvt = pa(lay.qr), pa(lay.kr), pa(lay.vt), pa(lay.pkr), pa(lay.pvt)
@@ -203,8 +197,20 @@ class LlsaFused(Function):
         f.B, f.H, f.N, f.T, f.T2, f.levels = B, H, N, T, T2, levels
         f.w1, f.w2 = 16.0, 256.0
         _check(lib, lib.attn_fwd(C.byref(f), stream), "attn_fwd")
-        if event is not None:
-            cur.wait_event(event)
+
+        if grad:
+            s_lists = stream
+            if side is not None:
+                side.wait_event(ev_idx)         # (the arena is older than the selection, so this covers it too)
+                s_lists = C.c_void_p(side.cuda_stream)
+            _check(lib, lib.transpose_indices(pi(lay.idx), pi(lay.off), pi(lay.flat), pi(lay.work), B, H, n1, n1, T, CHUNK_FINE,
+                                              s_lists), "transpose_indices")
+            if l2:
+                _check(lib, lib.transpose_indices(pi(lay.pidx), pi(lay.poff), pi(lay.pflat), pi(lay.pwork), B, H, n2, n2, T2,
+                                                  CHUNK_COARSE, s_lists), "transpose_indices (coarse)")
+            if side is not None:
+                ev_lists.record(side)
+                cur.wait_event(ev_lists)
 
         if grad:
             ctx.save_for_backward(A, I, o, lse, freq)
