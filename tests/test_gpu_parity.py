@@ -79,6 +79,13 @@ def test_attn_l1_small(dev):
     P.check_attn_l1(dev, B=1, H=2, N=1024, T=8)
 
 
+def test_attn_more_than_64_selected(dev):
+    """top-k above 64: the kernels fetch the indices of a query block 64 at a time, and every key
+    block's list (128 entries here: every query block selects every key block) has two chunks."""
+    P.check_attn_l1(dev, B=1, H=2, N=2048, T=128)
+    P.check_attn_reduces_to_sdpa(dev, B=1, H=1, N=2048)
+
+
 def test_attn_hot_blocks(dev):
     P.check_attn_l1(dev, B=1, H=2, N=4096, T=8, hot=5)
     P.check_attn_l2(dev, B=1, H=1, N=16384, T=8, T2=8, hot=3)
