@@ -130,9 +130,11 @@ __device__ __forceinline__ unsigned ordered_bits(float f) {
 // Each lane keeps its E entries (positions lane, lane + 64, ...) in registers, so a bit step is
 // E compares + ballots + scalar popcounts with no memory access.
 // sel_u / sel_i: 64 entries of LDS scratch each.  out[0..T): result, global memory.
+// low_bit: the keys' bits below it are known to be zero (16 for scores rounded to bf16) and are not
+// looked at; idx_bits: the global indices are below 2^idx_bits (the tie pass starts there).
 template <int E, typename IdxFn>
 __device__ __forceinline__ void wave_topk_radix(const unsigned* u, int npos, int T, IdxFn gidx_of, unsigned* sel_u,
-                                                int* sel_i, int* out, int lane) {
+                                                int* sel_i, int* out, int lane, int low_bit, int idx_bits) {
     unsigned uk[E];
     unsigned gk[E];
     bool ok[E];
@@ -149,7 +151,7 @@ __device__ __forceinline__ void wave_topk_radix(const unsigned* u, int npos, int
     // not be looked at (tau = prefix with zero low bits then selects exactly those).
     unsigned prefix = 0;
     int remaining = T, match = npos;
-    for (int bit = 31; bit >= 0 && match != remaining; bit--) {
+    for (int bit = 31; bit >= low_bit && match != remaining; bit--) {
         const unsigned msk = (bit == 31) ? 0x80000000u : ((0xFFFFFFFFu << (bit + 1)) | (1u << bit));
         const unsigned want = prefix | (1u << bit);
         int cnt1 = 0;
@@ -171,7 +173,7 @@ __device__ __forceinline__ void wave_topk_radix(const unsigned* u, int npos, int
     if (n_eq > remaining) {                                   // ties at the threshold: keep the smallest indices
         unsigned p2 = 0;
         int rem2 = remaining;
-        for (int bit = 30; bit >= 0; bit--) {
+        for (int bit = idx_bits - 1; bit >= 0; bit--) {
             const unsigned msk = (0xFFFFFFFFu << (bit + 1)) | (1u << bit);
             int cnt0 = 0;
 #pragma unroll
@@ -221,12 +223,12 @@ __device__ __forceinline__ void wave_topk_radix(const unsigned* u, int npos, int
 // entries per lane as a compile-time bound: 1, 2, 4, 8 or 16
 template <typename IdxFn>
 __device__ __forceinline__ void wave_topk_radix_any(const unsigned* u, int npos, int T, IdxFn gidx_of, unsigned* sel_u,
-                                                    int* sel_i, int* out, int lane) {
-    if (npos <= 64) wave_topk_radix<1>(u, npos, T, gidx_of, sel_u, sel_i, out, lane);
-    else if (npos <= 128) wave_topk_radix<2>(u, npos, T, gidx_of, sel_u, sel_i, out, lane);
-    else if (npos <= 256) wave_topk_radix<4>(u, npos, T, gidx_of, sel_u, sel_i, out, lane);
-    else if (npos <= 512) wave_topk_radix<8>(u, npos, T, gidx_of, sel_u, sel_i, out, lane);
-    else wave_topk_radix<16>(u, npos, T, gidx_of, sel_u, sel_i, out, lane);
+                                                    int* sel_i, int* out, int lane, int low_bit, int idx_bits) {
+    if (npos <= 64) wave_topk_radix<1>(u, npos, T, gidx_of, sel_u, sel_i, out, lane, low_bit, idx_bits);
+    else if (npos <= 128) wave_topk_radix<2>(u, npos, T, gidx_of, sel_u, sel_i, out, lane, low_bit, idx_bits);
+    else if (npos <= 256) wave_topk_radix<4>(u, npos, T, gidx_of, sel_u, sel_i, out, lane, low_bit, idx_bits);
+    else if (npos <= 512) wave_topk_radix<8>(u, npos, T, gidx_of, sel_u, sel_i, out, lane, low_bit, idx_bits);
+    else wave_topk_radix<16>(u, npos, T, gidx_of, sel_u, sel_i, out, lane, low_bit, idx_bits);
 }
 
 constexpr int kRadixMaxN = 1024;      // keys per row the radix kernels keep in LDS
@@ -250,13 +252,16 @@ __global__ __launch_bounds__(1024) void topk_dense_radix_kernel(const bf16* __re
         f32x4 s = score_tile(pkb + (int64_t)tile * 16 * kD, bq);
 #pragma unroll
         for (int e = 0; e < 4; e++)
-            su[(lane & 15) * stride + tile * 16 + 4 * (lane >> 4) + e] = ordered_bits(round_scores ? rn_bf16(s[e]) : s[e]);
+            // (a score rounded to bf16 has 16 constant low key bits -- ones when negative; cleared, the
+            // selection below need not look at them)
+            su[(lane & 15) * stride + tile * 16 + 4 * (lane >> 4) + e] =
+                round_scores ? (ordered_bits(rn_bf16(s[e])) & 0xFFFF0000u) : ordered_bits(s[e]);
     }
     __syncthreads();
     for (int row = wave; row < 16; row += 16)
         wave_topk_radix_any(
             su + row * stride, n, T, [](int pos) { return pos; }, sel_u[wave], sel_i[wave],
-            out + ((int64_t)bh * n + q0 + row) * T, lane);
+            out + ((int64_t)bh * n + q0 + row) * T, lane, round_scores ? 16 : 0, 32 - __builtin_clz(n - 1));
 }
 
 constexpr int kSparseWaves = 8;       // two rows per wave: four workgroups fit a CU and the grid is one round
@@ -290,7 +295,7 @@ __global__ __launch_bounds__(64 * kSparseWaves) void topk_sparse_kernel(const bf
     for (int row = wave; row < 16; row += kSparseWaves)
         wave_topk_radix_any(
             su[row], C, T, [&](int pos) { return cand[pos]; }, sel_u[wave], sel_i[wave],
-            out + ((int64_t)bh * N1 + G * kBlk + row) * T, lane);
+            out + ((int64_t)bh * N1 + G * kBlk + row) * T, lane, 0, 32 - __builtin_clz(N1 - 1));
 }
 
 }  // namespace llsa
