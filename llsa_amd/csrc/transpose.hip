@@ -37,6 +37,10 @@ __device__ __forceinline__ int wave_incl_scan(int v, int lane) {
 __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int* __restrict__ idx, int* __restrict__ offsets,
                                                                       int* __restrict__ flat, int* __restrict__ work,
                                                                       int Mb, int Kb, int T, int chunk, int work_stride) {
+    // These kernels run beside the forward attention kernel on a second stream and are on the
+    // critical path of nothing until the backward starts, but one slow workgroup per (b,h) is all
+    // there is of them: let their waves go first when they share a CU.
+    __builtin_amdgcn_s_setprio(3);
     HIP_DYNAMIC_SHARED(int, smem)
     int* pos = smem;                               // Kb
     int* wave_tot = smem + Kb;                     // 5 * kTrWaves
@@ -163,6 +167,7 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
 // entry in a private LDS bitmap over the query blocks and reads the bits back in order.
 __global__ __launch_bounds__(256) void sort_segments_kernel(const int* __restrict__ offsets, int* __restrict__ flat, int Mb,
                                                             int Kb, int T) {
+    __builtin_amdgcn_s_setprio(3);
     HIP_DYNAMIC_SHARED(unsigned, bitmaps)                     // 4 waves x words
     const int words = (Mb + 31) / 32;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;

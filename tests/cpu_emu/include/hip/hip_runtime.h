@@ -110,6 +110,7 @@ inline int __clz(int x) { return x ? __builtin_clz((unsigned)x) : 32; }
     __builtin_memcpy((char*)(l) + (size) * emu::lane_id(), (const char*)(g), (size))
 // the wave-wide effect of a wait (all lanes' copies into LDS have landed) needs a rendezvous of the lanes here
 #define __builtin_amdgcn_s_waitcnt(x) emu::wave_sync()
+#define __builtin_amdgcn_s_setprio(x) ((void)0)
 #define __builtin_amdgcn_fence(order, scope) ((void)0)
 #define hipFuncAttributeMaxDynamicSharedMemorySize 0
 template <typename F>
