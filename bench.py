@@ -137,8 +137,8 @@ def stage_profile(op, q, k, v, do, t1, t2, freq, iters, torch):
         # just filled with delta and the dO tiles); only its duration is used
         res[name] = timed(lambda: run(st), iters, torch)
     # the two launches that add up the partial sums of the K-side passes
-    res["bwd_reduce"] = timed(lambda: run(4 | 8 | 16), iters, torch) - res["bwd_dkv"] - res["bwd_dpkv_dense"] \
-        - res.get("bwd_dpkv1_sparse", 0.0)
+    res["bwd_reduce"] = max(0.0, timed(lambda: run(4 | 8 | 16), iters, torch) - res["bwd_dkv"] - res["bwd_dpkv_dense"]
+                            - res.get("bwd_dpkv1_sparse", 0.0))
     return res
 
 
