@@ -152,6 +152,7 @@ int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, 
  *   [4 + 4i ..]              item i = {key block, first entry in flat, entries, partial-sum slot or -1};
  *                            items with more than chunk/2 entries come first
  *   [4 + 4*max_items + 4j ..] j-th key block with more than one chunk = {key block, first slot, chunks, 0}
+ *   then Kb ints (rounded up to a multiple of 4) that the transpose itself uses as scratch
  * with max_items = Mb*T/chunk + Kb; every key block has at least one item. */
 int64_t llsa_work_list_len(int Mb, int Kb, int T, int chunk);
 #define LLSA_CHUNK_FINE 64

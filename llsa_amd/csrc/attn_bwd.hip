@@ -680,7 +680,7 @@ __global__ __launch_bounds__(256) void kside_reduce_kernel(ReduceParams rp) {
     const ReduceJob& jb = rp.job[j];
     const int step = reduce_slots(jb.max_units);
     const int* work = jb.work ? jb.work + (int64_t)bh * jb.work_stride : nullptr;
-    const int max_items = (int)(jb.work_stride - 4 - 4 * jb.max_units) / 4;
+    const int max_items = (int)(jb.work_stride - work_tail_len(jb.n_units) - 4 - 4 * jb.max_units) / 4;
     // the unit's record is fetched together with the count it is checked against (u0 is always
     // inside the list's storage): one memory round trip instead of two
     const int* multi = work ? work + 4 + 4 * max_items : nullptr;

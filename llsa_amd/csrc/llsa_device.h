@@ -131,6 +131,10 @@ __device__ __forceinline__ bf16x4 rope_bwd4(bf16x4 o, bf16x4 f) {
     return y;
 }
 
+// ints at the end of a (b,h)'s work list (see transpose.hip) that the transpose of many entries uses as
+// histogram, then as cursors
+__host__ __device__ inline int work_tail_len(int Kb) { return (Kb + 3) & ~3; }
+
 constexpr int kGroup = 4;      // pooled blocks per LDS buffer in the query-side attention kernels (one per wave)
 
 // 16- and 8-byte reads that are LDS reads by construction (ds_read_b128 / ds_read_b64)

@@ -22,6 +22,8 @@ __device__ __forceinline__ int wave_incl_scan(int v, int lane) {
     return v;
 }
 
+constexpr int kTrPart = 16 * kTrThreads;       // entries per workgroup of the split path
+
 // Work list (optional): the K-side kernels walk each key block's segment in chunks of at most
 // `chunk` entries so that a popular key block does not serialise on one wave.  Per (b,h), all
 // records 4 ints (16-byte aligned when the list is, so that one load fetches a record):
@@ -34,6 +36,11 @@ __device__ __forceinline__ int wave_incl_scan(int v, int lane) {
 // writes zeros), and max_items = Mb*T/chunk + Kb.  Items with more than chunk/2 entries come first
 // in the list: a wave walks its item serially, so the long ones have to start early or the kernel
 // ends with a few waves still working.
+// SPLIT = false: the whole job of one (b,h).  SPLIT = true (many entries): the middle step of three --
+// tr_count_kernel has left the histogram in the tail of the work list, this kernel scans it, writes
+// offsets and work list and leaves every segment's start in the same place as the cursor that
+// tr_scatter_kernel advances.
+template <bool SPLIT>
 __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int* __restrict__ idx, int* __restrict__ offsets,
                                                                       int* __restrict__ flat, int* __restrict__ work,
                                                                       int Mb, int Kb, int T, int chunk, int work_stride) {
@@ -43,7 +50,7 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
     __builtin_amdgcn_s_setprio(3);
     HIP_DYNAMIC_SHARED(int, smem)
     int* pos = smem;                               // Kb
-    int* wave_tot = smem + Kb;                     // 5 * kTrWaves
+    int* wave_tot = smem + (SPLIT ? 0 : Kb);       // 5 * kTrWaves (the split form keeps no counters in LDS)
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int bh = blockIdx.x;
@@ -52,11 +59,14 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
     flat += (int64_t)bh * E;
     offsets += (int64_t)bh * (Kb + 1);
 
-    for (int i = tid; i < Kb; i += kTrThreads) pos[i] = 0;
+    constexpr int kBatch = 16;
+    int* tail = SPLIT ? work + (int64_t)bh * work_stride + (work_stride - work_tail_len(Kb)) : nullptr;
+    if (!SPLIT) {
+        for (int i = tid; i < Kb; i += kTrThreads) pos[i] = 0;
+    }
     __syncthreads();
     // entries are taken 16 per thread at a time, all 16 loads issued before the first is used
-    constexpr int kBatch = 16;
-    for (int e0 = 0; e0 < E; e0 += kBatch * kTrThreads) {
+    for (int e0 = 0; e0 < (SPLIT ? 0 : E); e0 += kBatch * kTrThreads) {
         int v[kBatch];
 #pragma unroll
         for (int k = 0; k < kBatch; k++) {
@@ -76,7 +86,7 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
     const int long_min = chunk / 2 + 1;
     int local = 0, l_items = 0, l_slots = 0, l_multi = 0, l_long = 0;
     for (int i = c0; i < c1; i++) {
-        const int c = pos[i];
+        const int c = SPLIT ? tail[i] : pos[i];
         const int nch = max(1, (c + chunk - 1) / chunk);
         const int n_long = (nch - 1) + ((c - (nch - 1) * chunk >= long_min) ? 1 : 0);   // all chunks but the last are full
         local += c;
@@ -114,9 +124,10 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
     if (work != nullptr) work += (int64_t)bh * work_stride;
     const int max_items = E / chunk + Kb;
     for (int i = c0; i < c1; i++) {
-        const int c = pos[i];
+        const int c = SPLIT ? tail[i] : pos[i];
         offsets[i] = run;
-        pos[i] = run;
+        if (SPLIT) tail[i] = run;
+        else pos[i] = run;
         run += c;
         if (work != nullptr) {
             const int nch = max(1, (c + chunk - 1) / chunk);
@@ -147,7 +158,7 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
     }
     __syncthreads();
 
-    for (int e0 = 0; e0 < E; e0 += kBatch * kTrThreads) {
+    for (int e0 = 0; e0 < (SPLIT ? 0 : E); e0 += kBatch * kTrThreads) {
         int v[kBatch];
 #pragma unroll
         for (int k = 0; k < kBatch; k++) {
@@ -161,6 +172,49 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
         }
     }
     // pos[n] is now the END of segment n; the segments are sorted by sort_segments_kernel
+}
+
+// Split path, first and last step: one workgroup per kTrPart entries.
+__global__ __launch_bounds__(kTrThreads) void tr_zero_kernel(int* __restrict__ work, int Kb, int work_stride) {
+    int* tail = work + (int64_t)blockIdx.x * work_stride + (work_stride - work_tail_len(Kb));
+    for (int i = threadIdx.x; i < Kb; i += kTrThreads) tail[i] = 0;
+}
+__global__ __launch_bounds__(kTrThreads) void tr_count_kernel(const int* __restrict__ idx, int* __restrict__ work, int E, int Kb,
+                                                             int work_stride) {
+    // (global atomics, no LDS histogram: this kernel runs beside the forward attention kernel, whose
+    // workgroups leave no room for 64 KB of LDS, and its workgroups would wait for that kernel to end)
+    __builtin_amdgcn_s_setprio(3);
+    const int tid = threadIdx.x, bh = blockIdx.y;
+    int* tail = work + (int64_t)bh * work_stride + (work_stride - work_tail_len(Kb));
+    idx += (int64_t)bh * E;
+    int v[16];
+#pragma unroll
+    for (int k = 0; k < 16; k++) {
+        const int e = blockIdx.x * kTrPart + k * kTrThreads + tid;
+        v[k] = (e < E) ? idx[e] : -1;
+    }
+#pragma unroll
+    for (int k = 0; k < 16; k++)
+        if (blockIdx.x * kTrPart + k * kTrThreads + tid < E) atomicAdd(&tail[clampi(v[k], 0, Kb - 1)], 1);
+}
+__global__ __launch_bounds__(kTrThreads) void tr_scatter_kernel(const int* __restrict__ idx, int* __restrict__ flat,
+                                                               int* __restrict__ work, int E, int Kb, int T, int work_stride) {
+    __builtin_amdgcn_s_setprio(3);
+    const int tid = threadIdx.x, bh = blockIdx.y;
+    int* cursor = work + (int64_t)bh * work_stride + (work_stride - work_tail_len(Kb));
+    idx += (int64_t)bh * E;
+    flat += (int64_t)bh * E;
+    int v[16];
+#pragma unroll
+    for (int k = 0; k < 16; k++) {
+        const int e = blockIdx.x * kTrPart + k * kTrThreads + tid;
+        v[k] = (e < E) ? idx[e] : -1;
+    }
+#pragma unroll
+    for (int k = 0; k < 16; k++) {
+        const int e = blockIdx.x * kTrPart + k * kTrThreads + tid;
+        if (e < E) flat[atomicAdd(&cursor[clampi(v[k], 0, Kb - 1)], 1)] = e / T;      // order inside a segment: sorted afterwards
+    }
 }
 
 // Puts every segment of `flat` in ascending order: one wave per key block sets one bit per
@@ -209,7 +263,7 @@ using namespace llsa;
 extern "C" int64_t llsa_work_list_len(int Mb, int Kb, int T, int chunk) {
     if (Mb <= 0 || Kb <= 0 || T <= 0 || chunk <= 0) return -1;
     const int64_t e = (int64_t)Mb * T;
-    return 4 + 4 * (e / chunk + Kb) + 4 * (e / chunk + 1);
+    return 4 + 4 * (e / chunk + Kb) + 4 * (e / chunk + 1) + work_tail_len(Kb);
 }
 
 extern "C" int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, int32_t* work, int B, int H, int Mb,
@@ -220,15 +274,30 @@ extern "C" int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int3
     if (chunk < 1) chunk = 1;
     const size_t lds = sizeof(int) * ((size_t)Kb + 128);
     static_assert(5 * kTrWaves <= 128, "wave totals must fit their LDS slot");
-    LLSA_REQUIRE(lds <= 160 * 1024, "transpose_indices: Kb=%d needs %zu bytes of LDS (limit 163840)", Kb, lds);
+    LLSA_REQUIRE(lds <= 160 * 1024 || (work != nullptr && (int64_t)Mb * T >= 4 * kTrPart),
+                 "transpose_indices: Kb=%d needs %zu bytes of LDS (limit 163840)", Kb, lds);
     const size_t lds_sort = sizeof(unsigned) * 4 * ((size_t)(Mb + 31) / 32);
     LLSA_REQUIRE(lds_sort <= 64 * 1024, "transpose_indices: Mb=%d needs %zu bytes of LDS for the segment sort", Mb, lds_sort);
-    if (lds > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute((const void*)transpose_indices_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    const int64_t E = (int64_t)Mb * T;
+    const bool split = work != nullptr && E >= 4 * kTrPart;
+    if (!split && lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void*)transpose_indices_kernel<false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return fail(-101, "transpose_indices: cannot raise dynamic LDS to %zu bytes: %s", lds, hipGetErrorString(e));
     }
-    hipLaunchKernelGGL(transpose_indices_kernel, dim3(B * H), dim3(kTrThreads), lds, (hipStream_t)stream, idx, offsets, flat, work, Mb, Kb, T, chunk,
-                       (int)llsa_work_list_len(Mb, Kb, T, chunk));
+    const int wl = (int)llsa_work_list_len(Mb, Kb, T, chunk);
+    hipStream_t st = (hipStream_t)stream;
+    if (split) {
+        // many entries: histogram and scatter spread over E / kTrPart workgroups per (b,h)
+        const int parts = (int)((E + kTrPart - 1) / kTrPart);
+        hipLaunchKernelGGL(tr_zero_kernel, dim3(B * H), dim3(kTrThreads), 0, st, work, Kb, wl);
+        hipLaunchKernelGGL(tr_count_kernel, dim3(parts, B * H), dim3(kTrThreads), 0, st, idx, work, (int)E, Kb, wl);
+        hipLaunchKernelGGL(HIP_KERNEL_NAME(transpose_indices_kernel<true>), dim3(B * H), dim3(kTrThreads), sizeof(int) * 128, st, idx,
+                           offsets, flat, work, Mb, Kb, T, chunk, wl);
+        hipLaunchKernelGGL(tr_scatter_kernel, dim3(parts, B * H), dim3(kTrThreads), 0, st, idx, flat, work, (int)E, Kb, T, wl);
+    } else {
+        hipLaunchKernelGGL(HIP_KERNEL_NAME(transpose_indices_kernel<false>), dim3(B * H), dim3(kTrThreads), lds, st, idx, offsets, flat,
+                           work, Mb, Kb, T, chunk, wl);
+    }
     hipLaunchKernelGGL(sort_segments_kernel, dim3((Kb + 3) / 4, B * H), dim3(256), lds_sort, (hipStream_t)stream,
                        (const int*)offsets, flat, Mb, Kb, T);
     return launch_status("transpose_indices");

@@ -180,12 +180,14 @@ def check_topk_sparse(dev, B=1, H=2, N1=256, T=8, T2=4):
     assert (idx == ref).all(-1)[o_ok].all(), "order differs on rows with well separated scores"
 
 
-def check_transpose(dev, B=2, H=2, Mb=64, T=8, Kb=None):
+def check_transpose(dev, B=2, H=2, Mb=64, T=8, Kb=None, chunk=0):
+    """chunk > 0 also asks for the work list, which with Mb*T >= 65536 entries switches the kernel to
+    its split form (histogram and scatter over many workgroups)."""
     from llsa_amd.kernel.hip.indices_transpose import transpose_indices
     g = torch.Generator().manual_seed(12)
     kb = Kb or Mb
     idx = torch.stack([torch.randperm(kb, generator=g)[:T] for _ in range(B * H * Mb)]).reshape(B, H, Mb, T).int()
-    off, flat = transpose_indices(idx.to(dev), Kb)
+    off, flat = transpose_indices(idx.to(dev), Kb, chunk)[:2]
     ro, rf = O.transpose_indices(idx.long(), Kb)
     assert torch.equal(off.cpu().long(), ro), "offsets differ"
     assert torch.equal(flat.cpu().long(), rf), "flat list differs"

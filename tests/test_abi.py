@@ -67,7 +67,7 @@ def test_entry_points_reject_bad_arguments(lib):
     assert b"multiple of 4" in lib.last_error_string()
     assert lib.attn_bwd_workspace_bytes(2, 6, 16384, 16, 16, 2) > 0
     assert lib.attn_bwd_workspace_bytes(2, 6, 16384, 16, 16, 3) < 0
-    assert lib.work_list_len(1024, 1024, 16, 32) == 4 + 4 * (512 + 1024) + 4 * 513
+    assert lib.work_list_len(1024, 1024, 16, 32) == 4 + 4 * (512 + 1024) + 4 * 513 + 1024
 
 
 def test_python_layer_rejects_unsupported_inputs():

@@ -50,6 +50,7 @@ def test_topk_sparse():
 def test_transpose():
     P.check_transpose(DEV, Mb=64, T=8)
     P.check_transpose(DEV, B=1, H=1, Mb=64, T=4, Kb=16)
+    P.check_transpose(DEV, B=1, H=2, Mb=4096, T=16, chunk=64)        # 65536 entries: the split form
     P.check_transpose_hot_block(DEV)
 
 

@@ -68,6 +68,7 @@ def test_transpose(dev):
 
 def test_transpose_largest(dev):
     P.check_transpose(dev, B=1, H=1, Mb=16384, T=16)
+    P.check_transpose(dev, B=1, H=2, Mb=16384, T=16, chunk=64)       # with the work list: the split form
 
 
 @pytest.mark.parametrize("strided,smooth", [(False, False), (True, False), (False, True)])
