@@ -54,6 +54,11 @@ const char* llsa_last_error_string(void);
  * (kernel/triton/rope.py:100-127) in one pass over the input.  One launch serves up to 4
  * tensors.  Rounding follows the reference: the accumulator has the tensor dtype, summed in
  * token order.
+ * With `gamma` the rows are first RMS-normalised over the 64 channels,
+ *     x <- bf16( float(x) * rsqrt(mean(float(x)^2) + eps) * gamma ),
+ * which is the qk-norm the reference's attention processor applies before the RoPE
+ * (models/rope_dit_transformer_2d.py:215-219: attn.norm_q / attn.norm_k, diffusers' RMSNorm
+ * with an fp32 weight, result cast back to the input dtype).
  * ---------------------------------------------------------------------------------------- */
 typedef struct llsa_pool_item {
     const void* x;          /* (B,H,n,64) bf16, strides below                                   */
@@ -66,7 +71,10 @@ typedef struct llsa_pool_item {
     void* xt;               /* (B,H,n/16,1024)  T tiles of (rotated) x, or NULL                 */
     void* y1r;              /* (B,H,n/256,1024) R tiles of y1, or NULL (n % 256 == 0)           */
     void* y1t;              /* (B,H,n/256,1024) T tiles of y1, or NULL (n % 256 == 0)           */
-    void* xrot;             /* (B,H,n,64) contiguous rotated x, or NULL                         */
+    void* xrot;             /* (B,H,n,64) contiguous copy of the normalised / rotated x, or NULL */
+    const float* gamma;     /* (64) fp32 or NULL: RMS-normalise every row first (see below)     */
+    float eps;
+    int32_t reserved;       /* 0                                                                */
 } llsa_pool_item;
 
 int llsa_pool_pyramid_fwd(const llsa_pool_item* items, int n_items, const void* freq /* (n,64) bf16 or NULL */,
@@ -87,6 +95,15 @@ int llsa_mean_pool_bwd(const void* dy, const int64_t* sdy, void* dx, const int64
 int llsa_pool_bwd_accum(const void* dx, const int64_t* sdx /*3*/, const void* dy1, const void* dy2 /* or NULL */,
                         void* out, const int64_t* sout /*3*/, const void* freq /* or NULL */,
                         int B, int H, int N, void* stream);
+
+/* Backward of the RMS normalisation above: dy, x (B,H,N,64) bf16 with strides, gamma (64) fp32;
+ * dx (B,H,N,64) bf16 = rstd * (g - xn * mean(g * xn)) with xn = x * rstd, g = dy * gamma, and
+ * dgamma (64) fp32 = sum over all rows of dy * xn.  `partials` is scratch of
+ * llsa_rmsnorm_bwd_partials(B,H,N) floats; the sum over rows is taken in a fixed order. */
+int64_t llsa_rmsnorm_bwd_partials(int B, int H, int N);
+int llsa_rmsnorm_bwd(const void* dy, const int64_t* sdy /*3*/, const void* x, const int64_t* sx /*3*/, const float* gamma,
+                     float eps, void* dx, const int64_t* sdx /*3*/, float* dgamma, float* partials,
+                     int B, int H, int N, void* stream);
 
 /* 2-D RoPE rotation, forward and backward (rope.py:6-97,100-145).  freq is (S,64) with
  * [sin, cos] interleaved; arithmetic is rounded to bf16 after every operation. */

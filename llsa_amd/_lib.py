@@ -20,7 +20,8 @@ class PoolItem(C.Structure):
     _fields_ = [("x", c_void_p), ("sxb", c_int64), ("sxh", c_int64), ("sxn", c_int64),
                 ("n", c_int32), ("rope", c_int32),
                 ("y1", c_void_p), ("y2", c_void_p), ("xr", c_void_p), ("xt", c_void_p), ("y1r", c_void_p),
-                ("y1t", c_void_p), ("xrot", c_void_p)]
+                ("y1t", c_void_p), ("xrot", c_void_p),
+                ("gamma", c_void_p), ("eps", c_float), ("reserved", c_int32)]
 
 
 class AttnFwdArgs(C.Structure):
@@ -63,6 +64,9 @@ _SIGNATURES = {
     "llsa_mean_pool_fwd": (c_int, [c_void_p, P64, c_void_p, P64, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llsa_mean_pool_bwd": (c_int, [c_void_p, P64, c_void_p, P64, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llsa_pool_bwd_accum": (c_int, [c_void_p, P64, c_void_p, c_void_p, c_void_p, P64, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "llsa_rmsnorm_bwd_partials": (c_int64, [c_int, c_int, c_int]),
+    "llsa_rmsnorm_bwd": (c_int, [c_void_p, P64, c_void_p, P64, c_void_p, c_float, c_void_p, P64, c_void_p, c_void_p,
+                                 c_int, c_int, c_int, c_void_p]),
     "llsa_rope_fwd": (c_int, [c_void_p, P64, c_void_p, c_void_p, P64, c_int, c_int, c_int, c_void_p]),
     "llsa_rope_bwd": (c_int, [c_void_p, P64, c_void_p, c_void_p, P64, c_int, c_int, c_int, c_void_p]),
     "llsa_topk_dense": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),

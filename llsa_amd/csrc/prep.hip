@@ -75,6 +75,27 @@ __device__ __forceinline__ void stage_out(bf16* stage, bf16* tiles32k, int t, in
     __syncthreads();                              // and may be refilled
 }
 
+// RMS normalisation of the thread's 16 rows (8 channels of each; the row's other channels are
+// in the 7 neighbouring lanes): x <- bf16(x * rsqrt(mean(x^2) + eps) * gamma), in fp32.
+__device__ __forceinline__ void rms_norm_rows(bf16x8 xv[16], const float* gamma, float eps, int c) {
+    float g[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) g[e] = gamma[c * 8 + e];
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) ss += (float)xv[i][e] * (float)xv[i][e];
+        ss += __shfl_xor(ss, 1);
+        ss += __shfl_xor(ss, 2);
+        ss += __shfl_xor(ss, 4);
+        const float rstd = rsqrtf(ss * (1.f / kD) + eps);
+#pragma unroll
+        for (int e = 0; e < 8; e++) xv[i][e] = (bf16)((float)xv[i][e] * rstd * g[e]);
+    }
+}
+
+template <bool NORM>
 __global__ __launch_bounds__(128) void pool_pyramid_kernel(PoolParams p) {
     __shared__ __align__(16) bf16 stage[16 * 128 * 8];
     const llsa_pool_item& it = p.it[blockIdx.z];
@@ -92,15 +113,16 @@ __global__ __launch_bounds__(128) void pool_pyramid_kernel(PoolParams p) {
         const bf16* x = (const bf16*)it.x + b * it.sxb + h * it.sxh + (int64_t)blk * kBlk * it.sxn + c * 8;
 #pragma unroll
         for (int i = 0; i < 16; i++) xv[i] = ld16(x + i * it.sxn);
+        if (NORM && it.gamma != nullptr) rms_norm_rows(xv, it.gamma, it.eps, c);
         if (it.rope) {
             const bf16* f = p.freq + ((int64_t)blk * kBlk) * kD + c * 8;
 #pragma unroll
             for (int i = 0; i < 16; i++) xv[i] = rope_chunk_fwd(xv[i], ld16(f + i * kD));
-            if (it.xrot != nullptr) {
-                bf16* xo = (bf16*)it.xrot + ((int64_t)bh * it.n + (int64_t)blk * kBlk) * kD + c * 8;
+        }
+        if (it.xrot != nullptr) {        // the rows as the attention sees them (normalised, rotated), row-major
+            bf16* xo = (bf16*)it.xrot + ((int64_t)bh * it.n + (int64_t)blk * kBlk) * kD + c * 8;
 #pragma unroll
-                for (int i = 0; i < 16; i++) st16(xo + i * kD, xv[i]);
-            }
+            for (int i = 0; i < 16; i++) st16(xo + i * kD, xv[i]);
         }
         if (it.y1 != nullptr || it.y2 != nullptr || it.y1r != nullptr || it.y1t != nullptr) {
             float acc[8];
@@ -246,6 +268,69 @@ __global__ __launch_bounds__(256) void rope_kernel(const bf16* x, Strides3 sx, c
     st16(y + b * sy.b + h * sy.h + (int64_t)tok * sy.n + c * 8, v);
 }
 
+// ---------------------------------------------------------------------------------------
+// Backward of the RMS normalisation.  Thread mapping of the stand-alone RoPE: one thread per
+// (token, 8-channel chunk), 32 tokens per workgroup; a workgroup also sums dy * xn over its 32
+// tokens (fixed order) into one row of `partials`, which rmsnorm_dgamma_kernel adds up.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const bf16* dy, Strides3 sdy, const bf16* x, Strides3 sx,
+                                                          const float* __restrict__ gamma, float eps, bf16* dx, Strides3 sdx,
+                                                          float* __restrict__ partials, int H, int N) {
+    __shared__ float red[32][kD];
+    const int row = threadIdx.x >> 3, c = threadIdx.x & 7;
+    const int tok = blockIdx.x * 32 + row;
+    const int bh = blockIdx.y, b = bh / H, h = bh % H;
+    float contrib[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) contrib[e] = 0.f;
+    if (tok < N) {
+        const bf16x8 xv = ld16(x + b * sx.b + h * sx.h + (int64_t)tok * sx.n + c * 8);
+        const bf16x8 gv = ld16(dy + b * sdy.b + h * sdy.h + (int64_t)tok * sdy.n + c * 8);
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) ss += (float)xv[e] * (float)xv[e];
+        ss += __shfl_xor(ss, 1);
+        ss += __shfl_xor(ss, 2);
+        ss += __shfl_xor(ss, 4);
+        const float rstd = rsqrtf(ss * (1.f / kD) + eps);
+        float xn[8], g[8], dot = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            xn[e] = (float)xv[e] * rstd;
+            g[e] = (float)gv[e] * gamma[c * 8 + e];
+            dot += g[e] * xn[e];
+            contrib[e] = (float)gv[e] * xn[e];
+        }
+        dot += __shfl_xor(dot, 1);
+        dot += __shfl_xor(dot, 2);
+        dot += __shfl_xor(dot, 4);
+        dot *= 1.f / kD;
+        bf16x8 o;
+#pragma unroll
+        for (int e = 0; e < 8; e++) o[e] = (bf16)(rstd * (g[e] - xn[e] * dot));
+        st16(dx + b * sdx.b + h * sdx.h + (int64_t)tok * sdx.n + c * 8, o);
+    }
+#pragma unroll
+    for (int e = 0; e < 8; e++) red[row][c * 8 + e] = contrib[e];
+    __syncthreads();
+    if (threadIdx.x < kD) {
+        float s = 0.f;
+        for (int r = 0; r < 32; r++) s += red[r][threadIdx.x];
+        partials[((int64_t)bh * gridDim.x + blockIdx.x) * kD + threadIdx.x] = s;
+    }
+}
+
+// one workgroup: thread (j, ch) adds rows j, j + 4, ... of `partials`, then the four j's are added
+__global__ __launch_bounds__(256) void rmsnorm_dgamma_kernel(const float* __restrict__ partials, float* __restrict__ dgamma, int64_t rows) {
+    __shared__ float red[4][kD];
+    const int ch = threadIdx.x & 63, j = threadIdx.x >> 6;
+    float s = 0.f;
+    for (int64_t r = j; r < rows; r += 4) s += partials[r * kD + ch];
+    red[j][ch] = s;
+    __syncthreads();
+    if (j == 0) dgamma[ch] = (red[0][ch] + red[1][ch]) + (red[2][ch] + red[3][ch]);
+}
+
 }  // namespace llsa
 
 using namespace llsa;
@@ -266,6 +351,7 @@ extern "C" int llsa_pool_pyramid_fwd(const llsa_pool_item* items, int n_items, c
         LLSA_REQUIRE((it.y2 == nullptr && it.y1t == nullptr && it.y1r == nullptr) || it.n % 256 == 0,
                      "pool_pyramid: item %d: level-2 outputs need n %% 256 == 0 (n=%d)", i, it.n);
         LLSA_REQUIRE(!it.rope || freq != nullptr, "pool_pyramid: item %d: rope needs freq", i);
+        LLSA_REQUIRE(it.gamma == nullptr || it.eps >= 0.f, "pool_pyramid: item %d: eps must be >= 0", i);
         LLSA_REQUIRE(aligned16(it.y1) && aligned16(it.y2) && aligned16(it.xr) && aligned16(it.xt) && aligned16(it.y1r) &&
                          aligned16(it.y1t) && aligned16(it.xrot),
                      "pool_pyramid: item %d: outputs must be 16-byte aligned", i);
@@ -273,8 +359,13 @@ extern "C" int llsa_pool_pyramid_fwd(const llsa_pool_item* items, int n_items, c
         if (it.n > max_n) max_n = it.n;
     }
     for (int i = n_items; i < 4; i++) p.it[i] = items[0];
+    bool norm = false;
+    for (int i = 0; i < n_items; i++) norm = norm || items[i].gamma != nullptr;
     dim3 grid((max_n + 255) / 256, B * H, n_items);
-    hipLaunchKernelGGL(pool_pyramid_kernel, grid, dim3(128), 0, (hipStream_t)stream, p);
+    if (norm)
+        hipLaunchKernelGGL(HIP_KERNEL_NAME(pool_pyramid_kernel<true>), grid, dim3(128), 0, (hipStream_t)stream, p);
+    else
+        hipLaunchKernelGGL(HIP_KERNEL_NAME(pool_pyramid_kernel<false>), grid, dim3(128), 0, (hipStream_t)stream, p);
     return launch_status("pool_pyramid");
 }
 
@@ -351,4 +442,24 @@ extern "C" int llsa_rope_fwd(const void* x, const int64_t* sx, const void* freq,
 extern "C" int llsa_rope_bwd(const void* dy, const int64_t* sdy, const void* freq, void* dx, const int64_t* sdx, int B,
                              int H, int S, void* stream) {
     return rope_launch(true, dy, sdy, freq, dx, sdx, B, H, S, stream);
+}
+
+extern "C" int64_t llsa_rmsnorm_bwd_partials(int B, int H, int N) {
+    if (B <= 0 || H <= 0 || N <= 0) return -1;
+    return (int64_t)B * H * ((N + 31) / 32) * kD;
+}
+
+extern "C" int llsa_rmsnorm_bwd(const void* dy, const int64_t* sdy, const void* x, const int64_t* sx, const float* gamma, float eps,
+                                void* dx, const int64_t* sdx, float* dgamma, float* partials, int B, int H, int N, void* stream) {
+    LLSA_REQUIRE(dy && x && gamma && dx && dgamma && partials && sdy && sx && sdx, "rmsnorm_bwd: null argument");
+    LLSA_REQUIRE(B > 0 && H > 0 && N > 0 && eps >= 0.f, "rmsnorm_bwd: bad shape or eps");
+    LLSA_REQUIRE(aligned16(dy) && aligned16(x) && aligned16(dx) && s3_ok(sdy) && s3_ok(sx) && s3_ok(sdx),
+                 "rmsnorm_bwd: rows must be 16-byte aligned");
+    Strides3 a{sdy[0], sdy[1], sdy[2]}, bx{sx[0], sx[1], sx[2]}, o{sdx[0], sdx[1], sdx[2]};
+    const int parts = (N + 31) / 32;
+    hipLaunchKernelGGL(rmsnorm_bwd_kernel, dim3(parts, B * H), dim3(256), 0, (hipStream_t)stream, (const bf16*)dy, a, (const bf16*)x, bx,
+                       gamma, eps, (bf16*)dx, o, partials, H, N);
+    hipLaunchKernelGGL(rmsnorm_dgamma_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (const float*)partials, dgamma,
+                       (int64_t)B * H * parts);
+    return launch_status("rmsnorm_bwd");
 }

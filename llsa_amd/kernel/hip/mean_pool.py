@@ -83,11 +83,13 @@ def mean_pool1d(x: torch.Tensor, k: int, format='bhsc'):
 class PoolSpec:
     """What to produce from one (B,H,n,64) bf16 tensor in a pool_pyramid launch: y1 / y2 pooled
     rows, xr / xt operand tiles of the (rotated) tensor, y1r / y1t operand tiles of y1, xrot a
-    row-major rotated copy."""
+    row-major copy of the rows as transformed (normalised with `gamma` (64) fp32 and `eps` first, then
+    rotated)."""
 
-    def __init__(self, x, y1=False, y2=False, xr=False, xt=False, y1r=False, y1t=False, rope=False, xrot=False):
+    def __init__(self, x, y1=False, y2=False, xr=False, xt=False, y1r=False, y1t=False, rope=False, xrot=False,
+                 gamma=None, eps=0.0):
         self.x, self.y1, self.y2, self.xr, self.xt, self.y1r, self.y1t = x, y1, y2, xr, xt, y1r, y1t
-        self.rope, self.xrot = rope, xrot
+        self.rope, self.xrot, self.gamma, self.eps = rope, xrot, gamma, eps
 
 
 def pool_pyramid(specs: Sequence[PoolSpec], freq: Optional[torch.Tensor] = None):
@@ -130,8 +132,15 @@ def pool_pyramid(specs: Sequence[PoolSpec], freq: Optional[torch.Tensor] = None)
         if s.xrot:
             o["xrot"] = e(B, H, n, 64)
         outs.append(o)
+        gamma = None
+        if s.gamma is not None:
+            gamma = s.gamma.to(device=x.device, dtype=torch.float32).contiguous()
+            if gamma.numel() != HEAD_DIM:
+                raise ValueError("gamma must have 64 entries")
+            keep.append(gamma)
         items.append(PoolItem(x.data_ptr(), x.stride(0), x.stride(1), x.stride(2), n, 1 if s.rope else 0,
-                              *(o[k].data_ptr() if k in o else None for k in ("y1", "y2", "xr", "xt", "y1r", "y1t", "xrot"))))
+                              *(o[k].data_ptr() if k in o else None for k in ("y1", "y2", "xr", "xt", "y1r", "y1t", "xrot")),
+                              None if gamma is None else gamma.data_ptr(), float(s.eps), 0))
     if freq is not None:
         require_bf16(freq)
         freq = freq.contiguous()

@@ -114,10 +114,13 @@ def _check(lib, rc, what):
 
 
 class LlsaFused(Function):
-    """forward(q, k, v, levels, topk1, topk2, block_size, freq) -> o"""
+    """forward(q, k, v, levels, topk1, topk2, block_size, freq, gamma_q, gamma_k, eps) -> o
+
+    gamma_q / gamma_k ((64,) fp32 or None): RMS-normalise q / k over the head dimension first (the
+    qk-norm of the reference's attention processor), inside the pooling pass; they receive gradients."""
 
     @staticmethod
-    def forward(ctx, q, k, v, levels, topk1, topk2, block_size, freq):
+    def forward(ctx, q, k, v, levels, topk1, topk2, block_size, freq, gamma_q=None, gamma_k=None, eps=1e-5):
         lib = current_lib()
         if block_size != 16:
             raise NotImplementedError("block_size must be 16")
@@ -142,8 +145,15 @@ class LlsaFused(Function):
             if freq.dtype != torch.bfloat16 or tuple(freq.shape) != (N, 64):
                 raise ValueError("rope table must be bf16 (N, 64)")
             freq = freq.contiguous()
-        grad = any(ctx.needs_input_grad[:3])
+        grad = any(ctx.needs_input_grad[:3]) or ctx.needs_input_grad[8] or ctx.needs_input_grad[9]
         q, k, v = (t if _rows_ok(t) else t.contiguous() for t in (q, k, v))
+        gq = gk = None
+        if gamma_q is not None:
+            gq = gamma_q.detach().to(device=q.device, dtype=torch.float32).contiguous()
+        if gamma_k is not None:
+            gk = gamma_k.detach().to(device=q.device, dtype=torch.float32).contiguous()
+        if any(g is not None and g.numel() != 64 for g in (gq, gk)):
+            raise ValueError("qk-norm weights must have 64 entries")
         lay = _layout(lib, B, H, N, levels, T, T2, grad)
         dev = q.device
         A = torch.empty(lay.n_bf16, device=dev, dtype=torch.bfloat16)
@@ -158,9 +168,9 @@ class LlsaFused(Function):
 
         items = (PoolItem * 3)(
             PoolItem(q.data_ptr(), q.stride(0), q.stride(1), q.stride(2), N, int(rope), pa(lay.pq), pa(lay.pq2), pa(lay.qr),
-                     None, None, None, None),
+                     None, None, None, None, None if gq is None else gq.data_ptr(), float(eps), 0),
             PoolItem(k.data_ptr(), k.stride(0), k.stride(1), k.stride(2), N, int(rope), pa(lay.pk), pa(lay.pk2), pa(lay.kr),
-                     None, pa(lay.pkr), None, None),
+                     None, pa(lay.pkr), None, None, None if gk is None else gk.data_ptr(), float(eps), 0),
             PoolItem(v.data_ptr(), v.stride(0), v.stride(1), v.stride(2), N, 0, pa(lay.pv), pa(lay.pv2), pa(lay.vr),
                      pa(lay.vt), pa(lay.pvr), pa(lay.pvt), None))
         _check(lib, lib.pool_pyramid_fwd(items, 3, freq.data_ptr() if rope else None, B, H, stream), "pool_pyramid")
@@ -213,13 +223,16 @@ class LlsaFused(Function):
                 cur.wait_event(ev_lists)
 
         if grad:
-            ctx.save_for_backward(A, I, o, lse, freq)
+            # (q and k themselves are needed again only by the backward of the qk-norm)
+            ctx.save_for_backward(A, I, o, lse, freq, gq, gk, q if gq is not None else None, k if gk is not None else None)
             ctx.meta = (lib, lay, B, H, N, T, T2, levels, q.shape, q.stride(), k.stride(), v.stride())
+            ctx.eps = float(eps)
+            ctx.gamma_dtypes = (None if gamma_q is None else gamma_q.dtype, None if gamma_k is None else gamma_k.dtype)
         return o
 
     @staticmethod
     def backward(ctx, do):
-        A, I, o, lse, freq = ctx.saved_tensors
+        A, I, o, lse, freq, gq, gk, q_in, k_in = ctx.saved_tensors
         lib, lay, B, H, N, T, T2, levels, shape, sq, sk, sv = ctx.meta
         dev = o.device
         if not _rows_ok(do):
@@ -258,8 +271,24 @@ class LlsaFused(Function):
         # (sparse_attention_res_1.py:388-389) although the forward uses token_weight
         a.w1, a.w2, a.cgw1 = 16.0, 256.0, (16.0 if levels == 2 else 1.0)
         a.stages, a.fold_pooled = 0, 1
-        _check(lib, lib.attn_bwd(C.byref(a), _stream(lib, o)), "attn_bwd")
-        return dq, dk, dv, None, None, None, None, None
+        stream = _stream(lib, o)
+        _check(lib, lib.attn_bwd(C.byref(a), stream), "attn_bwd")
+        dgq = dgk = None
+        if gq is not None or gk is not None:      # back through the qk-norm, in place on dq / dk
+            P = torch.empty(lib.rmsnorm_bwd_partials(B, H, N), device=dev, dtype=torch.float32)
+            i3 = lambda t: (C.c_int64 * 3)(t.stride(0), t.stride(1), t.stride(2))
+            for g, x, d, which in ((gq, q_in, dq, 0), (gk, k_in, dk, 1)):
+                if g is None:
+                    continue
+                dg = torch.empty(64, device=dev, dtype=torch.float32)
+                _check(lib, lib.rmsnorm_bwd(d.data_ptr(), i3(d), x.data_ptr(), i3(x), g.data_ptr(), ctx.eps, d.data_ptr(), i3(d),
+                                            dg.data_ptr(), P.data_ptr(), B, H, N, stream), "rmsnorm_bwd")
+                dg = dg.to(ctx.gamma_dtypes[which])
+                if which == 0:
+                    dgq = dg
+                else:
+                    dgk = dg
+        return dq, dk, dv, None, None, None, None, None, dgq, dgk, None
 
 
 def selection(out):

@@ -6,6 +6,12 @@ reference: `FlashSparseResidualAttentionL1`, `flash_sparse_residual_attention_l1
 q and k are rotated inside the pooling pass and the gradients are rotated back inside the
 backward kernels, which is the same function as
 `llsa_l1(my_rope_fn(q, freq), my_rope_fn(k, freq), v, ...)`.
+
+`qk_norm=(gamma_q, gamma_k, eps)` (two fp32 vectors of 64 weights and the epsilon) moves the
+attention processor's RMS norms of q and k (rope_dit_transformer_2d.py:215-218) into the same
+pass: rows are normalised before the rotation, the gradients come back through the norm, and
+gamma_q / gamma_k receive theirs.  Same function as
+`llsa_l1(my_rms_norm_fn(q, gamma_q, eps), my_rms_norm_fn(k, gamma_k, eps), v, ...)`.
 """
 from __future__ import annotations
 
@@ -42,9 +48,10 @@ class FlashSparseResidualAttentionL1(Function):
 flash_sparse_residual_attention_l1_op = FlashSparseResidualAttentionL1.apply
 
 
-def llsa_l1(q, k, v, topk=8, block_size=16, rope=None):
+def llsa_l1(q, k, v, topk=8, block_size=16, rope=None, qk_norm=None):
     """flash_sparse_attention_res_1.py:41-47."""
-    return LlsaFused.apply(q, k, v, 1, topk, 0, block_size, rope)
+    gq, gk, eps = qk_norm if qk_norm is not None else (None, None, 0.0)
+    return LlsaFused.apply(q, k, v, 1, topk, 0, block_size, rope, gq, gk, eps)
 
 
 def llsa_l1_unfused(q, k, v, topk=8, block_size=16):

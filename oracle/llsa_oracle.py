@@ -35,6 +35,10 @@ Pinning status (what each function is checked against, see tests/test_oracle_*):
                          (sparse_attention_res_1.py:173); which reduction tree
                          Triton uses is not observable here: parity unpinned for
                          `delta_in_dtype=True`; the default keeps fp32.
+  rms_norm / _bwd        F.rms_norm and its autograd (fp32).  The module the model
+                         calls (diffusers' RMSNorm, rope_dit_transformer_2d.py:215-218)
+                         is not in the reference checkout: parity unpinned for its
+                         eps and rounding points.
 """
 from __future__ import annotations
 
@@ -146,6 +150,32 @@ def rope_apply_bwd(dy: torch.Tensor, freq: torch.Tensor) -> torch.Tensor:
     xe = _rn(_rn(cos * de, dt) + _rn(sin * do, dt), dt)
     xo = _rn(_rn(-sin * de, dt) + _rn(cos * do, dt), dt)
     return torch.stack([xe, xo], dim=-1).reshape(dy.shape).to(dt)
+
+
+# --------------------------------------------------------------------------------------
+# qk RMS norm  --  call site models/rope_dit_transformer_2d.py:215-219 (diffusers' RMSNorm)
+# --------------------------------------------------------------------------------------
+
+
+def rms_norm(x: torch.Tensor, gamma: torch.Tensor, eps: float) -> torch.Tensor:
+    """The qk-norm of the attention processor (rope_dit_transformer_2d.py:215-219: attn.norm_q /
+    attn.norm_k, applied to (B,H,N,D) before the RoPE, result cast back to the input dtype).
+    diffusers' RMSNorm is not in the reference checkout; this is the textbook definition it
+    implements, computed in fp32 with an fp32 weight: y = x * rsqrt(mean(x^2, -1) + eps) * gamma.
+    PARITY UNPINNED against diffusers itself (eps, and where exactly it rounds)."""
+    xf = _up(x)
+    y = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * _up(gamma)
+    return y.to(x.dtype)
+
+
+def rms_norm_bwd(dy: torch.Tensor, x: torch.Tensor, gamma: torch.Tensor, eps: float):
+    """Backward of rms_norm in fp32: returns (dx in x.dtype, dgamma fp32/fp64 like gamma)."""
+    xf, g = _up(x), _up(dy) * _up(gamma)
+    rstd = torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    xn = xf * rstd
+    dx = rstd * (g - xn * (g * xn).mean(-1, keepdim=True))
+    dgamma = (_up(dy) * xn).reshape(-1, x.shape[-1]).sum(0)
+    return dx.to(x.dtype), dgamma
 
 
 # --------------------------------------------------------------------------------------

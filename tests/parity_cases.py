@@ -324,7 +324,42 @@ def _grads(fn, q, k, v, do):
     return o.detach(), q.grad, k.grad, v.grad
 
 
-def check_op_l1(dev, B=1, H=2, N=1024, T=8, fused=True, rope=False, strided=False, smooth=False):
+def _norm_weights(dev):
+    """(gamma_q, gamma_k, eps) of a qk RMS norm, as the fused operators take them."""
+    g = torch.Generator().manual_seed(31)
+    return ((torch.rand(64, generator=g) + 0.5).to(dev), (torch.rand(64, generator=g) + 0.5).to(dev), 1e-5)
+
+
+def _apply_norm(qc, kc, norm):
+    if norm is None:
+        return qc, kc
+    return O.rms_norm(qc, norm[0].cpu(), norm[2]), O.rms_norm(kc, norm[1].cpu(), norm[2])
+
+
+def _norm_backward(rq, rk, qc, kc, norm):
+    if norm is None:
+        return rq, rk
+    return (O.rms_norm_bwd(rq.to(qc.dtype), qc, norm[0].cpu(), norm[2])[0], O.rms_norm_bwd(rk.to(kc.dtype), kc, norm[1].cpu(), norm[2])[0])
+
+
+def check_rms_norm(dev, B=2, H=3, N=512, strided=True):
+    """Stand-alone forms against the oracle: forward bit for bit up to one bf16 ulp of rounding-order
+    freedom (the row's sum of squares is added in another order), backward within the operator's
+    tolerance, dgamma in fp32."""
+    from llsa_amd.kernel.hip.rms_norm import rms_norm_bwd, rms_norm_fwd
+    x, _, _, dy = randn_inputs(B, H, N, 64, dev, seed=23, strided=strided)
+    gq, _, eps = _norm_weights(dev)
+    y = rms_norm_fwd(x, gq, eps)
+    ry = O.rms_norm(x.cpu(), gq.cpu(), eps)
+    assert (y.cpu().float() - ry.float()).abs().max() <= 2.0 ** -7 * ry.float().abs().max()
+    assert (y.cpu() != ry).float().mean() < 0.02, "more than 2 % of the normalised values differ from the oracle's"
+    dx, dg = rms_norm_bwd(dy, x, gq, eps)
+    rdx, rdg = O.rms_norm_bwd(dy.cpu(), x.cpu(), gq.cpu(), eps)
+    close("dx", dx, rdx)
+    assert torch.allclose(dg.cpu(), rdg, rtol=2e-3, atol=2e-2), f"dgamma differs by {(dg.cpu() - rdg).abs().max():.3e}"
+
+
+def check_op_l1(dev, B=1, H=2, N=1024, T=8, fused=True, rope=False, strided=False, smooth=False, qk_norm=False):
     """The whole operator through autograd, against the oracle's composition fed with the
     indices the device selected (selection itself is checked separately)."""
     from llsa_amd.kernel.hip.rope import my_rope_fn
@@ -334,10 +369,11 @@ def check_op_l1(dev, B=1, H=2, N=1024, T=8, fused=True, rope=False, strided=Fals
     q, k, v, do = smooth_inputs(B, H, N, 64, dev) if smooth else randn_inputs(B, H, N, 64, dev, seed=19, strided=strided)
     freq = rope_table(int(math.isqrt(N)), dtype=torch.bfloat16).to(dev) if rope else None
     captured = {}
+    norm = _norm_weights(dev) if qk_norm else None
 
     def run(q_, k_, v_):
         if fused:
-            out = M.llsa_l1(q_, k_, v_, T, 16, rope=freq)
+            out = M.llsa_l1(q_, k_, v_, T, 16, rope=freq, qk_norm=norm)
             captured["idx"] = selection(out)[0]
             return out
         if rope:
@@ -349,12 +385,14 @@ def check_op_l1(dev, B=1, H=2, N=1024, T=8, fused=True, rope=False, strided=Fals
     o, dq, dk, dv = _grads(run, q, k, v, do)
     qc, kc, vc, doc = (t.cpu() for t in (q, k, v, do))
     fc = freq.cpu() if rope else None
-    qr, kr = (O.rope_apply(qc, fc), O.rope_apply(kc, fc)) if rope else (qc, kc)
+    qn, kn = _apply_norm(qc, kc, norm)
+    qr, kr = (O.rope_apply(qn, fc), O.rope_apply(kn, fc)) if rope else (qn, kn)
     idx = captured["idx"].cpu().long()
     ro, ctx = O.llsa_l1_fwd(qr, kr, vc, T, 16, indices=idx)
     rq, rk, rv, _ = O.llsa_l1_bwd(doc, ctx)
     if rope:
         rq, rk = O.rope_apply_bwd(rq, fc), O.rope_apply_bwd(rk, fc)
+    rq, rk = _norm_backward(rq, rk, qc, kc, norm)
     close("o", o, ro)
     close("dq", dq, rq)
     close("dk", dk, rk)
@@ -366,7 +404,7 @@ def check_op_l1(dev, B=1, H=2, N=1024, T=8, fused=True, rope=False, strided=Fals
     assert (picked >= kth - 2.0 ** -6 * kth.abs().clamp_min(1.0)).all(), "selected a block below the top-k threshold"
 
 
-def check_op_l2(dev, B=1, H=1, N=16384, T=8, T2=4, fused=True, rope=False, smooth=False):
+def check_op_l2(dev, B=1, H=1, N=16384, T=8, T2=4, fused=True, rope=False, smooth=False, qk_norm=False):
     from llsa_amd.kernel.hip.rope import my_rope_fn
     from llsa_amd.kernel.torch_op import flash_sparse_attention_res_2 as M
     from llsa_amd.kernel.torch_op._fused import selection
@@ -374,10 +412,11 @@ def check_op_l2(dev, B=1, H=1, N=16384, T=8, T2=4, fused=True, rope=False, smoot
     q, k, v, do = smooth_inputs(B, H, N, 64, dev) if smooth else randn_inputs(B, H, N, 64, dev, seed=20)
     freq = rope_table(int(math.isqrt(N)), dtype=torch.bfloat16).to(dev) if rope else None
     captured = {}
+    norm = _norm_weights(dev) if qk_norm else None
 
     def run(q_, k_, v_):
         if fused:
-            out = M.llsa_l2(q_, k_, v_, T, T2, 16, rope=freq)
+            out = M.llsa_l2(q_, k_, v_, T, T2, 16, rope=freq, qk_norm=norm)
             captured["idx"], captured["pidx"] = selection(out)
             return out
         if rope:
@@ -389,11 +428,13 @@ def check_op_l2(dev, B=1, H=1, N=16384, T=8, T2=4, fused=True, rope=False, smoot
     o, dq, dk, dv = _grads(run, q, k, v, do)
     qc, kc, vc, doc = (t.cpu() for t in (q, k, v, do))
     fc = freq.cpu() if rope else None
-    qr, kr = (O.rope_apply(qc, fc), O.rope_apply(kc, fc)) if rope else (qc, kc)
+    qn, kn = _apply_norm(qc, kc, norm)
+    qr, kr = (O.rope_apply(qn, fc), O.rope_apply(kn, fc)) if rope else (qn, kn)
     ro, ctx = O.llsa_l2_fwd(qr, kr, vc, T, T2, 16, indices=captured["idx"].cpu(), p_indices=captured["pidx"].cpu().long())
     rq, rk, rv, _ = O.llsa_l2_bwd(doc, ctx)
     if rope:
         rq, rk = O.rope_apply_bwd(rq, fc), O.rope_apply_bwd(rk, fc)
+    rq, rk = _norm_backward(rq, rk, qc, kc, norm)
     close("o", o, ro)
     close("dq", dq, rq)
     close("dk", dk, rk)

@@ -47,6 +47,14 @@ def test_topk_sparse():
     P.check_topk_sparse(DEV, N1=256, T=8, T2=4)
 
 
+def test_rms_norm():
+    P.check_rms_norm(DEV, B=1, H=2, N=64, strided=True)
+
+
+def test_op_l1_qk_norm():
+    P.check_op_l1(DEV, B=1, H=1, N=1024, T=8, fused=True, rope=True, qk_norm=True)
+
+
 def test_transpose():
     P.check_transpose(DEV, Mb=64, T=8)
     P.check_transpose(DEV, B=1, H=1, Mb=64, T=4, Kb=16)

@@ -47,6 +47,16 @@ def test_rope(dev):
     P.check_rope(dev, B=1, H=2, side=8, strided=False)
 
 
+def test_rms_norm(dev):
+    P.check_rms_norm(dev, B=2, H=3, N=4096, strided=True)
+    P.check_rms_norm(dev, B=1, H=1, N=16, strided=False)
+
+
+def test_op_with_qk_norm(dev):
+    P.check_op_l1(dev, B=2, H=2, N=4096, T=16, fused=True, rope=True, strided=True, qk_norm=True)
+    P.check_op_l2(dev, B=1, H=2, N=16384, T=16, T2=16, fused=True, rope=True, smooth=True, qk_norm=True)
+
+
 def test_topk_dense(dev):
     P.check_topk_dense(dev, B=2, H=3, n=256, T=16, round_scores=True)
     P.check_topk_dense(dev, B=1, H=2, n=64, T=16, round_scores=False, min_safe=0.9)

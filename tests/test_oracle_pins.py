@@ -393,3 +393,24 @@ def test_whole_op_l2_backward_composition():
     # selection is hierarchical: every fine index lies inside a coarse block its parent selected
     par = ctx["p_indices"].repeat_interleave(16, dim=2)
     assert ((ctx["indices"].long()[..., None] // 16) == par[:, :, :, None, :]).any(-1).all()
+
+
+def test_rms_norm_against_torch():
+    """rms_norm / rms_norm_bwd against the library routine and its autograd (fp64, then the bf16 path
+    against an fp32 evaluation rounded once)."""
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(2, 3, 32, 64, generator=g, dtype=torch.float64)
+    gamma = torch.rand(64, generator=g, dtype=torch.float64) + 0.5
+    dy = torch.randn(2, 3, 32, 64, generator=g, dtype=torch.float64)
+    xr = x.clone().requires_grad_(True)
+    gr = gamma.clone().requires_grad_(True)
+    y = F.rms_norm(xr, (64,), gr, 1e-5)
+    y.backward(dy)
+    assert torch.allclose(O.rms_norm(x, gamma, 1e-5), y.detach(), rtol=1e-12, atol=1e-12)
+    dx, dgamma = O.rms_norm_bwd(dy, x, gamma, 1e-5)
+    assert torch.allclose(dx, xr.grad, rtol=1e-10, atol=1e-12)
+    assert torch.allclose(dgamma, gr.grad, rtol=1e-10, atol=1e-12)
+    xb = x.bfloat16()
+    want = F.rms_norm(xb.float(), (64,), gamma.float(), 1e-5).bfloat16()
+    got = O.rms_norm(xb, gamma.float(), 1e-5)
+    assert got.dtype == torch.bfloat16 and (got.float() - want.float()).abs().max() <= 2.0 ** -7 * want.float().abs().max()
