@@ -105,6 +105,15 @@ int llsa_rmsnorm_bwd(const void* dy, const int64_t* sdy /*3*/, const void* x, co
                      float eps, void* dx, const int64_t* sdx /*3*/, float* dgamma, float* partials,
                      int B, int H, int N, void* stream);
 
+/* Token permutation at the model's entry and exit (models/rope_dit_transformer_2d.py:963-965,
+ * 1028-1030: hidden_states[:, fwd_perm, :] and hidden_states[:, bwd_perm, :]), and the one after
+ * the REPA pooling (:1020).  y[b, i, :] = x[b, index[i], :] for b < B, i < n_out; rows are
+ * row_bytes long (a multiple of 16) and contiguous inside a batch, batches are x_batch_bytes /
+ * y_batch_bytes apart.  index is int32 on the device; an entry outside [0, n_in) gives zeros.
+ * The backward of a permutation is the same call with the inverse permutation. */
+int llsa_gather_rows(const void* x, void* y, const int32_t* index, int B, int n_out, int n_in, int row_bytes,
+                     int64_t x_batch_bytes, int64_t y_batch_bytes, void* stream);
+
 /* 2-D RoPE rotation, forward and backward (rope.py:6-97,100-145).  freq is (S,64) with
  * [sin, cos] interleaved; arithmetic is rounded to bf16 after every operation. */
 int llsa_rope_fwd(const void* x, const int64_t* sx /*3*/, const void* freq, void* y, const int64_t* sy /*3*/,

@@ -67,6 +67,7 @@ _SIGNATURES = {
     "llsa_rmsnorm_bwd_partials": (c_int64, [c_int, c_int, c_int]),
     "llsa_rmsnorm_bwd": (c_int, [c_void_p, P64, c_void_p, P64, c_void_p, c_float, c_void_p, P64, c_void_p, c_void_p,
                                  c_int, c_int, c_int, c_void_p]),
+    "llsa_gather_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int64, c_int64, c_void_p]),
     "llsa_rope_fwd": (c_int, [c_void_p, P64, c_void_p, c_void_p, P64, c_int, c_int, c_int, c_void_p]),
     "llsa_rope_bwd": (c_int, [c_void_p, P64, c_void_p, c_void_p, P64, c_int, c_int, c_int, c_void_p]),
     "llsa_topk_dense": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),

@@ -444,6 +444,40 @@ extern "C" int llsa_rope_bwd(const void* dy, const int64_t* sdy, const void* fre
     return rope_launch(true, dy, sdy, freq, dx, sdx, B, H, S, stream);
 }
 
+// ---------------------------------------------------------------------------------------
+// Token permutation: y[b, i, :] = x[b, index[i], :] for rows of `chunks` 16-byte pieces.  A
+// workgroup takes 256 consecutive pieces of the output, so stores are contiguous and every
+// source row is read in pieces of at least min(row, 4 KB).  An index outside [0, n_in) gives a
+// row of zeros.
+// ---------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void gather_rows_kernel(const i32x4* __restrict__ x, i32x4* __restrict__ y,
+                                                          const int32_t* __restrict__ index, int n_out, int n_in, int chunks,
+                                                          int64_t x_batch, int64_t y_batch) {
+    const int64_t piece = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (piece >= (int64_t)n_out * chunks) return;
+    const int row = (int)(piece / chunks), c = (int)(piece - (int64_t)row * chunks);
+    const int src = index[row];
+    i32x4 v = {0, 0, 0, 0};
+    if ((unsigned)src < (unsigned)n_in) v = x[blockIdx.y * x_batch + (int64_t)src * chunks + c];
+    y[blockIdx.y * y_batch + piece] = v;
+}
+
+extern "C" int llsa_gather_rows(const void* x, void* y, const int32_t* index, int B, int n_out, int n_in, int row_bytes,
+                                int64_t x_batch_bytes, int64_t y_batch_bytes, void* stream) {
+    LLSA_REQUIRE(x && y && index, "gather_rows: null argument");
+    LLSA_REQUIRE(B > 0 && n_out > 0 && n_in > 0 && row_bytes > 0 && row_bytes % 16 == 0, "gather_rows: rows must be a multiple of 16 bytes");
+    LLSA_REQUIRE(aligned16(x) && aligned16(y) && x_batch_bytes % 16 == 0 && y_batch_bytes % 16 == 0 &&
+                     x_batch_bytes >= (int64_t)n_in * row_bytes && y_batch_bytes >= (int64_t)n_out * row_bytes,
+                 "gather_rows: batches must be 16-byte aligned and hold their rows");
+    LLSA_REQUIRE(B <= 65535, "gather_rows: at most 65535 batches");
+    const int chunks = row_bytes / 16;
+    const int64_t pieces = (int64_t)n_out * chunks;
+    LLSA_REQUIRE(pieces < ((int64_t)1 << 31) * 256, "gather_rows: too many rows");
+    hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)((pieces + 255) / 256), B), dim3(256), 0, (hipStream_t)stream,
+                       (const i32x4*)x, (i32x4*)y, index, n_out, n_in, chunks, x_batch_bytes / 16, y_batch_bytes / 16);
+    return launch_status("gather_rows");
+}
+
 extern "C" int64_t llsa_rmsnorm_bwd_partials(int B, int H, int N) {
     if (B <= 0 || H <= 0 || N <= 0) return -1;
     return (int64_t)B * H * ((N + 31) / 32) * kD;

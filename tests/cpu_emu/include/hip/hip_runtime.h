@@ -133,5 +133,6 @@ inline unsigned __float_as_uint(float f) { unsigned u; memcpy(&u, &f, 4); return
 inline float __uint_as_float(unsigned u) { float f; memcpy(&f, &u, 4); return f; }
 inline float __expf(float x) { return expf(x); }
 inline float __logf(float x) { return logf(x); }
+inline float rsqrtf(float x) { return 1.0f / sqrtf(x); }
 template <typename T> inline T min(T a, T b) { return a < b ? a : b; }
 template <typename T> inline T max(T a, T b) { return a > b ? a : b; }

@@ -324,6 +324,31 @@ def _grads(fn, q, k, v, do):
     return o.detach(), q.grad, k.grad, v.grad
 
 
+def check_permute(dev, B=2, side=32, C=96, dtype=torch.bfloat16):
+    """gather_tokens / permute_tokens against plain indexing: bit for bit, gradients included."""
+    from llsa_amd.kernel.hip.permute import gather_tokens, permute_tokens
+    perm, inv = O.zorder_perm(side)
+    N = side * side
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(B, N, C, generator=g).to(dtype)
+    xd = x.clone().to(dev).requires_grad_(True)
+    y = permute_tokens(xd, inv.to(dev), perm.to(dev))
+    assert torch.equal(y.detach().cpu(), x[:, inv])
+    dy = torch.randn(B, N, C, generator=g).to(dtype)
+    y.backward(dy.to(dev))
+    ref = x.clone().requires_grad_(True)
+    ref[:, inv].backward(dy)
+    assert torch.equal(xd.grad.cpu(), ref.grad)
+    assert torch.equal(gather_tokens(y.detach(), perm.to(dev)).cpu(), x), "entry then exit is not the identity"
+    # a shorter index list (a pooled grid), a view with padded batches, and an index out of range
+    idx = torch.tensor([3, N - 1, 0, N, -1, 7], dtype=torch.int64)
+    wide = torch.randn(B, N + 5, C, generator=g).to(dtype).to(dev)
+    got = gather_tokens(wide[:, :N], idx.to(dev)).cpu()
+    want = wide.cpu()[:, idx.clamp(0, N - 1)]
+    want[:, 3:5] = 0
+    assert torch.equal(got, want)
+
+
 def _norm_weights(dev):
     """(gamma_q, gamma_k, eps) of a qk RMS norm, as the fused operators take them."""
     g = torch.Generator().manual_seed(31)

@@ -47,6 +47,11 @@ def test_topk_sparse():
     P.check_topk_sparse(DEV, N1=256, T=8, T2=4)
 
 
+def test_permute():
+    P.check_permute(DEV, B=2, side=8, C=24, dtype=torch.bfloat16)
+    P.check_permute(DEV, B=1, side=4, C=4, dtype=torch.float32)
+
+
 def test_rms_norm():
     P.check_rms_norm(DEV, B=1, H=2, N=64, strided=True)
 

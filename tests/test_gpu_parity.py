@@ -47,6 +47,11 @@ def test_rope(dev):
     P.check_rope(dev, B=1, H=2, side=8, strided=False)
 
 
+def test_permute(dev):
+    P.check_permute(dev, B=2, side=128, C=384, dtype=torch.bfloat16)
+    P.check_permute(dev, B=3, side=16, C=12, dtype=torch.float32)
+
+
 def test_rms_norm(dev):
     P.check_rms_norm(dev, B=2, H=3, N=4096, strided=True)
     P.check_rms_norm(dev, B=1, H=1, N=16, strided=False)
