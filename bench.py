@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the llsa hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c5|n65536] [--no-extras]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c5|n65536|c4] [--no-extras]
 
 A step is one forward + backward of the operator on one batch of synthetic input that is
 already resident in HBM.  The default workload is the configuration the headline metric is
@@ -16,6 +16,10 @@ One JSON line is printed:
   cpu_baseline the CPU oracle (plain PyTorch restatement) on the host cores, same workload in fp32
   kernels      per-stage times of that second pass (ms), with the achieved rate of each
   dense_sdpa   F.scaled_dot_product_attention forward+backward on the same shapes, same GPU
+
+--workload c4 times something else, one training step of the operator's caller (a pixel DiT-S with
+llsa_l2 in its 12 attention layers, batch 8 of 3x128x128, bf16 autocast, AdamW), and prints a line
+of its own kind: ms per step, images/s and the share of the step spent in the operator.
 """
 from __future__ import annotations
 
@@ -178,12 +182,81 @@ def cpu_baseline(op, B, H, N, D, t1, t2, rope):
             "ms": t_best * 1e3}
 
 
+def bench_dit(args):
+    """One flow-matching training step of llsa_amd.caller.PixelDiT (DiT-S: 12 layers, hidden 384, 6 heads
+    of 64, qk RMS norm, 2-D RoPE, llsa_l2 topk 16/16) on 8 synthetic 3x128x128 images."""
+    import torch
+    import llsa_amd
+    from llsa_amd._lib import get_lib
+    from llsa_amd.caller import FlowMatchingStep, PixelDiT
+    from llsa_amd.utils.synth import smooth_field
+    get_lib()
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    dev = torch.device("cuda:0")
+    B, side, layers, H, D, t1, t2 = 8, 128, 12, 6, 64, 16, 16
+    N = side * side
+    torch.manual_seed(0)
+    model = PixelDiT(num_layers=layers, num_attention_heads=H, attention_head_dim=D, sample_size=side, sparse_topk=(t2, t1),
+                     fused_prologue=not args.unfused).to(dev)
+    step = FlowMatchingStep(model)
+    # images: smooth fields in raster order scaled into [-1, 1]; timesteps uniform in [0, 1000); noise N(0,1)
+    f = smooth_field(7, B, 1, N, 3, dtype=torch.float32, mix=(1.0, 0.0), zorder=False).reshape(B, side, side, 3).permute(0, 3, 1, 2)
+    images = (f / f.abs().amax()).contiguous().to(dev)
+    g = torch.Generator().manual_seed(8)
+    noise = torch.randn(B, 3, side, side, generator=g).to(dev)
+    tsteps = torch.randint(0, 1000, (B,), generator=g).to(dev)
+
+    def time_fn(fn, warmup, steps):
+        for _ in range(warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    losses = []
+    ms = time_fn(lambda: losses.append(step(images, noise, tsteps)), args.warmup, args.steps)
+    losses = [float(l) for l in losses]
+    # the operator alone at the shape one layer gives it: (B, N, H, D) memory, qk norm and RoPE inside
+    x = (torch.randn(B, N, 3 * H * D, generator=torch.Generator().manual_seed(9)).bfloat16().to(dev))
+    q, k, v = (x[..., i * H * D:(i + 1) * H * D].reshape(B, N, H, D).transpose(1, 2).requires_grad_(True) for i in range(3))
+    do = torch.randn(B, N, H, D, generator=torch.Generator().manual_seed(10)).bfloat16().to(dev).transpose(1, 2)
+    gq = torch.ones(D, device=dev, requires_grad=True)
+    gk = torch.ones(D, device=dev, requires_grad=True)
+
+    def op_step():
+        q.grad = k.grad = v.grad = gq.grad = gk.grad = None
+        llsa_amd.llsa_l2(q, k, v, t1, t2, 16, rope=model.freq, qk_norm=(gq, gk, 1e-5)).backward(do)
+
+    ms_op = time_fn(op_step, 5, 20)
+    nparams = sum(p.numel() for p in model.parameters())
+    attn_flops = 14.0 * B * H * N * D * n_kv("l2", N, t1, t2) * layers
+    linear_flops = 6.0 * B * N * (nparams - 12 * (256 * 384 + 384 + 384 * 384 + 384 + 384 * 6 * 384 + 6 * 384))
+    print(json.dumps({
+        "metric": "pixel DiT-S training step with llsa_l2 in every attention layer, ms per step", "value": ms, "unit": "ms",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": False,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"c4: DiT-S {layers} layers hidden {H * D} heads {H}x{D}, batch {B} of 3x{side}x{side} (N={N} tokens, "
+                               f"Z-order), llsa_l2 topk {t1}/{t2}, qk RMS norm + RoPE "
+                               + ("composed before the operator" if args.unfused else "inside the operator")
+                               + ", bf16 autocast, AdamW, grad-norm clip 1.0",
+                   "parameters": nparams},
+        "images_per_s": B / (ms * 1e-3),
+        "operator": {"ms_fwd_bwd_one_layer": ms_op, "ms_all_layers": ms_op * layers, "share_of_step": ms_op * layers / ms,
+                     "tflops": attn_flops / layers / (ms_op * 1e-3) / 1e12},
+        "algorithmic_tflop_per_step": {"attention": attn_flops / 1e12, "linear_layers": linear_flops / 1e12},
+        "loss_first_last": [losses[0], losses[-1]],
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c4"])
     ap.add_argument("--no-extras", action="store_true", help="skip stage profile, CPU baseline and dense SDPA")
     ap.add_argument("--unfused", action="store_true", help="use the reference's composition (separate pools, autograd adds)")
     ap.add_argument("--graph", action="store_true",
@@ -197,6 +270,8 @@ def main():
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (one MI355X per box); --gpus must be 1", file=sys.stderr)
         sys.exit(2)
+    if args.workload == "c4":
+        return bench_dit(args)
 
     import torch
     import llsa_amd

@@ -270,20 +270,29 @@ __global__ __launch_bounds__(256) void rope_kernel(const bf16* x, Strides3 sx, c
 
 // ---------------------------------------------------------------------------------------
 // Backward of the RMS normalisation.  Thread mapping of the stand-alone RoPE: one thread per
-// (token, 8-channel chunk), 32 tokens per workgroup; a workgroup also sums dy * xn over its 32
-// tokens (fixed order) into one row of `partials`, which rmsnorm_dgamma_kernel adds up.
+// (token, 8-channel chunk), 32 tokens at a time, kNormTokens tokens per workgroup; a workgroup
+// also sums dy * xn over its tokens (fixed order) into one row of `partials`, which
+// rmsnorm_dgamma_kernel adds up.
 // ---------------------------------------------------------------------------------------
+constexpr int kNormTokens = 256;
+constexpr int kGammaGroups = 64;
+
 __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const bf16* dy, Strides3 sdy, const bf16* x, Strides3 sx,
                                                           const float* __restrict__ gamma, float eps, bf16* dx, Strides3 sdx,
                                                           float* __restrict__ partials, int H, int N) {
     __shared__ float red[32][kD];
     const int row = threadIdx.x >> 3, c = threadIdx.x & 7;
-    const int tok = blockIdx.x * 32 + row;
     const int bh = blockIdx.y, b = bh / H, h = bh % H;
-    float contrib[8];
+    float contrib[8], gam[8];
 #pragma unroll
-    for (int e = 0; e < 8; e++) contrib[e] = 0.f;
-    if (tok < N) {
+    for (int e = 0; e < 8; e++) {
+        contrib[e] = 0.f;
+        gam[e] = gamma[c * 8 + e];
+    }
+#pragma unroll 2
+    for (int it = 0; it < kNormTokens / 32; it++) {
+        const int tok = blockIdx.x * kNormTokens + it * 32 + row;
+        if (tok >= N) break;
         const bf16x8 xv = ld16(x + b * sx.b + h * sx.h + (int64_t)tok * sx.n + c * 8);
         const bf16x8 gv = ld16(dy + b * sdy.b + h * sdy.h + (int64_t)tok * sdy.n + c * 8);
         float ss = 0.f;
@@ -297,9 +306,9 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const bf16* dy, Stride
 #pragma unroll
         for (int e = 0; e < 8; e++) {
             xn[e] = (float)xv[e] * rstd;
-            g[e] = (float)gv[e] * gamma[c * 8 + e];
+            g[e] = (float)gv[e] * gam[e];
             dot += g[e] * xn[e];
-            contrib[e] = (float)gv[e] * xn[e];
+            contrib[e] += (float)gv[e] * xn[e];
         }
         dot += __shfl_xor(dot, 1);
         dot += __shfl_xor(dot, 2);
@@ -320,15 +329,19 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_kernel(const bf16* dy, Stride
     }
 }
 
-// one workgroup: thread (j, ch) adds rows j, j + 4, ... of `partials`, then the four j's are added
-__global__ __launch_bounds__(256) void rmsnorm_dgamma_kernel(const float* __restrict__ partials, float* __restrict__ dgamma, int64_t rows) {
+// Workgroup g of G adds rows g, g + G, g + 2G, ... of `partials` (thread (j, ch) every fourth of
+// them, then the four j's) into row g of `out`.  With out == partials a workgroup overwrites a
+// row that only it has read, so a first launch with G workgroups can fold the rows in place and
+// a second with one workgroup finishes.
+__global__ __launch_bounds__(256) void rmsnorm_dgamma_kernel(const float* partials, float* out, int64_t rows) {
     __shared__ float red[4][kD];
     const int ch = threadIdx.x & 63, j = threadIdx.x >> 6;
+    const int64_t G = gridDim.x;
     float s = 0.f;
-    for (int64_t r = j; r < rows; r += 4) s += partials[r * kD + ch];
+    for (int64_t r = blockIdx.x + j * G; r < rows; r += 4 * G) s += partials[r * kD + ch];
     red[j][ch] = s;
     __syncthreads();
-    if (j == 0) dgamma[ch] = (red[0][ch] + red[1][ch]) + (red[2][ch] + red[3][ch]);
+    if (j == 0) out[blockIdx.x * kD + ch] = (red[0][ch] + red[1][ch]) + (red[2][ch] + red[3][ch]);
 }
 
 }  // namespace llsa
@@ -480,7 +493,7 @@ extern "C" int llsa_gather_rows(const void* x, void* y, const int32_t* index, in
 
 extern "C" int64_t llsa_rmsnorm_bwd_partials(int B, int H, int N) {
     if (B <= 0 || H <= 0 || N <= 0) return -1;
-    return (int64_t)B * H * ((N + 31) / 32) * kD;
+    return (int64_t)B * H * ((N + kNormTokens - 1) / kNormTokens) * kD;
 }
 
 extern "C" int llsa_rmsnorm_bwd(const void* dy, const int64_t* sdy, const void* x, const int64_t* sx, const float* gamma, float eps,
@@ -490,10 +503,15 @@ extern "C" int llsa_rmsnorm_bwd(const void* dy, const int64_t* sdy, const void* 
     LLSA_REQUIRE(aligned16(dy) && aligned16(x) && aligned16(dx) && s3_ok(sdy) && s3_ok(sx) && s3_ok(sdx),
                  "rmsnorm_bwd: rows must be 16-byte aligned");
     Strides3 a{sdy[0], sdy[1], sdy[2]}, bx{sx[0], sx[1], sx[2]}, o{sdx[0], sdx[1], sdx[2]};
-    const int parts = (N + 31) / 32;
+    const int parts = (N + kNormTokens - 1) / kNormTokens;
+    int64_t rows = (int64_t)B * H * parts;
     hipLaunchKernelGGL(rmsnorm_bwd_kernel, dim3(parts, B * H), dim3(256), 0, (hipStream_t)stream, (const bf16*)dy, a, (const bf16*)x, bx,
                        gamma, eps, (bf16*)dx, o, partials, H, N);
-    hipLaunchKernelGGL(rmsnorm_dgamma_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (const float*)partials, dgamma,
-                       (int64_t)B * H * parts);
+    if (rows > 4 * kGammaGroups) {
+        hipLaunchKernelGGL(rmsnorm_dgamma_kernel, dim3(kGammaGroups), dim3(256), 0, (hipStream_t)stream, (const float*)partials,
+                           partials, rows);
+        rows = kGammaGroups;
+    }
+    hipLaunchKernelGGL(rmsnorm_dgamma_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (const float*)partials, dgamma, rows);
     return launch_status("rmsnorm_bwd");
 }

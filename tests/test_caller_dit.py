@@ -1,0 +1,151 @@
+"""The small DiT around the operator (llsa_amd/caller/dit.py): the same module is run once with
+the HIP kernels and once with every kernel replaced by the CPU oracle's function (attention,
+RMS norm, RoPE) or by plain indexing (token permutation); loss and parameter gradients of one
+flow-matching step must agree.  The torch layers are identical on both sides, so a difference
+comes from the operators or from how the module wires them."""
+import pytest
+import torch
+from torch.autograd import Function
+
+from oracle import llsa_oracle as O
+from emu_util import emu_lib
+from llsa_amd._lib import override_library_for_tests
+from llsa_amd.caller import dit as D
+
+
+class _OracleAttn(Function):
+    @staticmethod
+    def forward(ctx, q, k, v, levels, t1, t2):
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        if levels == 1:
+            o, c = O.llsa_l1_fwd(q, k, v, t1, 16)
+        else:
+            o, c = O.llsa_l2_fwd(q, k, v, t1, t2, 16)
+        ctx.c, ctx.levels = c, levels
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        bwd = O.llsa_l1_bwd if ctx.levels == 1 else O.llsa_l2_bwd
+        dq, dk, dv, _ = bwd(do.contiguous(), ctx.c)
+        return dq, dk, dv, None, None, None
+
+
+class _OracleRms(Function):
+    @staticmethod
+    def forward(ctx, x, g, eps):
+        ctx.save_for_backward(x, g)
+        ctx.eps = eps
+        return O.rms_norm(x, g, eps)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, g = ctx.saved_tensors
+        dx, dg = O.rms_norm_bwd(dy, x, g, ctx.eps)
+        return dx, dg.to(g.dtype), None
+
+
+class _OracleRope(Function):
+    @staticmethod
+    def forward(ctx, x, f):
+        ctx.save_for_backward(f)
+        return O.rope_apply(x, f)
+
+    @staticmethod
+    def backward(ctx, dy):
+        return O.rope_apply_bwd(dy, ctx.saved_tensors[0]), None
+
+
+def _oracle_ops(mp):
+    mp.setattr(D, "llsa_l1", lambda q, k, v, t, bs, rope=None, qk_norm=None: _OracleAttn.apply(q, k, v, 1, t, 0))
+    mp.setattr(D, "llsa_l2", lambda q, k, v, t1, t2, bs, rope=None, qk_norm=None: _OracleAttn.apply(q, k, v, 2, t1, t2))
+    mp.setattr(D, "my_rms_norm_fn", lambda x, g, eps: _OracleRms.apply(x.contiguous(), g, eps))
+    mp.setattr(D, "my_rope_fn", lambda x, f: _OracleRope.apply(x.contiguous(), f))
+    mp.setattr(D, "permute_tokens", lambda x, perm, inv: x[:, perm.long()])
+
+
+def _batch(B, side, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    images = torch.randn(B, 3, side, side, generator=g).clamp(-1, 1)
+    noise = torch.randn(B, 3, side, side, generator=g)
+    t = torch.randint(0, 1000, (B,), generator=g)
+    return images, noise, t
+
+
+def _loss_and_grads(model, batch, dev):
+    step = D.FlowMatchingStep(model)
+    loss = step.loss(*(x.to(dev) for x in batch))
+    loss.backward()
+    return loss.item(), {n: p.grad.detach().float().cpu() for n, p in model.named_parameters() if p.grad is not None}
+
+
+def _compare(dev, monkeypatch, fused, **cfg):
+    torch.manual_seed(3)
+    ref = D.PixelDiT(fused_prologue=False, **cfg)
+    with torch.no_grad():                       # the adaLN gates start at random values: every block contributes
+        for p in ref.parameters():
+            if p.dim() == 1 and p.numel() == 64:
+                p.uniform_(0.5, 1.5)
+    got = D.PixelDiT(fused_prologue=fused, **cfg)
+    got.load_state_dict(ref.state_dict())
+    got.to(dev)
+    batch = _batch(1, cfg["sample_size"])
+    loss, grads = _loss_and_grads(got, batch, dev)
+    with monkeypatch.context() as mp:
+        _oracle_ops(mp)
+        rloss, rgrads = _loss_and_grads(ref, batch, torch.device("cpu"))
+    assert abs(loss - rloss) <= 1e-2 * abs(rloss), (loss, rloss)
+    assert set(grads) == set(rgrads)
+    worst = ("", 0.0)
+    for n, g in grads.items():
+        r = rgrads[n]
+        err = ((g - r).norm() / r.norm().clamp_min(1e-12)).item()
+        if err > worst[1]:
+            worst = (n, err)
+    assert worst[1] <= 5e-2, f"gradient of {worst[0]} differs by rel-L2 {worst[1]:.3e}"
+
+
+def test_parameter_count_of_dit_s():
+    """DiT-S as the model file configures it: hidden 384, 12 blocks.  Per block: timestep embedder
+    (256->384->384), modulation 384->6*384, q/k/v/out 384->384 with biases, two 64-wide RMS weights,
+    MLP 384->1536->384."""
+    m = D.PixelDiT()
+    d = 384
+    block = (256 * d + d) + (d * d + d) + (d * 6 * d + 6 * d) + 4 * (d * d + d) + 2 * 64 + (d * 4 * d + 4 * d) + (4 * d * d + d)
+    total = 12 * block + (3 * d + d) + (d * 2 * d + 2 * d) + (d * 3 + 3)
+    assert sum(p.numel() for p in m.parameters()) == total
+
+
+def test_timestep_channels():
+    t = torch.tensor([0.0, 1.0, 999.0])
+    e = D.timestep_channels(t)
+    assert e.shape == (3, 256)
+    assert torch.allclose(e[0, :128], torch.ones(128)) and torch.allclose(e[0, 128:], torch.zeros(128))
+    assert torch.allclose(e[1, 0], torch.cos(torch.tensor(1.0))) and torch.allclose(e[1, 128], torch.sin(torch.tensor(1.0)))
+    assert torch.allclose(e[2, 127], torch.cos(torch.tensor(999.0 / 10000.0)), atol=1e-6)
+
+
+@pytest.mark.parametrize("fused", [True, False])
+def test_step_against_oracle_ops_emulated(monkeypatch, fused):
+    with override_library_for_tests(emu_lib()):
+        _compare(torch.device("cpu"), monkeypatch, fused, num_attention_heads=1, num_layers=2, sample_size=32, levels=1,
+                 sparse_topk=8)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("fused,levels,side", [(True, 2, 128), (False, 2, 128), (True, 1, 64)])
+def test_step_against_oracle_ops_gpu(monkeypatch, fused, levels, side):
+    _compare(torch.device("cuda:0"), monkeypatch, fused, num_attention_heads=2, num_layers=2, sample_size=side,
+             levels=levels, sparse_topk=8)
+
+
+@pytest.mark.gpu
+def test_training_reduces_the_loss():
+    torch.manual_seed(0)
+    dev = torch.device("cuda:0")
+    model = D.PixelDiT(num_attention_heads=2, num_layers=2, sample_size=64, levels=1).to(dev)
+    step = D.FlowMatchingStep(model, lr=1e-3)
+    batch = [x.to(dev) for x in _batch(2, 64)]
+    losses = [step(*batch).item() for _ in range(12)]
+    assert all(l == l for l in losses)
+    assert losses[-1] < 0.8 * losses[0], losses

@@ -55,6 +55,7 @@ def test_permute(dev):
 def test_rms_norm(dev):
     P.check_rms_norm(dev, B=2, H=3, N=4096, strided=True)
     P.check_rms_norm(dev, B=1, H=1, N=16, strided=False)
+    P.check_rms_norm(dev, B=4, H=6, N=16384, strided=True)        # 1536 partial rows: folded in two launches
 
 
 def test_op_with_qk_norm(dev):
