@@ -20,3 +20,11 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture(autouse=True)
+def _seed_every_test():
+    """Tests that draw from torch's global generator see the same numbers whatever ran before them."""
+    import torch
+    torch.manual_seed(1234)
+    yield

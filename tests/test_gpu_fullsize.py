@@ -27,6 +27,24 @@ def dev():
     return torch.device("cuda:0")
 
 
+def test_c1_inputs_in_bf16(dev):
+    """Benchmark configuration 1 (llsa_l1, B=1, H=6, N=1024, topk 8, N(0,1) inputs) is an fp32 CPU case
+    of the reference; the kernels are bf16, so the same inputs are rounded to bf16 and checked against
+    the oracle in bf16 (forward and backward), and the output against the fp32 oracle on the
+    operator's own selection within the bf16 tolerance."""
+    import llsa_amd
+    from oracle import llsa_oracle as O
+    from llsa_amd.kernel.torch_op._fused import selection
+    P.check_op_l1(dev, B=1, H=6, N=1024, T=8, fused=True, rope=False)
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(1, 6, 1024, 64, generator=g) for _ in range(3))
+    out = llsa_amd.llsa_l1(*(t.bfloat16().to(dev).requires_grad_(True) for t in (q, k, v)), 8, 16)
+    idx = selection(out)[0].cpu().long()
+    ref, _ = O.llsa_l1_fwd(q, k, v, 8, 16, indices=idx)
+    err = (out.detach().float().cpu() - ref)
+    assert err.norm() / ref.norm() <= 1e-2 and err.abs().max() <= 2e-2
+
+
 def test_c2_full_size_against_oracle(dev):
     P.check_op_l1(dev, B=4, H=6, N=4096, T=16, fused=True, rope=False, smooth=True)
 

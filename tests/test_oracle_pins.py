@@ -235,6 +235,24 @@ def test_forward_l1_matches_closed_form_fp32():
     assert (ow - oc).abs().max() > 1e-2
 
 
+def test_benchmark_configuration_1_fp32():
+    """The reference's own CPU-runnable case: llsa_l1 forward, B=1, H=6, N=1024, D=64, fp32, block 16,
+    topk 8, q, k, v ~ N(0,1) from a fixed seed.  Selection against a brute-force sort (fp32 scores of
+    random data do not tie), output against the fp64 closed form on that selection."""
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(1, 6, 1024, 64, generator=g) for _ in range(3))
+    o, ctx = O.llsa_l1_fwd(q, k, v, 8, 16)
+    idx = ctx["indices"]
+    pq, pk, pv = q.reshape(1, 6, 64, 16, 64).mean(3), k.reshape(1, 6, 64, 16, 64).mean(3), v.reshape(1, 6, 64, 16, 64).mean(3)
+    score = torch.einsum("bhqd,bhkd->bhqk", pq.double(), pk.double())
+    for h in range(6):
+        for r in range(64):
+            want = sorted(range(64), key=lambda j: -score[0, h, r, j].item())[:8]
+            assert idx[0, h, r].tolist() == want
+    oc, _ = O.closed_form_l1(q.double(), k.double(), v.double(), pk.double(), pv.double(), idx, 16)
+    assert torch.allclose(o.double(), oc, atol=2e-5)
+
+
 def test_forward_l1_explicit_formula_one_query():
     """L_i = sum_fine e^s + w sum_coarse e^s, O_i = (sum_fine e^s v + w sum_coarse e^s pv) / L_i, by hand."""
     q, k, v, pk, pv, idx = _rand_problem(1, 1, 1024, 16, 4, torch.float64, seed=3)
@@ -335,8 +353,9 @@ def test_backward_l2_matches_autograd_of_closed_form():
 
 
 def test_delta_variants():
-    o = torch.randn(1, 1, 8, 64).bfloat16()
-    do = torch.randn(1, 1, 8, 64).bfloat16()
+    g = torch.Generator().manual_seed(11)
+    o = torch.randn(1, 1, 8, 64, generator=g).bfloat16()
+    do = torch.randn(1, 1, 8, 64, generator=g).bfloat16()
     d32 = O.attn_delta(o, do)
     assert torch.allclose(d32, (o.double() * do.double()).sum(-1).float(), atol=1e-5)
     dbf = O.attn_delta(o, do, in_dtype=True)
