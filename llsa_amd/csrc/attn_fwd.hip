@@ -25,8 +25,10 @@
 
 namespace llsa {
 
+constexpr float kMaxSlack = 8.f;     // log2 units
+
 struct SoftmaxState {
-    float m2;        // running max, in log2 units (score / sqrt(D) * log2 e)
+    float m2;        // reference point of the exponentials (at most kMaxSlack below the running max), log2 units
     float lsum;      // this lane's share of the running sum, in units of the current weight
     f32x4 acc[4];    // O^T: channel 16*dt + 4*(l/16) + e of query l%16
 };
@@ -74,7 +76,12 @@ __device__ __forceinline__ void compute_step(SoftmaxState& st, const bf16x8 bq[2
 #pragma unroll
         for (int e = 0; e < 4; e++) mx = fmaxf(mx, s[j][e]);
     mx = quad_max(mx);
-    const float m2n = fmaxf(st.m2, mx * kScaleLog2e);
+    // The exponentials refer to st.m2, which follows the running maximum lazily: it moves only when the
+    // maximum has grown by more than kMaxSlack (then p <= 2^kMaxSlack, harmless in bf16 and in the fp32
+    // sums), so that the accumulator is rescaled a few times per query block instead of at most steps.
+    // O = acc / lsum and lse = m2 + log2(lsum) hold for any reference point.
+    const float cand = mx * kScaleLog2e;
+    const float m2n = (cand > st.m2 + kMaxSlack) ? cand : st.m2;
     const float alpha = exp2_fast(st.m2 - m2n) * wratio;
     float rs = 0.f;
     bf16x8 bp[NB / 2];
@@ -208,6 +215,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(llsa_attn_fwd_args a) {
         compute_step(st, bq, rb, 1.f);
     }
 
+    wait_all_mem();     // nothing is in flight here: said for the compiler (see wait_all_mem)
     // ---- fine blocks, private to the wave.  Their indices are fetched 64 at a time, entry i into
     // lane i, and handed out with readlane (a copy into LDS counts as a store for the compiler,
     // after which it no longer turns uniform loads into scalar loads; a vector load inside the

@@ -64,16 +64,23 @@ __device__ __forceinline__ float rn_bf16(float x) { return (float)(bf16)x; }
 
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// reductions over the four lanes {l, l^16, l^32, l^48} that share one MFMA column
+// Reductions over the four lanes {l, l^16, l^32, l^48} that share one MFMA column, with the lane
+// swaps of gfx950 (v_permlane16_swap, v_permlane32_swap: vector-ALU instructions, where a shuffle
+// goes through the LDS unit and makes the wave wait for it).  swap16(v, v) leaves in its two
+// results v of this lane and v of lane l^16 (which is which depends on the row), swap32 the same
+// for l^32; both reductions are symmetric, so every lane of the four ends with the same bits.
+typedef __attribute__((ext_vector_type(2))) unsigned u32x2;
 __device__ __forceinline__ float quad_max(float v) {
-    v = fmaxf(v, __shfl_xor(v, 16));
-    v = fmaxf(v, __shfl_xor(v, 32));
-    return v;
+    u32x2 a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+    u32x2 b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
 }
 __device__ __forceinline__ float quad_sum(float v) {
-    v += __shfl_xor(v, 16);
-    v += __shfl_xor(v, 32);
-    return v;
+    u32x2 a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    u32x2 b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
 }
 
 // Operand tiles.  The attention kernels never read K/V/Q/dO row-major: a 16-row x 64-channel
@@ -115,6 +122,9 @@ __device__ __forceinline__ void copy16_global_to_lds(const bf16* g_lane, bf16* l
                                      (__attribute__((address_space(3))) void*)lds_wave_base, 16, 0, 0);
 }
 __device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }   // vmcnt(0), other counters untouched
+// vmcnt(0) and lgkmcnt(0).  The compiler books a copy into LDS against both counters; until it has seen
+// both drained it takes the vector-memory queue for out of order and turns every later wait into vmcnt(0).
+__device__ __forceinline__ void wait_all_mem() { __builtin_amdgcn_s_waitcnt(0x0070); }
 
 // Rotates a gradient back through the 2-D RoPE: 4 consecutive channels = two (even, odd) pairs, f
 // holds their [sin, cos] entries.  Every product and sum is rounded to bf16 like the forward rotation.

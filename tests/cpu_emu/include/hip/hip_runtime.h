@@ -93,6 +93,20 @@ inline T __shfl_up(T v, unsigned d, int width = 64) {
     return __shfl(v, (l >= (int)d) ? l - (int)d : l, width);
 }
 inline uint64_t __ballot(int pred) { return emu::ballot(pred != 0); }
+// v_permlane16_swap / v_permlane32_swap of gfx950: rows of 16 lanes [r0 r1 r2 r3] of a and [s0 s1 s2 s3] of b become
+// a' = [r0 s0 r2 s2], b' = [r1 s1 r3 s3]; halves of 32 lanes [a_lo a_hi], [b_lo b_hi] become a' = [a_lo b_lo], b' = [a_hi b_hi]
+typedef __attribute__((ext_vector_type(2))) unsigned emu_u32x2;
+inline emu_u32x2 emu_permlane_swap(unsigned a, unsigned b, int width) {
+    const int l = emu::lane_id();
+    const bool upper = (l & width) != 0;
+    const unsigned b_below = __shfl(b, (l - width) & 63), a_above = __shfl(a, (l + width) & 63);
+    emu_u32x2 r;
+    r[0] = upper ? b_below : a;
+    r[1] = upper ? b : a_above;
+    return r;
+}
+#define __builtin_amdgcn_permlane16_swap(a, b, fi, bc) emu_permlane_swap((a), (b), 16)
+#define __builtin_amdgcn_permlane32_swap(a, b, fi, bc) emu_permlane_swap((a), (b), 32)
 inline int __popcll(unsigned long long x) { return __builtin_popcountll(x); }
 inline int __popc(unsigned x) { return __builtin_popcount(x); }
 inline int __ffsll(unsigned long long x) { return __builtin_ffsll(x); }
