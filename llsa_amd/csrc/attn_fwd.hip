@@ -134,7 +134,7 @@ __device__ __forceinline__ void load_step_lds(KvRegs<NB>& t, const bf16* blocks,
 // undo the register ping-pong.  This is what bounds the kernel: without the sharing every wave
 // pulls all of its 4 KB per block through the L2, and the L2's bandwidth, not the MFMA, sets the time.
 template <int NB>
-__global__ __launch_bounds__(256) void attn_fwd_kernel(llsa_attn_fwd_args a) {
+__global__ __launch_bounds__(256, 4) void attn_fwd_kernel(llsa_attn_fwd_args a) {
     static_assert(NB == 2, "the shared phase reads an LDS buffer as two steps of two blocks");
     __shared__ __align__(16) bf16 sh[2][kGroup][2 * kTile];
     const int lane = threadIdx.x & 63;

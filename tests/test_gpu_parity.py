@@ -128,6 +128,22 @@ def test_op_l2(dev, fused, rope):
     P.check_op_l2(dev, B=1, H=2, N=16384, T=16, T2=16, fused=fused, rope=rope, smooth=True)
 
 
+@pytest.mark.parametrize("B,H,N,T", [(1, 1, 1024, 4), (3, 1, 3072, 12), (1, 5, 5120, 16), (2, 3, 2048, 32), (1, 2, 7168, 64),
+                                     (1, 7, 1024, 64)])
+def test_op_l1_shapes(dev, B, H, N, T):
+    """Token counts that are not powers of two (any multiple of 1024), odd batch and head counts, every
+    topk the kernels take (multiples of 4 up to N/16)."""
+    P.check_op_l1(dev, B=B, H=H, N=N, T=T, fused=True, rope=False, strided=(B + H) % 2 == 1)
+
+
+@pytest.mark.parametrize("B,H,N,T,T2", [(1, 1, 16384, 4, 4), (1, 3, 32768, 12, 8), (2, 1, 49152, 16, 12), (1, 2, 16384, 32, 16),
+                                        (1, 1, 16384, 64, 64), (3, 2, 16384, 8, 8)])
+def test_op_l2_shapes(dev, B, H, N, T, T2):
+    """Multiples of 16384 tokens that are not squares, topk1 up to 64 and topk2 up to N/256 (then every
+    coarse block is selected and the level-1 candidates are all of level 1)."""
+    P.check_op_l2(dev, B=B, H=H, N=N, T=T, T2=T2, fused=True, rope=False)
+
+
 @pytest.mark.skip(reason="capturing this case (B=1, H=2, N=16384, topk 8/4) ended in a segmentation fault of the host "
                          "process inside torch.cuda.graph's capture_end (hipStreamEndCapture), twice; the cause is not "
                          "known, so the case stays off the GPU.  The same capture and replay at the bench shapes "
