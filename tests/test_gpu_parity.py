@@ -137,11 +137,23 @@ def test_op_l1_shapes(dev, B, H, N, T):
 
 
 @pytest.mark.parametrize("B,H,N,T,T2", [(1, 1, 16384, 4, 4), (1, 3, 32768, 12, 8), (2, 1, 49152, 16, 12), (1, 2, 16384, 32, 16),
-                                        (1, 1, 16384, 64, 64), (3, 2, 16384, 8, 8)])
+                                        (1, 1, 16384, 64, 32), (3, 2, 16384, 8, 8)])
 def test_op_l2_shapes(dev, B, H, N, T, T2):
-    """Multiples of 16384 tokens that are not squares, topk1 up to 64 and topk2 up to N/256 (then every
-    coarse block is selected and the level-1 candidates are all of level 1)."""
+    """Multiples of 16384 tokens that are not squares, topk1 up to 64 and topk2 up to 32, the largest the
+    selection kernels take."""
     P.check_op_l2(dev, B=B, H=H, N=N, T=T, T2=T2, fused=True, rope=False)
+
+
+def test_selection_limits_are_errors(dev):
+    import llsa_amd
+    from llsa_amd._lib import LlsaError
+    x = torch.randn(1, 1, 16384, 64).bfloat16().to(dev)
+    with pytest.raises(LlsaError, match="T2 <= min"):
+        llsa_amd.llsa_l2(x, x, x, 16, 64, 16)
+    with pytest.raises(LlsaError, match="T <= min"):
+        llsa_amd.llsa_l2(x, x, x, 128, 16, 16)
+    with pytest.raises(ValueError, match="multiple of 16384"):
+        llsa_amd.llsa_l2(x[:, :, :4096], x[:, :, :4096], x[:, :, :4096], 8, 8, 16)
 
 
 @pytest.mark.skip(reason="capturing this case (B=1, H=2, N=16384, topk 8/4) ended in a segmentation fault of the host "
