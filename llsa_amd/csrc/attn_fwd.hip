@@ -207,7 +207,7 @@ __global__ __launch_bounds__(256, 4) void attn_fwd_kernel(llsa_attn_fwd_args a) 
         // weight(previous segment) / weight(this one); nothing is accumulated before group 0
         const float wr = (a.levels == 2 && kGroup * grp == n_mid) ? a.w1 / a.w2 : 1.f;
         // (LDS reads first: the compiler makes every LDS read wait for all copies into LDS that
-        // were issued before it, which would serialise the next fetch with this round's arithmetic)
+        // were issued before it, which would serialise the next fetch with the arithmetic of this group)
         load_step_lds(ra, &sh[grp & 1][0][0], lane);
         load_step_lds(rb, &sh[grp & 1][NB][0], lane);
         if (grp + 1 < n_groups) issue_group(grp + 1);
