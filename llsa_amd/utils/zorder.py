@@ -41,6 +41,8 @@ def gen_permutations(log_num_tokens: int):
 gen_permuatations = gen_permutations      # the reference's spelling
 
 
+# Host-side helpers for preparing inputs and tables (plain indexing on whatever device x lives on).
+# Inside a model the permutation of (B, N, C) activations is llsa_amd.permute_tokens, a HIP kernel.
 def to_zorder(x: torch.Tensor, side: int, dim: int = 1) -> torch.Tensor:
     _, inv_perm = zorder_perm(side)
     return x.index_select(dim, inv_perm.to(x.device))
