@@ -144,6 +144,33 @@ def test_op_l2_shapes(dev, B, H, N, T, T2):
     P.check_op_l2(dev, B=B, H=H, N=N, T=T, T2=T2, fused=True, rope=False)
 
 
+@pytest.mark.parametrize("levels", [1, 2])
+def test_step_is_deterministic(dev, levels):
+    """Every reduction has a fixed order (sorted CSR segments, partial sums added in chunk order, no
+    atomics in the floating-point path), so two runs give the same bits -- with hot key blocks, whose
+    lists are cut into chunks, and with other work in between."""
+    import math
+    import llsa_amd
+    from llsa_amd.utils.rope_table import rope_table
+    B, H, N = 2, 3, 16384
+    q, k, v, do = P.smooth_inputs(B, H, N, 64, dev)
+    k[:, :, 160:176] *= 3.0                            # a key block that very many query blocks select
+    freq = rope_table(math.isqrt(N), dtype=torch.bfloat16).to(dev)
+    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+
+    def step():
+        q.grad = k.grad = v.grad = None
+        o = llsa_amd.llsa_l2(q, k, v, 16, 16, 16, rope=freq) if levels == 2 else llsa_amd.llsa_l1(q, k, v, 16, 16, rope=freq)
+        o.backward(do)
+        torch.cuda.synchronize()
+        return [t.clone() for t in (o, q.grad, k.grad, v.grad)]
+
+    first = step()
+    torch.randn(1 << 22, device=dev).sum().item()      # other kernels and allocations in between
+    for name, a, b in zip(("o", "dq", "dk", "dv"), first, step()):
+        assert torch.equal(a, b), f"{name} differs between two runs of the same step"
+
+
 def test_selection_limits_are_errors(dev):
     import llsa_amd
     from llsa_amd._lib import LlsaError
