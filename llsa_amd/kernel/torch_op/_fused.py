@@ -24,6 +24,7 @@ from torch.autograd import Function
 from ..._lib import CHUNK_COARSE, CHUNK_FINE, AttnBwdArgs, AttnFwdArgs, PoolItem, current_lib
 
 _side = {}          # device -> (second stream, two events)
+_SIDE_STREAM_MIN_TOKENS = 1 << 17
 
 
 def _rows_ok(t):
@@ -189,8 +190,10 @@ class LlsaFused(Function):
         # The lists of the backward go to a second stream, beside the attention kernel.  The attention
         # kernel is issued first (the GPU is waiting for it); an event recorded before it lets the
         # second stream start as soon as the selection is done.
+        # (Below _SIDE_STREAM_MIN_TOKENS tokens over all heads the step is bound by the host, which the two
+        # event waits cost 30 us; the GPU then has the time to build the lists on the one stream.)
         cur = side = None
-        if grad and lib.device_library:
+        if grad and lib.device_library and B * H * N >= _SIDE_STREAM_MIN_TOKENS:
             cur = torch.cuda.current_stream(dev)
             pack = _side.get(dev)
             if pack is None:
