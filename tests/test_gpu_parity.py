@@ -171,6 +171,38 @@ def test_step_is_deterministic(dev, levels):
         assert torch.equal(a, b), f"{name} differs between two runs of the same step"
 
 
+def test_mixed_layouts_and_partial_grads(dev):
+    """q in (B,N,H,D) memory, k contiguous, v a slice of a packed projection; the output of a no-grad call
+    equals the output of a call that records the backward; gradients arrive in the layout of their
+    inputs, and asking for only some of them changes none of the values."""
+    import llsa_amd
+    B, H, N = 2, 3, 4096
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(B, N, H, 64, generator=g).bfloat16().to(dev).transpose(1, 2)
+    k = torch.randn(B, H, N, 64, generator=g).bfloat16().to(dev)
+    packed = torch.randn(B, N, 2 * H * 64, generator=g).bfloat16().to(dev)
+    v = packed[..., H * 64:].reshape(B, N, H, 64).transpose(1, 2)
+    do = torch.randn(B, N, H, 64, generator=g).bfloat16().to(dev).transpose(1, 2)
+    with torch.no_grad():
+        o0 = llsa_amd.llsa_l1(q, k, v, 8, 16)
+    qa, ka, va = (t.detach().requires_grad_(True) for t in (q, k, v))
+    o1 = llsa_amd.llsa_l1(qa, ka, va, 8, 16)
+    assert torch.equal(o0, o1) and o1.stride() == q.stride()
+    from llsa_amd.kernel.torch_op._fused import selection
+    idx = selection(o1)[0].cpu().long()              # (the node's saved tensors are gone after the backward)
+    o1.backward(do)
+    assert qa.grad.stride() == q.stride() and ka.grad.is_contiguous()
+    qb, kb, vb = q.detach(), k.detach(), v.detach().requires_grad_(True)       # only dV asked for
+    llsa_amd.llsa_l1(qb, kb, vb, 8, 16).backward(do)
+    assert torch.equal(vb.grad, va.grad)
+    # and against the oracle on the same inputs
+    from oracle import llsa_oracle as O
+    ro, ctx = O.llsa_l1_fwd(q.cpu().contiguous(), k.cpu(), v.cpu().contiguous(), 8, 16, indices=idx)
+    rq, rk, rv, _ = O.llsa_l1_bwd(do.cpu().contiguous(), ctx)
+    for name, a, b in (("o", o1, ro), ("dq", qa.grad, rq), ("dk", ka.grad, rk), ("dv", va.grad, rv)):
+        P.close(name, a, b)
+
+
 def test_selection_limits_are_errors(dev):
     import llsa_amd
     from llsa_amd._lib import LlsaError
