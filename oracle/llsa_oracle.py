@@ -298,9 +298,9 @@ def _gather_blocks(x: torch.Tensor, idx: torch.Tensor, bs: int) -> torch.Tensor:
     B, H, n, D = x.shape
     G, T = idx.shape[2], idx.shape[3]
     xb = x.reshape(B, H, n // bs, bs * D)
-    g = torch.gather(xb[:, :, None].expand(B, H, G, n // bs, bs * D), 3,
-                     idx.long()[..., None].expand(B, H, G, T, bs * D))
-    return g.reshape(B, H, G, T * bs, D)
+    bi = torch.arange(B)[:, None, None, None]
+    hi = torch.arange(H)[None, :, None, None]
+    return xb[bi, hi, idx.long()].reshape(B, H, G, T * bs, D)
 
 
 def _segments_l1(q, k, v, pk, pv, indices, token_weight, bs):
@@ -326,6 +326,24 @@ def _segments_l2(q, k, v, pk, pv, pk2, pv2, indices, p_indices, w1, w2, bs):
     k2 = pk2[:, :, None].expand(B, H, N1, pk2.shape[2], D)
     v2 = pv2[:, :, None].expand(B, H, N1, pv2.shape[2], D)
     return [(kf, vf, 1.0), (k1, v1, float(w1)), (k2, v2, float(w2))]
+
+
+def _segments_l3(q, k, v, pk, pv, pk2, pv2, pk3, pv3, indices, p_indices, pp_indices, w1, w2, w3, bs):
+    """Three pooled levels, the two-level scheme (sparse_attention_res_2.py:94-149) continued by one step: a
+    query block sees its selected fine blocks, the level-1 pooled tokens inside its parent's selected level-1
+    blocks, the level-2 pooled tokens inside its grand-parent's selected level-2 blocks, and every level-3
+    pooled token.  The reference stops at two levels; there is nothing of its to compare this with."""
+    B, H, N, D = q.shape
+    N1 = N // bs
+    kf = _gather_blocks(k, indices, bs)
+    vf = _gather_blocks(v, indices, bs)
+    par = p_indices.long().repeat_interleave(bs, dim=2)              # (B,H,N1,T2): parent of block g is g // bs
+    k1, v1 = _gather_blocks(pk, par, bs), _gather_blocks(pv, par, bs)
+    gpar = pp_indices.long().repeat_interleave(bs * bs, dim=2)       # (B,H,N1,T3): grand-parent is g // bs^2
+    k2, v2 = _gather_blocks(pk2, gpar, bs), _gather_blocks(pv2, gpar, bs)
+    k3 = pk3[:, :, None].expand(B, H, N1, pk3.shape[2], D)
+    v3 = pv3[:, :, None].expand(B, H, N1, pv3.shape[2], D)
+    return [(kf, vf, 1.0), (k1, v1, float(w1)), (k2, v2, float(w2)), (k3, v3, float(w3))]
 
 
 def _online_softmax(q, segments, bs, tile=64):
@@ -368,6 +386,12 @@ def attn_fwd_l2(q, k, v, pk, pv, pk2, pv2, indices, p_indices, token_weight=16, 
     return _online_softmax(q, seg, block_size)
 
 
+def attn_fwd_l3(q, k, v, pk, pv, pk2, pv2, pk3, pv3, indices, p_indices, pp_indices, w1=16, w2=256, w3=4096, block_size=16):
+    """Three-level forward, same tile loop (no counterpart in the reference)."""
+    seg = _segments_l3(q, k, v, pk, pv, pk2, pv2, pk3, pv3, indices, p_indices, pp_indices, w1, w2, w3, block_size)
+    return _online_softmax(q, seg, block_size)
+
+
 # --------------------------------------------------------------------------------------
 # closed form (fp64), used to pin the faithful forward/backward above
 # --------------------------------------------------------------------------------------
@@ -397,6 +421,11 @@ def closed_form_l1(q, k, v, pk, pv, indices, token_weight=16, bs=16):
 
 def closed_form_l2(q, k, v, pk, pv, pk2, pv2, indices, p_indices, w1=16, w2=256, bs=16):
     return attn_closed_form(q, _segments_l2(q, k, v, pk, pv, pk2, pv2, indices, p_indices, w1, w2, bs), bs)
+
+
+def closed_form_l3(q, k, v, pk, pv, pk2, pv2, pk3, pv3, indices, p_indices, pp_indices, w1=16, w2=256, w3=4096, bs=16):
+    return attn_closed_form(q, _segments_l3(q, k, v, pk, pv, pk2, pv2, pk3, pv3, indices, p_indices, pp_indices,
+                                            w1, w2, w3, bs), bs)
 
 
 # --------------------------------------------------------------------------------------
@@ -499,6 +528,33 @@ def attn_bwd_l2(do, q, k, v, pk, pv, pk2, pv2, o, lse, indices, p_indices, token
     return tuple(_rn(x, dt).to(dt) for x in (dq, dk, dv, dpk, dpv, dpk2, dpv2))
 
 
+def attn_bwd_l3(do, q, k, v, pk, pv, pk2, pv2, pk3, pv3, o, lse, indices, p_indices, pp_indices, w1=16, w2=256, w3=4096,
+                block_size=16, delta_in_dtype=False):
+    """Backward of the three-level forward, the two-level launcher continued by one level: every pooled path
+    carries its weight.  Returns dq, dk, dv, dpk, dpv, dpk2, dpv2, dpk3, dpv3."""
+    B, H, N, D = q.shape
+    bs, dt = block_size, q.dtype
+    G = N // bs
+    scale = 1.0 / math.sqrt(D)
+    qb = q.float().reshape(B, H, G, bs, D)
+    dob = do.float().reshape(B, H, G, bs, D)
+    lse_b = lse.reshape(B, H, G, bs)
+    delta = attn_delta(o, do, delta_in_dtype).reshape(B, H, G, bs)
+    segs = _segments_l3(q, k, v, pk, pv, pk2, pv2, pk3, pv3, indices, p_indices, pp_indices, w1, w2, w3, bs)
+    parts = [_bwd_segment(qb, dob, lse_b, delta, ks, vs, w, scale, dt) for ks, vs, w in segs]
+    dq = sum(p[0] for p in parts).reshape(B, H, N, D)
+    dk = _scatter_blocks(torch.zeros(B, H, N, D), parts[0][1], indices, bs)
+    dv = _scatter_blocks(torch.zeros(B, H, N, D), parts[0][2], indices, bs)
+    par = p_indices.long().repeat_interleave(bs, dim=2)
+    dpk = _scatter_blocks(torch.zeros(B, H, pk.shape[2], D), parts[1][1], par, bs)
+    dpv = _scatter_blocks(torch.zeros(B, H, pv.shape[2], D), parts[1][2], par, bs)
+    gpar = pp_indices.long().repeat_interleave(bs * bs, dim=2)
+    dpk2 = _scatter_blocks(torch.zeros(B, H, pk2.shape[2], D), parts[2][1], gpar, bs)
+    dpv2 = _scatter_blocks(torch.zeros(B, H, pv2.shape[2], D), parts[2][2], gpar, bs)
+    dpk3, dpv3 = parts[3][1].sum(2), parts[3][2].sum(2)
+    return tuple(_rn(x, dt).to(dt) for x in (dq, dk, dv, dpk, dpv, dpk2, dpv2, dpk3, dpv3))
+
+
 # --------------------------------------------------------------------------------------
 # whole operators  --  torch_op/flash_sparse_attention_res_{1,2}.py
 # --------------------------------------------------------------------------------------
@@ -559,3 +615,37 @@ def llsa_l2_bwd(do, ctx, delta_in_dtype=False):
     dk = dk + mean_pool_bwd(dpk_t, bs)
     dv = dv + mean_pool_bwd(dpv_t, bs)
     return dq, dk, dv, dict(dpk=dpk, dpv=dpv, dpk2=dpk2, dpv2=dpv2)
+
+
+def llsa_l3_fwd(q, k, v, topk1=8, topk2=8, topk3=8, block_size=16, indices=None, p_indices=None, pp_indices=None):
+    """Three levels (no counterpart in the reference, whose deepest operator is llsa_l2): dense selection on the
+    level-3 pooled tokens, then parent-guided selection twice, as llsa_l2 does once."""
+    bs = block_size
+    pq, pk, pv = mean_pool(q, bs), mean_pool(k, bs), mean_pool(v, bs)
+    pq2, pk2, pv2 = mean_pool(pq, bs), mean_pool(pk, bs), mean_pool(pv, bs)
+    pq3, pk3, pv3 = mean_pool(pq2, bs), mean_pool(pk2, bs), mean_pool(pv2, bs)
+    if pp_indices is None:
+        pp_indices = gen_sparse_indices(pq3, pk3, topk3)
+    if p_indices is None:
+        p_indices = topk_sparse(pq2, pk2, pp_indices, topk2, bs)
+    if indices is None:
+        indices = topk_sparse(pq, pk, p_indices, topk1, bs)
+    o, lse = attn_fwd_l3(q, k, v, pk, pv, pk2, pv2, pk3, pv3, indices, p_indices, pp_indices, bs, bs * bs, bs ** 3, bs)
+    return o, dict(q=q, k=k, v=v, pq=pq, pk=pk, pv=pv, pq2=pq2, pk2=pk2, pv2=pv2, pq3=pq3, pk3=pk3, pv3=pv3, o=o, lse=lse,
+                   indices=indices, p_indices=p_indices, pp_indices=pp_indices, block_size=bs)
+
+
+def llsa_l3_bwd(do, ctx, delta_in_dtype=False):
+    """Backward of llsa_l3 with the chain of pool backwards autograd would add around it."""
+    c = ctx
+    bs = c["block_size"]
+    dq, dk, dv, dpk, dpv, dpk2, dpv2, dpk3, dpv3 = attn_bwd_l3(
+        do, c["q"], c["k"], c["v"], c["pk"], c["pv"], c["pk2"], c["pv2"], c["pk3"], c["pv3"], c["o"], c["lse"],
+        c["indices"], c["p_indices"], c["pp_indices"], bs, bs * bs, bs ** 3, bs, delta_in_dtype=delta_in_dtype)
+    dpk2_t = dpk2 + mean_pool_bwd(dpk3, bs)
+    dpv2_t = dpv2 + mean_pool_bwd(dpv3, bs)
+    dpk_t = dpk + mean_pool_bwd(dpk2_t, bs)
+    dpv_t = dpv + mean_pool_bwd(dpv2_t, bs)
+    dk = dk + mean_pool_bwd(dpk_t, bs)
+    dv = dv + mean_pool_bwd(dpv_t, bs)
+    return dq, dk, dv, dict(dpk=dpk, dpv=dpv, dpk2=dpk2, dpv2=dpv2, dpk3=dpk3, dpv3=dpv3)

@@ -352,6 +352,44 @@ def test_backward_l2_matches_autograd_of_closed_form():
         assert (a.double() - b).norm() / b.norm() < 2e-5
 
 
+def test_three_levels_match_closed_form_and_its_autograd():
+    """llsa_l3 has no counterpart in the reference; what can be pinned is that the faithful tile loop and the
+    explicit backward of the three-level oracle are the soft-max over the four weighted segments and its
+    gradient (fp64 closed form, torch.autograd), including the whole-operator composition with the chain of
+    pool backwards.  N = 262144 is the smallest size with a full 64-token tile of level-3 tokens; D = 8 keeps it small."""
+    g = torch.Generator().manual_seed(9)
+    B, H, N, D = 1, 1, 262144, 8
+    q, k, v, do = (torch.randn(B, H, N, D, generator=g) for _ in range(4))
+    o, ctx = O.llsa_l3_fwd(q, k, v, 4, 4, 4)
+    idx, pidx, ppidx = ctx["indices"], ctx["p_indices"], ctx["pp_indices"]
+    assert idx.shape == (1, 1, N // 16, 4) and pidx.shape == (1, 1, N // 256, 4) and ppidx.shape == (1, 1, N // 4096, 4)
+    # every selected block lies under a block its parent selected
+    par = pidx.long().repeat_interleave(16, dim=2)
+    assert ((idx.long()[..., :, None] // 16) == par[..., None, :]).any(-1).all()
+    gpar = ppidx.long().repeat_interleave(16, dim=2)
+    assert ((pidx.long()[..., :, None] // 16) == gpar[..., None, :]).any(-1).all()
+    pooled = [ctx[n] for n in ("pk", "pv", "pk2", "pv2", "pk3", "pv3")]
+    oc, lc = O.closed_form_l3(*[t.double() for t in (q, k, v, *pooled)], idx, pidx, ppidx)
+    assert torch.allclose(o.double(), oc, atol=2e-5) and torch.allclose(ctx["lse"].double(), lc, atol=2e-5)
+    # a wrong weight on the deepest level is far outside that tolerance
+    ow, _ = O.closed_form_l3(*[t.double() for t in (q, k, v, *pooled)], idx, pidx, ppidx, w3=256)
+    assert (ow - oc).abs().max() > 1e-3
+    got = O.attn_bwd_l3(do, q, k, v, *pooled, o, ctx["lse"], idx, pidx, ppidx)
+    want = _autograd_grads(lambda *a: O.closed_form_l3(*a, idx, pidx, ppidx), (q, k, v, *pooled), do)
+    for a, b in zip(got, want):
+        assert (a.double() - b).norm() / b.norm() < 2e-5
+    # whole operator: pooled gradients flow back through three mean pools
+    pool64 = lambda x: x.reshape(B, H, -1, 16, D).mean(3)
+    ql, kl, vl = (t.double().requires_grad_(True) for t in (q, k, v))
+    pk1, pv1 = pool64(kl), pool64(vl)
+    pk2, pv2 = pool64(pk1), pool64(pv1)
+    oc2, _ = O.closed_form_l3(ql, kl, vl, pk1, pv1, pk2, pv2, pool64(pk2), pool64(pv2), idx, pidx, ppidx)
+    wq, wk, wv = torch.autograd.grad(oc2, (ql, kl, vl), do.double())
+    dq, dk, dv, _ = O.llsa_l3_bwd(do, ctx)
+    for a, b in ((dq, wq), (dk, wk), (dv, wv)):
+        assert (a.double() - b).norm() / b.norm() < 2e-5
+
+
 def test_delta_variants():
     g = torch.Generator().manual_seed(11)
     o = torch.randn(1, 1, 8, 64, generator=g).bfloat16()
