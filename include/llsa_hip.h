@@ -155,6 +155,13 @@ typedef struct llsa_attn_fwd_args {
     float* lse;                                /* (B,H,N) out, m + log(l)                          */
     int32_t B, H, N, T, T2, levels;
     float w1, w2;                              /* token_weight, token_weight_2                    */
+    /* levels == 3 (no counterpart in the reference): one more pooled level.  pkr/pvt then hold
+     * N/256 tiles, pk2r/pv2t N/4096 tiles, pidx is (B,H,N/256,T2) as before. */
+    const void* pk3r;                          /* (B,H,N/65536,1024) R tiles of level-3 pooled k  */
+    const void* pv3t;                          /* (B,H,N/65536,1024) T tiles of level-3 pooled v  */
+    const int32_t* ppidx;                      /* (B,H,N/4096,T3) selected level-2 blocks         */
+    int32_t T3;
+    float w3;                                  /* token_weight_3                                  */
 } llsa_attn_fwd_args;
 
 int llsa_attn_fwd(const llsa_attn_fwd_args* a, void* stream);

@@ -31,7 +31,8 @@ class AttnFwdArgs(C.Structure):
                 ("o", c_void_p), ("sob", c_int64), ("soh", c_int64), ("son", c_int64),
                 ("lse", c_void_p),
                 ("B", c_int32), ("H", c_int32), ("N", c_int32), ("T", c_int32), ("T2", c_int32), ("levels", c_int32),
-                ("w1", c_float), ("w2", c_float)]
+                ("w1", c_float), ("w2", c_float),
+                ("pk3r", c_void_p), ("pv3t", c_void_p), ("ppidx", c_void_p), ("T3", c_int32), ("w3", c_float)]
 
 
 def _t3(name):

@@ -39,7 +39,7 @@ class _Layout:
     """Offsets (in elements) of everything the forward produces, inside one bf16 arena and one
     int32 arena; every section is contiguous (B*H, ...) and starts 256-byte aligned."""
 
-    def __init__(self, lib, B, H, N, levels, T, T2, grad):
+    def __init__(self, lib, B, H, N, levels, T, T2, grad, T3=0):
         BH = B * H
         n1, n2 = N // 16, N // 256
         self.n1, self.n2 = n1, n2
@@ -53,13 +53,17 @@ class _Layout:
             o = _align(o + BH * rows_per_bh * width, 128)
             return at
 
-        l2 = levels == 2
+        l2, l3 = levels >= 2, levels == 3
         self.pq, self.pk, self.pv = take(n1, 64), take(n1, 64), take(n1, 64)
         self.pq2, self.pk2, self.pv2 = take(n2, 64, l2), take(n2, 64, l2), take(n2, 64, l2)
         self.qr, self.kr, self.vr, self.vt = take(n1, 1024), take(n1, 1024), take(n1, 1024, grad), take(n1, 1024)
         self.pkr, self.pvr, self.pvt = take(n2, 1024), take(n2, 1024, grad), take(n2, 1024)
         n3 = max(n2 // 16, 1)
         self.pk2r, self.pv2r, self.pv2t = take(n3, 1024, l2), take(n3, 1024, l2 and grad), take(n3, 1024, l2)
+        n4 = max(n3 // 16, 1)
+        self.n3 = n3
+        self.pq3, self.pk3, self.pv3 = take(n3, 64, l3), take(n3, 64, l3), take(n3, 64, l3)
+        self.pk3r, self.pv3r, self.pv3t = take(n4, 1024, l3), take(n4, 1024, l3 and grad), take(n4, 1024, l3)
         self.n_bf16 = o
 
         o = 0
@@ -74,7 +78,7 @@ class _Layout:
 
         self.wl_f = lib.work_list_len(n1, n1, T, CHUNK_FINE)
         self.wl_c = lib.work_list_len(n2, n2, T2, CHUNK_COARSE) if l2 else 0
-        self.idx, self.pidx = take_i(n1 * T), take_i(n2 * T2, l2)
+        self.idx, self.pidx, self.ppidx = take_i(n1 * T), take_i(n2 * T2, l2), take_i(n3 * T3, l3)
         self.off, self.flat, self.work = take_i(n1 + 1, grad), take_i(n1 * T, grad), take_i(self.wl_f, grad)
         self.poff, self.pflat, self.pwork = (take_i(n2 + 1, grad and l2), take_i(n2 * T2, grad and l2),
                                              take_i(self.wl_c, grad and l2))
@@ -92,13 +96,13 @@ class _Layout:
 _layouts = {}
 
 
-def _layout(lib, B, H, N, levels, T, T2, grad):
-    key = (id(lib), B, H, N, levels, T, T2, grad)
+def _layout(lib, B, H, N, levels, T, T2, grad, T3=0):
+    key = (id(lib), B, H, N, levels, T, T2, grad, T3)
     lay = _layouts.get(key)
     if lay is None:
         if len(_layouts) > 64:
             _layouts.clear()
-        lay = _layouts[key] = _Layout(lib, B, H, N, levels, T, T2, grad)
+        lay = _layouts[key] = _Layout(lib, B, H, N, levels, T, T2, grad, T3)
     return lay
 
 
@@ -121,7 +125,7 @@ class LlsaFused(Function):
     qk-norm of the reference's attention processor), inside the pooling pass; they receive gradients."""
 
     @staticmethod
-    def forward(ctx, q, k, v, levels, topk1, topk2, block_size, freq, gamma_q=None, gamma_k=None, eps=1e-5):
+    def forward(ctx, q, k, v, levels, topk1, topk2, block_size, freq, gamma_q=None, gamma_k=None, eps=1e-5, topk3=0):
         lib = current_lib()
         if block_size != 16:
             raise NotImplementedError("block_size must be 16")
@@ -135,12 +139,13 @@ class LlsaFused(Function):
         if k.shape != q.shape or v.shape != q.shape:
             raise ValueError("self-attention only: q, k, v must have the same shape")
         B, H, N, _ = q.shape
-        mult = 1024 if levels == 1 else 16384
+        mult = {1: 1024, 2: 16384, 3: 262144}[levels]
         if N % mult != 0:
             raise ValueError(f"llsa_l{levels} needs a token count that is a multiple of {mult} (got {N})")
-        n1, n2 = N // 16, N // 256
+        n1, n2, n3 = N // 16, N // 256, N // 4096
         T = min(topk1, n1)
-        T2 = min(topk2, n2) if levels == 2 else 0
+        T2 = min(topk2, n2) if levels >= 2 else 0
+        T3 = min(topk3, n3) if levels == 3 else 0
         rope = freq is not None
         if rope:
             if freq.dtype != torch.bfloat16 or tuple(freq.shape) != (N, 64):
@@ -155,7 +160,9 @@ class LlsaFused(Function):
             gk = gamma_k.detach().to(device=q.device, dtype=torch.float32).contiguous()
         if any(g is not None and g.numel() != 64 for g in (gq, gk)):
             raise ValueError("qk-norm weights must have 64 entries")
-        lay = _layout(lib, B, H, N, levels, T, T2, grad)
+        if grad and levels == 3:
+            raise NotImplementedError("llsa_l3: the backward is not built yet")
+        lay = _layout(lib, B, H, N, levels, T, T2, grad, T3)
         dev = q.device
         A = torch.empty(lay.n_bf16, device=dev, dtype=torch.bfloat16)
         I = torch.empty(lay.n_i32, device=dev, dtype=torch.int32)
@@ -165,7 +172,7 @@ class LlsaFused(Function):
         pa = lambda off: None if off is None else a0 + 2 * off
         pi = lambda off: None if off is None else i0 + 4 * off
         stream = _stream(lib, q)
-        l2 = levels == 2
+        l2, l3 = levels >= 2, levels == 3
 
         items = (PoolItem * 3)(
             PoolItem(q.data_ptr(), q.stride(0), q.stride(1), q.stride(2), N, int(rope), pa(lay.pq), pa(lay.pq2), pa(lay.qr),
@@ -177,11 +184,18 @@ class LlsaFused(Function):
         _check(lib, lib.pool_pyramid_fwd(items, 3, freq.data_ptr() if rope else None, B, H, stream), "pool_pyramid")
         if l2:
             s2 = (H * n2 * 64, n2 * 64, 64)
-            items2 = (PoolItem * 2)(
-                PoolItem(pa(lay.pk2), *s2, n2, 0, None, None, pa(lay.pk2r), None, None, None, None),
-                PoolItem(pa(lay.pv2), *s2, n2, 0, None, None, pa(lay.pv2r), pa(lay.pv2t), None, None, None))
-            _check(lib, lib.pool_pyramid_fwd(items2, 2, None, B, H, stream), "pool_pyramid (level-2 tiles)")
-            _check(lib, lib.topk_dense(pa(lay.pq2), pa(lay.pk2), pi(lay.pidx), B, H, n2, T2, 1, stream), "gen_sparse_indices")
+            # the level-2 rows again: their tiles and (three levels) the level-3 rows with theirs
+            items2 = (PoolItem * 3)(
+                PoolItem(pa(lay.pk2), *s2, n2, 0, pa(lay.pk3), None, pa(lay.pk2r), None, pa(lay.pk3r), None, None),
+                PoolItem(pa(lay.pv2), *s2, n2, 0, pa(lay.pv3), None, pa(lay.pv2r), pa(lay.pv2t), pa(lay.pv3r), pa(lay.pv3t), None),
+                PoolItem(pa(lay.pq2), *s2, n2, 0, pa(lay.pq3), None, None, None, None, None, None))
+            _check(lib, lib.pool_pyramid_fwd(items2, 3 if l3 else 2, None, B, H, stream), "pool_pyramid (level-2 tiles)")
+            if l3:
+                _check(lib, lib.topk_dense(pa(lay.pq3), pa(lay.pk3), pi(lay.ppidx), B, H, n3, T3, 1, stream), "gen_sparse_indices")
+                _check(lib, lib.topk_sparse(pa(lay.pq2), pa(lay.pk2), pi(lay.ppidx), pi(lay.pidx), B, H, n2, T2, T3, stream),
+                       "compute_topk_indices_sparse (level 2)")
+            else:
+                _check(lib, lib.topk_dense(pa(lay.pq2), pa(lay.pk2), pi(lay.pidx), B, H, n2, T2, 1, stream), "gen_sparse_indices")
             _check(lib, lib.topk_sparse(pa(lay.pq), pa(lay.pk), pi(lay.pidx), pi(lay.idx), B, H, n1, T, T2, stream),
                    "compute_topk_indices_sparse")
         else:
@@ -209,6 +223,8 @@ class LlsaFused(Function):
         f.lse = lse.data_ptr()
         f.B, f.H, f.N, f.T, f.T2, f.levels = B, H, N, T, T2, levels
         f.w1, f.w2 = 16.0, 256.0
+        if l3:
+            f.pk3r, f.pv3t, f.ppidx, f.T3, f.w3 = pa(lay.pk3r), pa(lay.pv3t), pi(lay.ppidx), T3, 4096.0
         _check(lib, lib.attn_fwd(C.byref(f), stream), "attn_fwd")
 
         if grad:
@@ -231,6 +247,8 @@ class LlsaFused(Function):
             ctx.meta = (lib, lay, B, H, N, T, T2, levels, q.shape, q.stride(), k.stride(), v.stride())
             ctx.eps = float(eps)
             ctx.gamma_dtypes = (None if gamma_q is None else gamma_q.dtype, None if gamma_k is None else gamma_k.dtype)
+        global _last
+        _last = (I, lay, B, H, T, T2, T3, levels)
         return o
 
     @staticmethod
@@ -291,7 +309,19 @@ class LlsaFused(Function):
                     dgq = dg
                 else:
                     dgk = dg
-        return dq, dk, dv, None, None, None, None, None, dgq, dgk, None
+        return dq, dk, dv, None, None, None, None, None, dgq, dgk, None, None
+
+
+_last = None        # int32 arena and layout of the most recent forward (for last_selection)
+
+
+def last_selection():
+    """(indices, p_indices or None, pp_indices or None) of the most recent forward in this process, also
+    one that recorded no backward."""
+    I, lay, B, H, T, T2, T3, levels = _last
+    view = lambda off, rows, t: I[off:off + B * H * rows * t].view(B, H, rows, t)
+    return (view(lay.idx, lay.n1, T), view(lay.pidx, lay.n2, T2) if levels >= 2 else None,
+            view(lay.ppidx, lay.n3, T3) if levels == 3 else None)
 
 
 def selection(out):
@@ -301,5 +331,5 @@ def selection(out):
     I = node.saved_tensors[1]
     _, lay, B, H, N, T, T2, levels = node.meta[:8]
     idx = I[lay.idx:lay.idx + B * H * lay.n1 * T].view(B, H, lay.n1, T)
-    pidx = I[lay.pidx:lay.pidx + B * H * lay.n2 * T2].view(B, H, lay.n2, T2) if levels == 2 else None
+    pidx = I[lay.pidx:lay.pidx + B * H * lay.n2 * T2].view(B, H, lay.n2, T2) if levels >= 2 else None
     return idx, pidx
