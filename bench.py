@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the llsa hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c5|n65536|c4] [--no-extras]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c5|n65536|c4|c5_l3] [--no-extras]
 
 A step is one forward + backward of the operator on one batch of synthetic input that is
 already resident in HBM.  The default workload is the configuration the headline metric is
@@ -50,10 +50,13 @@ WORKLOADS = {
     "c3": ("l2", 2, 6, 16384, 16, 16, True),
     "c5": ("l2", 1, 6, 262144, 16, 16, True),
     "n65536": ("l2", 1, 6, 65536, 16, 16, True),
+    "c5_l3": ("l3", 1, 6, 262144, 16, 16, True),      # three pooled levels (topk 16/16/16), no counterpart in the reference
 }
 
 
 def n_kv(op, N, t1, t2):
+    if op == "l3":
+        return 16 * t1 + 16 * t2 + 16 * t2 + N // 4096
     return 16 * t1 + N // 16 if op == "l1" else 16 * t1 + 16 * t2 + N // 256
 
 
@@ -290,6 +293,8 @@ def main():
         if args.unfused:
             qq, kk = (llsa_amd.my_rope_fn(q_, freq), llsa_amd.my_rope_fn(k_, freq)) if rope else (q_, k_)
             return llsa_amd.llsa_l2_unfused(qq, kk, v_, t1, t2, 16) if op == "l2" else llsa_amd.llsa_l1_unfused(qq, kk, v_, t1, 16)
+        if op == "l3":
+            return llsa_amd.llsa_l3(q_, k_, v_, t1, t2, t2, 16, rope=freq)
         return llsa_amd.llsa_l2(q_, k_, v_, t1, t2, 16, rope=freq) if op == "l2" else llsa_amd.llsa_l1(q_, k_, v_, t1, 16, rope=freq)
 
     def eager_step():
@@ -332,14 +337,14 @@ def main():
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: llsa_{op} fwd+bwd B={B} H={H} N={N} D={D} block_size=16 topk={t1}"
-                               + (f"/{t2}" if op == "l2" else "") + (" rope=in-kernel" if rope else "")
+                               + (f"/{t2}" if op == "l2" else f"/{t2}/{t2}" if op == "l3" else "") + (" rope=in-kernel" if rope else "")
                                + (" (unfused composition)" if args.unfused else ""),
                    "n_kv_per_query": nkv, "algorithmic_gflop": flops / 1e9},
         "frac_of_bf16_mfma_peak": flops / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
         "ms_per_step_graph": ms_graph,
     }
 
-    if not args.no_extras:
+    if not args.no_extras and op != "l3":      # (the stage profile and the CPU baseline know one and two levels)
         prof_iters = max(5, min(args.steps, 20))
         with torch.no_grad():
             st = stage_profile(op, q.detach(), k.detach(), v.detach(), do, t1, t2, freq, prof_iters, torch)

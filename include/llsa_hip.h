@@ -190,6 +190,7 @@ int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, 
 int64_t llsa_work_list_len(int Mb, int Kb, int T, int chunk);
 #define LLSA_CHUNK_FINE 64
 #define LLSA_CHUNK_COARSE 8
+#define LLSA_CHUNK_COARSE2 1
 
 /* ------------------------------------------------------------------------------------------
  * Backward.  Replaces sparse_indices_attn_res_scatter_bwd_v2 (sparse_attention_res_1.py:403-471)
@@ -228,17 +229,25 @@ typedef struct llsa_attn_bwd_args {
                                                     receive the pooled gradients of their blocks, with the
                                                     same bf16 roundings (= llsa_pool_bwd_accum), and dk is
                                                     rotated back with freq_dk                          */
+    /* levels == 3 (no counterpart in the reference): one more pooled level */
+    const void* pk3r; const void* pv3r;          /* R tiles of pk3, pv3 (B,H,N/65536,1024)        */
+    const int32_t* ppidx;                        /* (B,H,N/4096,T3) selected level-2 blocks        */
+    const int32_t* ppoff; const int32_t* ppflat; const int32_t* ppwork;  /* transposed ppidx (Kb = N/4096,
+                                                    chunk = LLSA_CHUNK_COARSE2)                    */
+    void* dpk3; void* dpv3;                      /* (B,H,N/4096,64) contiguous out                 */
+    int32_t T3;
+    float w3;
 } llsa_attn_bwd_args;
 
 #define LLSA_BWD_DQ 2       /* dq; also delta = rowsum(o * dout) and the R tiles of dout, which the
                                stages below read from the workspace                              */
 #define LLSA_BWD_DKV 4      /* dK/dV of the fine tokens                                          */
-#define LLSA_BWD_DPKV1 8    /* sparse level-1 pooled gradients (levels == 2)                     */
+#define LLSA_BWD_DPKV1 8    /* sparse pooled gradients: level 1 (levels >= 2), level 2 (levels == 3) */
 #define LLSA_BWD_DENSE 16   /* dense coarsest pooled gradients (partials + reduction)            */
 #define LLSA_BWD_NO_REDUCE 32 /* with an explicit mask: leave out the reductions of partial sums (results
                                  are then incomplete; for timing the K-side kernels alone)          */
 
-int64_t llsa_attn_bwd_workspace_bytes(int B, int H, int N, int T, int T2, int levels);
+int64_t llsa_attn_bwd_workspace_bytes(int B, int H, int N, int T, int T2, int T3, int levels);
 int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream);
 
 #ifdef __cplusplus

@@ -53,7 +53,9 @@ class AttnBwdArgs(C.Structure):
         + [("dpk", c_void_p), ("dpv", c_void_p), ("dpk2", c_void_p), ("dpv2", c_void_p),
            ("workspace", c_void_p), ("workspace_bytes", c_int64), ("freq_dq", c_void_p), ("freq_dk", c_void_p),
            ("B", c_int32), ("H", c_int32), ("N", c_int32), ("T", c_int32), ("T2", c_int32), ("levels", c_int32),
-           ("w1", c_float), ("w2", c_float), ("cgw1", c_float), ("stages", c_int32), ("fold_pooled", c_int32)])
+           ("w1", c_float), ("w2", c_float), ("cgw1", c_float), ("stages", c_int32), ("fold_pooled", c_int32),
+           ("pk3r", c_void_p), ("pv3r", c_void_p), ("ppidx", c_void_p), ("ppoff", c_void_p), ("ppflat", c_void_p),
+           ("ppwork", c_void_p), ("dpk3", c_void_p), ("dpv3", c_void_p), ("T3", c_int32), ("w3", c_float)])
 
 
 P64 = C.POINTER(c_int64)
@@ -76,12 +78,12 @@ _SIGNATURES = {
     "llsa_attn_fwd": (c_int, [C.POINTER(AttnFwdArgs), c_void_p]),
     "llsa_transpose_indices": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llsa_work_list_len": (c_int64, [c_int, c_int, c_int, c_int]),
-    "llsa_attn_bwd_workspace_bytes": (c_int64, [c_int, c_int, c_int, c_int, c_int, c_int]),
+    "llsa_attn_bwd_workspace_bytes": (c_int64, [c_int, c_int, c_int, c_int, c_int, c_int, c_int]),
     "llsa_attn_bwd": (c_int, [C.POINTER(AttnBwdArgs), c_void_p]),
 }
 
 EXPORTS = tuple(_SIGNATURES)
-CHUNK_FINE, CHUNK_COARSE = 64, 8          # LLSA_CHUNK_FINE / LLSA_CHUNK_COARSE of include/llsa_hip.h
+CHUNK_FINE, CHUNK_COARSE, CHUNK_COARSE2 = 64, 8, 1          # LLSA_CHUNK_* of include/llsa_hip.h
 
 
 class LlsaError(RuntimeError):

@@ -86,7 +86,7 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, floa
     __shared__ __align__(16) bf16 sh[2][kGroup][2 * kTile];   // per block: R tile of K, R tile of V
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int N1 = a.N / kBlk, N2 = N1 / kBlk;
+    const int N1 = a.N / kBlk, N2 = N1 / kBlk, N3 = N2 / kBlk;
     const int lid = xcd_logical_id();
     const int g = (lid % (int)gridDim.x) * 4 + wave;          // < N1: the host checks N1 % 4 == 0
     const int bh = lid / (int)gridDim.x, b = bh / a.H, h = bh % a.H;
@@ -97,17 +97,23 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, floa
     const bf16* vr = (const bf16*)a.vr + (int64_t)bh * N1 * kTile;
     const bf16* pk = (const bf16*)a.pkr + (int64_t)bh * N2 * kTile;
     const bf16* pv = (const bf16*)a.pvr + (int64_t)bh * N2 * kTile;
+    const bf16* pk2 = (a.levels >= 2) ? (const bf16*)a.pk2r + (int64_t)bh * N3 * kTile : nullptr;
+    const bf16* pv2 = (a.levels >= 2) ? (const bf16*)a.pv2r + (int64_t)bh * N3 * kTile : nullptr;
     const int* ip = a.idx + ((int64_t)bh * N1 + g) * a.T;
-    const int* pip = (a.levels == 2) ? a.pidx + ((int64_t)bh * N2 + g / kBlk) * a.T2 : nullptr;
+    const int* pip = (a.levels >= 2) ? a.pidx + ((int64_t)bh * N2 + g / kBlk) * a.T2 : nullptr;
+    const int* ppip = (a.levels == 3) ? a.ppidx + ((int64_t)bh * N3 + g / (kBlk * kBlk)) * a.T3 : nullptr;
 
-    // shared list: (l2) T2 blocks of level-1 pooled tokens, then every block of the coarsest level
-    const int n_mid = (a.levels == 2) ? a.T2 : 0;
-    const int n_dense = (a.levels == 2) ? N2 / kBlk : N1 / kBlk;
-    const int n_groups = (n_mid + n_dense) / kGroup;
-    const int pmine = (a.levels == 2 && lane < a.T2) ? pip[lane] : 0;   // first 64 parent entries, entry i in lane i
-    const bf16* dense_k = (a.levels == 2) ? (const bf16*)a.pk2r + (int64_t)bh * (N2 / kBlk) * kTile : pk;
-    const bf16* dense_v = (a.levels == 2) ? (const bf16*)a.pv2r + (int64_t)bh * (N2 / kBlk) * kTile : pv;
-    const float w_dense = (a.levels == 2) ? a.w2 : a.w1;
+    // shared list: (l2, l3) T2 blocks of level-1 pooled tokens, (l3) T3 blocks of level-2 pooled tokens, then
+    // every block of the coarsest level
+    const int n_mid = (a.levels >= 2) ? a.T2 : 0;
+    const int n_mid2 = (a.levels == 3) ? a.T3 : 0;
+    const int n_dense = (a.levels == 3) ? N3 / kBlk : (a.levels == 2) ? N2 / kBlk : N1 / kBlk;
+    const int n_groups = (n_mid + n_mid2 + n_dense) / kGroup;
+    const int pmine = (a.levels >= 2 && lane < a.T2) ? pip[lane] : 0;   // first 64 parent entries, entry i in lane i
+    const int ppmine = (a.levels == 3 && lane < a.T3) ? ppip[lane] : 0;
+    const bf16* dense_k = (a.levels == 3) ? (const bf16*)a.pk3r + (int64_t)bh * (N3 / kBlk) * kTile : (a.levels == 2) ? pk2 : pk;
+    const bf16* dense_v = (a.levels == 3) ? (const bf16*)a.pv3r + (int64_t)bh * (N3 / kBlk) * kTile : (a.levels == 2) ? pv2 : pv;
+    const float w_dense = (a.levels == 3) ? a.w3 : (a.levels == 2) ? a.w2 : a.w1;
     bf16* const sh0 = &sh[0][0][0];
     auto issue_group = [=](int grp) __attribute__((always_inline)) {   // this wave brings in block kGroup*grp + wave
         const int sblk = kGroup * grp + wave;
@@ -116,8 +122,13 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, floa
             const int blk = clampi(sblk < kWave ? __builtin_amdgcn_readlane(pmine, sblk) : pip[sblk], 0, N2 - 1);
             kb = pk + (int64_t)blk * kTile;
             vb = pv + (int64_t)blk * kTile;
+        } else if (sblk < n_mid + n_mid2) {
+            const int j = sblk - n_mid;
+            const int blk = clampi(j < kWave ? __builtin_amdgcn_readlane(ppmine, j) : ppip[j], 0, N3 - 1);
+            kb = pk2 + (int64_t)blk * kTile;
+            vb = pv2 + (int64_t)blk * kTile;
         } else {
-            const int u = sblk - n_mid;
+            const int u = sblk - n_mid - n_mid2;
             kb = dense_k + (int64_t)u * kTile;
             vb = dense_v + (int64_t)u * kTile;
         }
@@ -168,7 +179,7 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, floa
     for (int grp = 0; grp < n_groups; grp++) {
         wait_vm0();
         __syncthreads();
-        const float w = (kGroup * grp < n_mid) ? a.w1 : w_dense;
+        const float w = (kGroup * grp < n_mid) ? a.w1 : (kGroup * grp < n_mid + n_mid2) ? a.w2 : w_dense;
         const bf16* blk = sh0 + (grp & 1) * kGroup * (2 * kTile);
         PairR r0;
         PairT t0;
@@ -239,7 +250,8 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, floa
 // blocks; the unit's waves walk the list two query blocks at a time.  attn_kside_kernel serves
 // the two list-driven passes, attn_kside_dense_kernel the dense one.
 // ---------------------------------------------------------------------------------------
-enum { MODE_FINE = 0, MODE_SPARSE1 = 1 };       // (the dense coarsest level has a kernel of its own)
+enum { MODE_FINE = 0, MODE_SPARSE1 = 1, MODE_SPARSE2 = 2 };   // (the dense coarsest level has a kernel of its own)
+// SPARSE1: a list entry is a parent and stands for its 16 children; SPARSE2 (three levels): a grand-parent, 256 query blocks
 
 // Optional last step of the fine dK / dV: add the pooled gradients the token's block received
 // (what the backward of the two mean pools and autograd's accumulation do in the reference:
@@ -248,11 +260,17 @@ struct PoolFold {
     const bf16* g1k; const bf16* g1v;             // level-1 pooled gradients (BH, N/16, 64); nullptr: no folding
     const bf16* g2k; const bf16* g2v;             // level-2 pooled gradients (BH, N/256, 64) or nullptr
     const bf16* freq;                             // (N, 64) or nullptr
+    const bf16* g3k; const bf16* g3v;             // level-3 pooled gradients (BH, N/4096, 64) or nullptr
 };
 // x: four channels of one token; g / gg: the same channels of its block's level-1 / level-2 pooled
 // gradient; f: their [sin, cos] entries.  Mirrors pool_bwd_accum_kernel.
-__device__ __forceinline__ bf16x4 fold_math(bf16x4 x, bf16x4 g, bool has_gg, bf16x4 gg, bool has_f, bf16x4 f) {
+__device__ __forceinline__ bf16x4 fold_math(bf16x4 x, bf16x4 g, bool has_gg, bf16x4 gg, bool has_f, bf16x4 f,
+                                            bool has_g3 = false, bf16x4 g3 = bf16x4{}) {
 #pragma clang fp contract(off)
+    if (has_g3) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) gg[e] = (bf16)((float)gg[e] + rn_bf16((float)g3[e] * 0.0625f));
+    }
     if (has_gg) {
 #pragma unroll
         for (int e = 0; e < 4; e++) g[e] = (bf16)((float)g[e] + rn_bf16((float)gg[e] * 0.0625f));
@@ -265,15 +283,17 @@ __device__ __forceinline__ bf16x4 fold_math(bf16x4 x, bf16x4 g, bool has_gg, bf1
 __device__ __forceinline__ bf16x4 fold_pooled(bf16x4 x, const PoolFold& f, int which, int64_t bh, int N, int tok, int c0) {
     const bf16* g1 = which ? f.g1v : f.g1k;
     const bf16* g2 = which ? f.g2v : f.g2k;
+    const bf16* g3 = which ? f.g3v : f.g3k;
     const int N1 = N / kBlk;
     const bf16x4 g = ld8(g1 + (bh * N1 + tok / kBlk) * kD + c0);
-    bf16x4 gg = g, fr = g;
+    bf16x4 gg = g, fr = g, g3v = g;
     if (g2 != nullptr) gg = ld8(g2 + (bh * (N1 / kBlk) + tok / (kBlk * kBlk)) * kD + c0);
+    if (g3 != nullptr) g3v = ld8(g3 + (bh * (N1 / (kBlk * kBlk)) + tok / (kBlk * kBlk * kBlk)) * kD + c0);
     const bool rot = which == 0 && f.freq != nullptr;
     if (rot) fr = ld8(f.freq + (int64_t)tok * kD + c0);
-    return fold_math(x, g, g2 != nullptr, gg, rot, fr);
+    return fold_math(x, g, g2 != nullptr, gg, rot, fr, g3 != nullptr, g3v);
 }
-constexpr int kFoldRows = 4 * kD;                 // LDS copy of a unit's fold operands: 4 pooled rows, then 16 freq rows
+constexpr int kFoldRows = 6 * kD;                 // LDS copy of a unit's fold operands: 6 pooled rows, then 16 freq rows
 constexpr int kFoldElems = kFoldRows + kBlk * kD;
 
 struct KSideParams {
@@ -362,6 +382,7 @@ __device__ __forceinline__ f32x4* part_slot(f32x4* part, int64_t slot) { return 
 template <int MODE>
 __device__ __forceinline__ void kside_item(const KSideParams& p, int bx, int bh, unsigned char* smem_raw, bf16* fold_buf) {
     constexpr int W = (MODE == MODE_FINE) ? 1 : 4;            // waves per work item = waves per workgroup
+    constexpr int kFanShift = (MODE == MODE_SPARSE2) ? 8 : 4;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int N1 = p.N / kBlk;
@@ -385,7 +406,7 @@ __device__ __forceinline__ void kside_item(const KSideParams& p, int bx, int bh,
         cnt = rec[2];
         const int sl = rec[3];
         if (item >= n_items) return;                          // uniform over the item's waves
-        if (MODE == MODE_SPARSE1) cnt *= kBlk;                // every parent stands for its 16 children
+        if (MODE != MODE_FINE) cnt <<= kFanShift;             // every entry stands for its children
         if (sl >= 0) slot = (int64_t)bh * p.slot_stride + sl;
         fl = p.flat + (int64_t)bh * p.flat_stride;
     }
@@ -393,11 +414,14 @@ __device__ __forceinline__ void kside_item(const KSideParams& p, int bx, int bh,
     // is copied into LDS now, without registers, so that no load waits at the end of the wave.
     const bool folding = MODE == MODE_FINE && p.fold.g1k != nullptr && slot < 0;
     if (folding) {
-        const int row = lane >> 3, piece = lane & 7;          // rows: dpk, dpv, dpk2, dpv2 of the unit; 8 x 16 bytes each
-        const bool two = p.fold.g2k != nullptr;
-        if (lane < (two ? 32 : 16)) {
-            const bf16* src = (row & 1) ? ((row & 2) ? p.fold.g2v : p.fold.g1v) : ((row & 2) ? p.fold.g2k : p.fold.g1k);
-            src += ((int64_t)bh * ((row & 2) ? N1 / kBlk : N1) + ((row & 2) ? unit / kBlk : unit)) * kD;
+        const int row = lane >> 3, piece = lane & 7;          // rows: dpk, dpv, dpk2, dpv2, dpk3, dpv3 of the unit; 8 x 16 bytes each
+        const int deep = p.fold.g3k != nullptr ? 3 : p.fold.g2k != nullptr ? 2 : 1;
+        if (lane < 16 * deep) {
+            const int lvl = row >> 1;                         // pooled level 1, 2, 3 -> 0, 1, 2
+            const bf16* src = (row & 1) ? (lvl == 2 ? p.fold.g3v : lvl == 1 ? p.fold.g2v : p.fold.g1v)
+                                        : (lvl == 2 ? p.fold.g3k : lvl == 1 ? p.fold.g2k : p.fold.g1k);
+            const int div = lvl == 2 ? kBlk * kBlk : lvl == 1 ? kBlk : 1;
+            src += ((int64_t)bh * (N1 / div) + unit / div) * kD;
             copy16_global_to_lds(src + piece * 8, fold_buf);
         }
         if (p.fold.freq != nullptr) {
@@ -412,7 +436,7 @@ __device__ __forceinline__ void kside_item(const KSideParams& p, int bx, int bh,
     if (MODE == MODE_FINE) mine = (lane < cnt) ? fl[start + lane] : 0;
     auto entry = [&](int i) -> int {                          // i-th query block of this item (i is wave-uniform)
         if (MODE == MODE_FINE) return clampi(__builtin_amdgcn_readlane(mine, i), 0, N1 - 1);
-        return clampi(fl[start + i / kBlk], 0, N1 / kBlk - 1) * kBlk + (i % kBlk);
+        return (clampi(fl[start + (i >> kFanShift)], 0, (N1 >> kFanShift) - 1) << kFanShift) + (i & ((1 << kFanShift) - 1));
     };
 
     f32x4 dk[4], dv[4];
@@ -459,10 +483,11 @@ __device__ __forceinline__ void kside_item(const KSideParams& p, int bx, int bh,
             bf16x4 ok = cvt4(dk[dt] * kScale), ov = cvt4(dv[dt]);
             if (folding) {
                 const int c0 = dt * 16 + quad * 4;
-                const bool two = p.fold.g2k != nullptr, rot = p.fold.freq != nullptr;
+                const bool two = p.fold.g2k != nullptr, three = p.fold.g3k != nullptr, rot = p.fold.freq != nullptr;
                 ok = fold_math(ok, lds_ld8(fold_buf + c0), two, lds_ld8(fold_buf + 2 * kD + c0), rot,
-                               lds_ld8(fold_buf + kFoldRows + r * kD + c0));
-                ov = fold_math(ov, lds_ld8(fold_buf + kD + c0), two, lds_ld8(fold_buf + 3 * kD + c0), false, ov);
+                               lds_ld8(fold_buf + kFoldRows + r * kD + c0), three, lds_ld8(fold_buf + 4 * kD + c0));
+                ov = fold_math(ov, lds_ld8(fold_buf + kD + c0), two, lds_ld8(fold_buf + 3 * kD + c0), false, ov, three,
+                               lds_ld8(fold_buf + 5 * kD + c0));
             }
             st8(kp + dt * 16, ok);
             st8(vp + dt * 16, ov);
@@ -652,7 +677,7 @@ struct ReduceJob {
     PoolFold fold;           // fine job only
 };
 struct ReduceParams {
-    ReduceJob job[3];
+    ReduceJob job[4];
     int n_jobs, H, N;
 };
 
@@ -738,7 +763,7 @@ struct DensePlan {
 static DensePlan dense_plan(int B, int H, int N, int levels) {
     const int N1 = N / 16;
     DensePlan d;
-    d.n_tok = (levels == 2) ? N1 / 16 : N1;
+    d.n_tok = (levels == 3) ? N1 / 256 : (levels == 2) ? N1 / 16 : N1;
     const int groups = (d.n_tok / 16 / 4) * B * H;            // workgroups per piece of the query range (4 units each)
     int chunks = (512 + groups - 1) / groups;                 // aim at two workgroups per CU
     if (chunks > N1 / 16) chunks = N1 / 16;
@@ -754,23 +779,25 @@ static int64_t align256(int64_t x) { return (x + 255) & ~(int64_t)255; }
 constexpr int64_t kSlotBytes = 8 * kWave * sizeof(f32x4);     // one partial: 16 rows x 64 ch x (dK, dV) fp32
 
 struct BwdWorkspace {
-    int64_t delta, dor, part_fine, part_coarse, part_dense, total;
-    int64_t slots_fine, slots_coarse;                           // per (b,h)
+    int64_t delta, dor, part_fine, part_coarse, part_coarse2, part_dense, total;
+    int64_t slots_fine, slots_coarse, slots_coarse2;            // per (b,h)
 };
 
-static BwdWorkspace bwd_workspace(int B, int H, int N, int T, int T2, int levels) {
-    const int64_t BH = (int64_t)B * H, N1 = N / 16, N2 = N1 / 16;
+static BwdWorkspace bwd_workspace(int B, int H, int N, int T, int T2, int T3, int levels) {
+    const int64_t BH = (int64_t)B * H, N1 = N / 16, N2 = N1 / 16, N3 = N2 / 16;
     const DensePlan d = dense_plan(B, H, N, levels);
     BwdWorkspace w;
     // a key block has several chunks only if it has more than `chunk` entries, so at most
     // E/chunk such blocks with at most E/chunk + E/chunk chunks in total
     w.slots_fine = 2 * (N1 * T / LLSA_CHUNK_FINE) + 2;
-    w.slots_coarse = (levels == 2) ? 2 * (N2 * T2 / LLSA_CHUNK_COARSE) + 2 : 0;
+    w.slots_coarse = (levels >= 2) ? 2 * (N2 * T2 / LLSA_CHUNK_COARSE) + 2 : 0;
+    w.slots_coarse2 = (levels == 3) ? 2 * (N3 * T3 / LLSA_CHUNK_COARSE2) + 2 : 0;
     int64_t o = 0;
     w.delta = o;        o += align256(BH * N * 4);
     w.dor = o;          o += align256(BH * N * 64 * 2);
     w.part_fine = o;    o += align256(BH * w.slots_fine * kSlotBytes);
     w.part_coarse = o;  o += align256(BH * w.slots_coarse * kSlotBytes);
+    w.part_coarse2 = o; o += align256(BH * w.slots_coarse2 * kSlotBytes);
     w.part_dense = o;   o += align256((int64_t)d.chunks * BH * (d.n_tok / 16) * kSlotBytes);
     w.total = o;
     return w;
@@ -780,14 +807,14 @@ static BwdWorkspace bwd_workspace(int B, int H, int N, int T, int T2, int levels
 
 using namespace llsa;
 
-extern "C" int64_t llsa_attn_bwd_workspace_bytes(int B, int H, int N, int T, int T2, int levels) {
-    if (B <= 0 || H <= 0 || N <= 0 || N % 16 != 0 || T <= 0 || (levels != 1 && levels != 2)) return -1;
-    return bwd_workspace(B, H, N, T, T2, levels).total;
+extern "C" int64_t llsa_attn_bwd_workspace_bytes(int B, int H, int N, int T, int T2, int T3, int levels) {
+    if (B <= 0 || H <= 0 || N <= 0 || N % 16 != 0 || T <= 0 || levels < 1 || levels > 3) return -1;
+    return bwd_workspace(B, H, N, T, T2, T3, levels).total;
 }
 
 extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     LLSA_REQUIRE(a != nullptr, "attn_bwd: null args");
-    LLSA_REQUIRE(a->levels == 1 || a->levels == 2, "attn_bwd: levels must be 1 or 2");
+    LLSA_REQUIRE(a->levels >= 1 && a->levels <= 3, "attn_bwd: levels must be 1, 2 or 3");
     LLSA_REQUIRE(a->B > 0 && a->H > 0 && a->N > 0, "attn_bwd: bad B/H/N");
     LLSA_REQUIRE(a->dout && a->o && a->lse && a->qr && a->kr && a->vr && a->pkr && a->pvr && a->idx &&
                      a->off && a->flat && a->dq && a->dk && a->dv && a->dpk && a->dpv && a->workspace,
@@ -797,25 +824,31 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     if (a->levels == 1) {
         LLSA_REQUIRE(a->N % 1024 == 0, "attn_bwd: llsa_l1 needs N %% 1024 == 0 (N=%d)", a->N);
     } else {
-        LLSA_REQUIRE(a->N % 16384 == 0, "attn_bwd: llsa_l2 needs N %% 16384 == 0 (N=%d)", a->N);
+        LLSA_REQUIRE(a->N % (a->levels == 3 ? 262144 : 16384) == 0, "attn_bwd: %d levels need N %% %d == 0 (N=%d)", a->levels,
+                     a->levels == 3 ? 262144 : 16384, a->N);
         LLSA_REQUIRE(a->pk2r && a->pv2r && a->pidx && a->poff && a->pflat && a->dpk2 && a->dpv2, "attn_bwd: level-2 tensors missing");
         LLSA_REQUIRE(a->T2 >= 4 && a->T2 % 4 == 0 && a->T2 <= a->N / 256, "attn_bwd: topk2=%d must be a multiple of 4 and <= N/256", a->T2);
         LLSA_REQUIRE(a->w2 > 0.f, "attn_bwd: token_weight_2 must be > 0");
     }
-    const void* al[] = {a->dout, a->o, a->qr, a->kr, a->vr, a->pkr, a->pvr, a->pk2r, a->pv2r,
-                        a->dq, a->dk, a->dv, a->dpk, a->dpv, a->dpk2, a->dpv2, a->workspace, a->freq_dq, a->lse};
+    if (a->levels == 3) {
+        LLSA_REQUIRE(a->pk3r && a->pv3r && a->ppidx && a->ppoff && a->ppflat && a->ppwork && a->dpk3 && a->dpv3, "attn_bwd: level-3 tensors missing");
+        LLSA_REQUIRE(a->T3 >= 4 && a->T3 % 4 == 0 && a->T3 <= a->N / 4096, "attn_bwd: topk3=%d must be a multiple of 4 and <= N/4096", a->T3);
+        LLSA_REQUIRE(a->w3 > 0.f, "attn_bwd: token_weight_3 must be > 0");
+    }
+    const void* al[] = {a->dout, a->o, a->qr, a->kr, a->vr, a->pkr, a->pvr, a->pk2r, a->pv2r, a->pk3r, a->pv3r,
+                        a->dq, a->dk, a->dv, a->dpk, a->dpv, a->dpk2, a->dpv2, a->dpk3, a->dpv3, a->workspace, a->freq_dq, a->lse};
     for (const void* p : al) LLSA_REQUIRE(aligned16(p), "attn_bwd: tensors must be 16-byte aligned");
     const int64_t st[] = {a->sdob, a->sdoh, a->sdon, a->sob, a->soh, a->son};
     for (int64_t s : st) LLSA_REQUIRE(stride_ok(s), "attn_bwd: input row strides must keep rows 16-byte aligned");
     const int64_t so[] = {a->sdqb, a->sdqh, a->sdqn, a->sdkb, a->sdkh, a->sdkn, a->sdvb, a->sdvh, a->sdvn};
     for (int64_t s : so) LLSA_REQUIRE(s % 4 == 0, "attn_bwd: output row strides must keep rows 8-byte aligned");
-    const BwdWorkspace wsp = bwd_workspace(a->B, a->H, a->N, a->T, a->T2, a->levels);
+    const BwdWorkspace wsp = bwd_workspace(a->B, a->H, a->N, a->T, a->T2, a->T3, a->levels);
     LLSA_REQUIRE(a->workspace_bytes >= wsp.total, "attn_bwd: workspace too small (%lld < %lld)", (long long)a->workspace_bytes,
                  (long long)wsp.total);
     LLSA_REQUIRE(a->work != nullptr && (a->levels == 1 || a->pwork != nullptr), "attn_bwd: work lists missing");
 
     hipStream_t s = (hipStream_t)stream;
-    const int B = a->B, H = a->H, N = a->N, N1 = N / 16, N2 = N1 / 16, BH = B * H;
+    const int B = a->B, H = a->H, N = a->N, N1 = N / 16, N2 = N1 / 16, N3 = N2 / 16, BH = B * H;
     const DensePlan d = dense_plan(B, H, N, a->levels);
     char* ws = (char*)a->workspace;
     float* delta = (float*)(ws + wsp.delta);
@@ -852,9 +885,10 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     base.qr = (const bf16*)a->qr; base.dor = dor;
     base.lse = a->lse; base.delta = delta;
     base.H = H; base.N = N; base.chunk_len = 0;
-    base.fold = PoolFold{nullptr, nullptr, nullptr, nullptr, nullptr};
+    base.fold = PoolFold{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
     const int64_t s1b = (int64_t)H * N1 * 64, s1h = (int64_t)N1 * 64;
     const int64_t s2b = (int64_t)H * N2 * 64, s2h = (int64_t)N2 * 64;
+    const int64_t s3b = (int64_t)H * N3 * 64, s3h = (int64_t)N3 * 64;
 
     auto run_fine = [&]() {                                   // dK / dV of the fine tokens
         if (!(stages & LLSA_BWD_DKV)) return;
@@ -867,14 +901,15 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
         p.dv = (bf16*)a->dv; p.sdvb = a->sdvb; p.sdvh = a->sdvh; p.sdvn = a->sdvn;
         p.n_units = N1; p.w = 1.f;
         if (fold)
-            p.fold = PoolFold{(const bf16*)a->dpk, (const bf16*)a->dpv, (a->levels == 2) ? (const bf16*)a->dpk2 : nullptr,
-                              (a->levels == 2) ? (const bf16*)a->dpv2 : nullptr, (const bf16*)a->freq_dk};
+            p.fold = PoolFold{(const bf16*)a->dpk, (const bf16*)a->dpv, (a->levels >= 2) ? (const bf16*)a->dpk2 : nullptr,
+                              (a->levels >= 2) ? (const bf16*)a->dpv2 : nullptr, (const bf16*)a->freq_dk,
+                              (a->levels == 3) ? (const bf16*)a->dpk3 : nullptr, (a->levels == 3) ? (const bf16*)a->dpv3 : nullptr};
         const int max_items = N1 * a->T / LLSA_CHUNK_FINE + N1;
         hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_FINE>), dim3((max_items + KS_IPW - 1) / KS_IPW, BH), dim3(64), 0, s, p);
         add_job(p, LLSA_CHUNK_FINE, N1 * a->T / LLSA_CHUNK_FINE + 1, 0);
     };
     auto run_sparse1 = [&]() {                                // level-1 pooled tokens, through the transposed coarse index
-        if (a->levels != 2 || !(stages & LLSA_BWD_DPKV1)) return;
+        if (a->levels < 2 || !(stages & LLSA_BWD_DPKV1)) return;
         KSideParams p = base;
         p.kk = (const bf16*)a->pkr; p.vv = (const bf16*)a->pvr;
         p.off = a->poff; p.flat = a->pflat; p.flat_stride = (int64_t)N2 * a->T2;
@@ -887,12 +922,31 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
         hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_SPARSE1>), dim3(max_items, BH), dim3(256), 0, s, p);
         add_job(p, LLSA_CHUNK_COARSE, N2 * a->T2 / LLSA_CHUNK_COARSE + 1, 0);
     };
+    auto run_sparse2 = [&]() {                                // (l3) level-2 pooled tokens, through the transposed level-3 selection:
+        if (a->levels != 3 || !(stages & LLSA_BWD_DPKV1)) return;   // an entry is a grand-parent, 256 query blocks
+        KSideParams p = base;
+        p.kk = (const bf16*)a->pk2r; p.vv = (const bf16*)a->pv2r;
+        p.off = a->ppoff; p.flat = a->ppflat; p.flat_stride = (int64_t)N3 * a->T3;
+        p.work = a->ppwork; p.work_stride = llsa_work_list_len(N3, N3, a->T3, LLSA_CHUNK_COARSE2);
+        p.part = (f32x4*)(ws + wsp.part_coarse2); p.slot_stride = wsp.slots_coarse2;
+        p.dk = (bf16*)a->dpk2; p.sdkb = s2b; p.sdkh = s2h; p.sdkn = 64;
+        p.dv = (bf16*)a->dpv2; p.sdvb = s2b; p.sdvh = s2h; p.sdvn = 64;
+        p.n_units = N3; p.w = a->w2;
+        const int max_items = N3 * a->T3 / LLSA_CHUNK_COARSE2 + N3;
+        hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_SPARSE2>), dim3(max_items, BH), dim3(256), 0, s, p);
+        add_job(p, LLSA_CHUNK_COARSE2, N3 * a->T3 / LLSA_CHUNK_COARSE2 + 1, 0);
+    };
     // dense coarsest level: every unit (16 pooled tokens) meets every query block; the query
     // range is cut into d.chunks pieces whose partial sums are added afterwards
     auto run_dense = [&]() {
         if (!(stages & LLSA_BWD_DENSE)) return;
         KSideParams p = base;
-        if (a->levels == 2) {
+        if (a->levels == 3) {
+            p.kk = (const bf16*)a->pk3r; p.vv = (const bf16*)a->pv3r;
+            p.dk = (bf16*)a->dpk3; p.dv = (bf16*)a->dpv3;
+            p.sdkb = p.sdvb = s3b; p.sdkh = p.sdvh = s3h;
+            p.w = a->w3;
+        } else if (a->levels == 2) {
             p.kk = (const bf16*)a->pk2r; p.vv = (const bf16*)a->pv2r;
             p.dk = (bf16*)a->dpk2; p.dv = (bf16*)a->dpv2;
             p.sdkb = p.sdvb = s2b; p.sdkh = p.sdvh = s2h;
@@ -914,6 +968,7 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     if (fold) {
         // the fine pass adds the finished pooled gradients on its way out, so they come first
         run_sparse1();
+        run_sparse2();
         run_dense();
         run_reduce();
         run_fine();
@@ -921,6 +976,7 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     } else {
         run_fine();
         run_sparse1();
+        run_sparse2();
         run_dense();
         run_reduce();
     }

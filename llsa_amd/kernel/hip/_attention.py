@@ -122,7 +122,7 @@ def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_wei
     mk = lambda t: torch.empty_like(t) if rows_ok8(t) else torch.empty(t.shape, device=t.device, dtype=t.dtype)
     dq, dk, dv = mk(q), mk(k), mk(v)
     dpk, dpv = torch.empty_like(pk, memory_format=torch.contiguous_format), torch.empty_like(pv, memory_format=torch.contiguous_format)
-    ws_bytes = lib.attn_bwd_workspace_bytes(B, H, N, T, T2, levels)
+    ws_bytes = lib.attn_bwd_workspace_bytes(B, H, N, T, T2, 0, levels)
     ws = torch.empty(ws_bytes, device=q.device, dtype=torch.uint8)
     a = AttnBwdArgs()
     a.dout, (a.sdob, a.sdoh, a.sdon) = do.data_ptr(), s3(do)

@@ -21,7 +21,7 @@ import ctypes as C
 import torch
 from torch.autograd import Function
 
-from ..._lib import CHUNK_COARSE, CHUNK_FINE, AttnBwdArgs, AttnFwdArgs, PoolItem, current_lib
+from ..._lib import CHUNK_COARSE, CHUNK_COARSE2, CHUNK_FINE, AttnBwdArgs, AttnFwdArgs, PoolItem, current_lib
 
 _side = {}          # device -> (second stream, two events)
 _SIDE_STREAM_MIN_TOKENS = 1 << 17
@@ -78,18 +78,23 @@ class _Layout:
 
         self.wl_f = lib.work_list_len(n1, n1, T, CHUNK_FINE)
         self.wl_c = lib.work_list_len(n2, n2, T2, CHUNK_COARSE) if l2 else 0
+        self.wl_c2 = lib.work_list_len(n3, n3, T3, CHUNK_COARSE2) if l3 else 0
         self.idx, self.pidx, self.ppidx = take_i(n1 * T), take_i(n2 * T2, l2), take_i(n3 * T3, l3)
         self.off, self.flat, self.work = take_i(n1 + 1, grad), take_i(n1 * T, grad), take_i(self.wl_f, grad)
         self.poff, self.pflat, self.pwork = (take_i(n2 + 1, grad and l2), take_i(n2 * T2, grad and l2),
                                              take_i(self.wl_c, grad and l2))
+        self.ppoff, self.ppflat, self.ppwork = (take_i(n3 + 1, grad and l3), take_i(n3 * T3, grad and l3),
+                                                take_i(self.wl_c2, grad and l3))
         self.n_i32 = o
         # backward arena (bytes): pooled gradients, then the kernels' workspace
-        self.ws_bytes = lib.attn_bwd_workspace_bytes(B, H, N, T, T2, levels)
+        self.ws_bytes = lib.attn_bwd_workspace_bytes(B, H, N, T, T2, T3, levels)
         self.dpk = 0
         self.dpv = _align(BH * n1 * 128, 256)
         self.dpk2 = self.dpv + _align(BH * n1 * 128, 256)
         self.dpv2 = self.dpk2 + _align(BH * n2 * 128, 256)
-        self.ws = self.dpv2 + _align(BH * n2 * 128, 256)
+        self.dpk3 = self.dpv2 + _align(BH * n2 * 128, 256)
+        self.dpv3 = self.dpk3 + _align(BH * n3 * 128, 256)
+        self.ws = self.dpv3 + _align(BH * n3 * 128, 256)
         self.n_bwd = self.ws + self.ws_bytes
 
 
@@ -160,8 +165,6 @@ class LlsaFused(Function):
             gk = gamma_k.detach().to(device=q.device, dtype=torch.float32).contiguous()
         if any(g is not None and g.numel() != 64 for g in (gq, gk)):
             raise ValueError("qk-norm weights must have 64 entries")
-        if grad and levels == 3:
-            raise NotImplementedError("llsa_l3: the backward is not built yet")
         lay = _layout(lib, B, H, N, levels, T, T2, grad, T3)
         dev = q.device
         A = torch.empty(lay.n_bf16, device=dev, dtype=torch.bfloat16)
@@ -237,6 +240,9 @@ class LlsaFused(Function):
             if l2:
                 _check(lib, lib.transpose_indices(pi(lay.pidx), pi(lay.poff), pi(lay.pflat), pi(lay.pwork), B, H, n2, n2, T2,
                                                   CHUNK_COARSE, s_lists), "transpose_indices (coarse)")
+            if l3:
+                _check(lib, lib.transpose_indices(pi(lay.ppidx), pi(lay.ppoff), pi(lay.ppflat), pi(lay.ppwork), B, H, n3, n3, T3,
+                                                  CHUNK_COARSE2, s_lists), "transpose_indices (level 3)")
             if side is not None:
                 ev_lists.record(side)
                 cur.wait_event(ev_lists)
@@ -244,7 +250,7 @@ class LlsaFused(Function):
         if grad:
             # (q and k themselves are needed again only by the backward of the qk-norm)
             ctx.save_for_backward(A, I, o, lse, freq, gq, gk, q if gq is not None else None, k if gk is not None else None)
-            ctx.meta = (lib, lay, B, H, N, T, T2, levels, q.shape, q.stride(), k.stride(), v.stride())
+            ctx.meta = (lib, lay, B, H, N, T, T2, levels, q.shape, q.stride(), k.stride(), v.stride(), T3)
             ctx.eps = float(eps)
             ctx.gamma_dtypes = (None if gamma_q is None else gamma_q.dtype, None if gamma_k is None else gamma_k.dtype)
         global _last
@@ -254,7 +260,7 @@ class LlsaFused(Function):
     @staticmethod
     def backward(ctx, do):
         A, I, o, lse, freq, gq, gk, q_in, k_in = ctx.saved_tensors
-        lib, lay, B, H, N, T, T2, levels, shape, sq, sk, sv = ctx.meta
+        lib, lay, B, H, N, T, T2, levels, shape, sq, sk, sv, T3 = ctx.meta
         dev = o.device
         if not _rows_ok(do):
             do = do.contiguous()
@@ -282,15 +288,19 @@ class LlsaFused(Function):
         a.dk, a.sdkb, a.sdkh, a.sdkn = dk.data_ptr(), dk.stride(0), dk.stride(1), dk.stride(2)
         a.dv, a.sdvb, a.sdvh, a.sdvn = dv.data_ptr(), dv.stride(0), dv.stride(1), dv.stride(2)
         a.dpk, a.dpv = w0 + lay.dpk, w0 + lay.dpv
-        if levels == 2:
+        if levels >= 2:
             a.dpk2, a.dpv2 = w0 + lay.dpk2, w0 + lay.dpv2
+        if levels == 3:
+            a.pk3r, a.pv3r, a.ppidx = pa(lay.pk3r), pa(lay.pv3r), pi(lay.ppidx)
+            a.ppoff, a.ppflat, a.ppwork = pi(lay.ppoff), pi(lay.ppflat), pi(lay.ppwork)
+            a.dpk3, a.dpv3, a.T3, a.w3 = w0 + lay.dpk3, w0 + lay.dpv3, T3, 4096.0
         a.workspace, a.workspace_bytes = w0 + lay.ws, lay.ws_bytes
         if freq is not None:
             a.freq_dq = a.freq_dk = freq.data_ptr()
         a.B, a.H, a.N, a.T, a.T2, a.levels = B, H, N, T, T2, levels
         # llsa_l1 keeps the reference's quirk: its pooled path is differentiated with weight 1
         # (sparse_attention_res_1.py:388-389) although the forward uses token_weight
-        a.w1, a.w2, a.cgw1 = 16.0, 256.0, (16.0 if levels == 2 else 1.0)
+        a.w1, a.w2, a.cgw1 = 16.0, 256.0, (16.0 if levels >= 2 else 1.0)
         a.stages, a.fold_pooled = 0, 1
         stream = _stream(lib, o)
         _check(lib, lib.attn_bwd(C.byref(a), stream), "attn_bwd")
@@ -332,4 +342,7 @@ def selection(out):
     _, lay, B, H, N, T, T2, levels = node.meta[:8]
     idx = I[lay.idx:lay.idx + B * H * lay.n1 * T].view(B, H, lay.n1, T)
     pidx = I[lay.pidx:lay.pidx + B * H * lay.n2 * T2].view(B, H, lay.n2, T2) if levels >= 2 else None
+    if levels == 3:
+        T3 = node.meta[12]
+        return idx, pidx, I[lay.ppidx:lay.ppidx + B * H * lay.n3 * T3].view(B, H, lay.n3, T3)
     return idx, pidx

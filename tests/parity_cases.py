@@ -464,3 +464,45 @@ def check_op_l2(dev, B=1, H=1, N=16384, T=8, T2=4, fused=True, rope=False, smoot
     close("dq", dq, rq)
     close("dk", dk, rk)
     close("dv", dv, rv)
+
+
+def check_op_l3(dev, B=1, H=1, N=262144, T=16, T2=16, T3=16, rope=True, qk_norm=False):
+    """llsa_l3 through autograd against the oracle's three-level composition fed with the device's own
+    selection; the selection itself must be a legal cascade (every block under a block its parent chose) and,
+    on these smooth inputs, equal to the oracle's at the two coarse levels wherever the bf16 scores do not tie."""
+    import llsa_amd
+    from llsa_amd.kernel.torch_op._fused import selection
+    from llsa_amd.utils.rope_table import rope_table
+    q, k, v, do = smooth_inputs(B, H, N, 64, dev)
+    freq = rope_table(int(math.isqrt(N)), dtype=torch.bfloat16).to(dev) if rope else None
+    norm = _norm_weights(dev) if qk_norm else None
+    captured = {}
+
+    def run(q_, k_, v_):
+        out = llsa_amd.llsa_l3(q_, k_, v_, T, T2, T3, 16, rope=freq, qk_norm=norm)
+        captured["sel"] = [t.cpu().long() for t in selection(out)]
+        return out
+
+    o, dq, dk, dv = _grads(run, q, k, v, do)
+    idx, pidx, ppidx = captured["sel"]
+    assert idx.shape == (B, H, N // 16, T) and pidx.shape == (B, H, N // 256, T2) and ppidx.shape == (B, H, N // 4096, T3)
+    par = pidx.repeat_interleave(16, dim=2)
+    assert ((idx[..., :, None] // 16) == par[..., None, :]).any(-1).all(), "a fine block outside its parent's selection"
+    gpar = ppidx.repeat_interleave(16, dim=2)
+    assert ((pidx[..., :, None] // 16) == gpar[..., None, :]).any(-1).all(), "a level-1 block outside its grand-parent's selection"
+    qc, kc, vc, doc = (t.cpu() for t in (q, k, v, do))
+    fc = freq.cpu() if rope else None
+    qn, kn = _apply_norm(qc, kc, norm)
+    qr, kr = (O.rope_apply(qn, fc), O.rope_apply(kn, fc)) if rope else (qn, kn)
+    ro, ctx = O.llsa_l3_fwd(qr, kr, vc, T, T2, T3, 16, indices=idx, p_indices=pidx, pp_indices=ppidx)
+    rq, rk, rv, _ = O.llsa_l3_bwd(doc, ctx)
+    if rope:
+        rq, rk = O.rope_apply_bwd(rq, fc), O.rope_apply_bwd(rk, fc)
+    rq, rk = _norm_backward(rq, rk, qc, kc, norm)
+    close("o", o, ro)
+    close("dq", dq, rq)
+    close("dk", dk, rk)
+    close("dv", dv, rv)
+    _, own = O.llsa_l3_fwd(qr, kr, vc, T, T2, T3, 16)
+    same = lambda a, b: (a.sort(-1).values == b.long().sort(-1).values).all(-1).float().mean().item()
+    assert same(ppidx, own["pp_indices"]) > 0.9 and same(pidx, own["p_indices"]) > 0.9 and same(idx, own["indices"]) > 0.9

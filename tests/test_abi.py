@@ -65,8 +65,9 @@ def test_entry_points_reject_bad_arguments(lib):
     a.N, a.T = 1024, 6
     assert lib.attn_fwd(C.byref(a), None) != 0
     assert b"multiple of 4" in lib.last_error_string()
-    assert lib.attn_bwd_workspace_bytes(2, 6, 16384, 16, 16, 2) > 0
-    assert lib.attn_bwd_workspace_bytes(2, 6, 16384, 16, 16, 3) < 0
+    assert lib.attn_bwd_workspace_bytes(2, 6, 16384, 16, 16, 0, 2) > 0
+    assert lib.attn_bwd_workspace_bytes(1, 1, 262144, 16, 16, 16, 3) > lib.attn_bwd_workspace_bytes(1, 1, 262144, 16, 16, 0, 2) > 0
+    assert lib.attn_bwd_workspace_bytes(2, 6, 16384, 16, 16, 0, 4) < 0
     assert lib.work_list_len(1024, 1024, 16, 32) == 4 + 4 * (512 + 1024) + 4 * 513 + 1024
 
 

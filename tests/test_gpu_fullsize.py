@@ -53,6 +53,13 @@ def test_c3_full_size_against_oracle(dev):
     P.check_op_l2(dev, B=2, H=6, N=16384, T=16, T2=16, fused=True, rope=True, smooth=True)
 
 
+@pytest.mark.parametrize("H,T,T2,T3,rope,qk_norm", [(1, 16, 16, 16, True, False), (2, 8, 4, 8, False, True)])
+def test_three_levels_against_oracle(dev, H, T, T2, T3, rope, qk_norm):
+    """llsa_l3 (no counterpart in the reference) at its smallest size, N = 262144, against the oracle's
+    three-level composition."""
+    P.check_op_l3(dev, B=1, H=H, N=262144, T=T, T2=T2, T3=T3, rope=rope, qk_norm=qk_norm)
+
+
 def _rel(a, b):
     return ((a.double() - b.double()).norm() / b.double().norm().clamp_min(1e-30)).item()
 
