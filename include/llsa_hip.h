@@ -199,7 +199,9 @@ int64_t llsa_work_list_len(int Mb, int Kb, int T, int chunk);
  * and the dense coarsest pooled gradients.  The k*scale temporaries of the reference
  * (:420-422) do not exist here.  cgw1 is the factor used on the dpk/dpv path of the level-1
  * pooled tokens: the reference uses 1 for l1 (sparse_attention_res_1.py:388-389) and w1 for
- * l2 (sparse_attention_res_2.py:564).
+ * l2 (sparse_attention_res_2.py:564).  With levels == 3 (no counterpart in the reference) the
+ * level-2 pooled gradients come from a second list-driven pass over the transposed ppidx, the
+ * dense pass runs on level 3, and fold_pooled chains three pool backwards.
  * ---------------------------------------------------------------------------------------- */
 typedef struct llsa_attn_bwd_args {
     const void* dout; int64_t sdob, sdoh, sdon;  /* (B,H,N,64) upstream gradient                 */

@@ -35,6 +35,8 @@ Pinning status (what each function is checked against, see tests/test_oracle_*):
                          (sparse_attention_res_1.py:173); which reduction tree
                          Triton uses is not observable here: parity unpinned for
                          `delta_in_dtype=True`; the default keeps fp32.
+  *_l3                   three levels, no counterpart in the reference: fp64 closed form over the four
+                         weighted segments and torch.autograd on it, selection cascade property
   rms_norm / _bwd        F.rms_norm and its autograd (fp32).  The module the model
                          calls (diffusers' RMSNorm, rope_dit_transformer_2d.py:215-218)
                          is not in the reference checkout: parity unpinned for its
