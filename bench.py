@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the llsa hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c5|n65536|c4|c5_l3] [--no-extras]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c2|c5|n65536|c4|c5_l3|fwd_sweep] [--no-extras]
 
 A step is one forward + backward of the operator on one batch of synthetic input that is
 already resident in HBM.  The default workload is the configuration the headline metric is
@@ -254,12 +254,56 @@ def bench_dit(args):
     }))
 
 
+def bench_fwd_sweep(args):
+    """The reference's own harness restated (test_kernel.py:27-58): forward only, B=2, H=4, D=64, bf16 N(0,1)
+    inputs, default topk 8, N = 128^2, 256^2, 512^2; median and 20 % / 80 % quantiles of the time of one call,
+    the L2 flushed before every call as triton.testing.do_bench does.  llsa_l3 is added where N allows it."""
+    import torch
+    import llsa_amd
+    from llsa_amd._lib import get_lib
+    get_lib()
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    dev = torch.device("cuda:0")
+    B, H, D, topk = 2, 4, 64, 8
+    flush = torch.empty(256 << 20, dtype=torch.int8, device=dev)
+    rows = []
+    for size in (128, 256, 512):
+        N = size * size
+        g = torch.Generator().manual_seed(size)
+        q, k, v = (torch.randn(B, H, N, D, generator=g).bfloat16().to(dev) for _ in range(3))
+        ops = {"l1": lambda: llsa_amd.llsa_l1(q, k, v, topk, 16), "l2": lambda: llsa_amd.llsa_l2(q, k, v, topk, topk, 16)}
+        if N % 262144 == 0:
+            ops["l3"] = lambda: llsa_amd.llsa_l3(q, k, v, topk, topk, topk, 16)
+        for name, fn in ops.items():
+            with torch.no_grad():
+                for _ in range(max(3, args.warmup)):
+                    fn()
+                times = []
+                for _ in range(max(10, args.steps)):
+                    flush.zero_()
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    fn()
+                    e1.record()
+                    e1.synchronize()
+                    times.append(e0.elapsed_time(e1))
+            t = torch.tensor(times)
+            rows.append({"op": "llsa_" + name, "size": size, "N": N, "ms_median": t.median().item(),
+                         "ms_p20": t.quantile(0.2).item(), "ms_p80": t.quantile(0.8).item()})
+    print(json.dumps({
+        "metric": "forward-only time of one call, the reference's test_kernel.py harness", "unit": "ms", "n_gpus": 1,
+        "steps": max(10, args.steps), "warmup": max(3, args.warmup), "higher_is_better": False, "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"fwd_sweep: B={B} H={H} D={D} topk={topk} block_size=16, N(0,1) inputs, no RoPE, L2 flushed before every call"},
+        "value": next(r["ms_median"] for r in rows if r["op"] == "llsa_l2" and r["size"] == 128), "rows": rows}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c4"])
+    ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c4", "fwd_sweep"])
     ap.add_argument("--no-extras", action="store_true", help="skip stage profile, CPU baseline and dense SDPA")
     ap.add_argument("--unfused", action="store_true", help="use the reference's composition (separate pools, autograd adds)")
     ap.add_argument("--graph", action="store_true",
@@ -275,6 +319,8 @@ def main():
         sys.exit(2)
     if args.workload == "c4":
         return bench_dit(args)
+    if args.workload == "fwd_sweep":
+        return bench_fwd_sweep(args)
 
     import torch
     import llsa_amd
