@@ -67,6 +67,8 @@ def test_topk_dense(dev):
     P.check_topk_dense(dev, B=2, H=3, n=256, T=16, round_scores=True)
     P.check_topk_dense(dev, B=1, H=2, n=64, T=16, round_scores=False, min_safe=0.9)
     P.check_topk_dense(dev, B=1, H=2, n=1024, T=16, round_scores=False, min_safe=0.9)
+    P.check_topk_dense(dev, B=1, H=2, n=2048, T=16, round_scores=False, min_safe=0.9)     # rows longer than the radix kernel keeps: chunked arg-max
+    P.check_topk_dense(dev, B=1, H=1, n=4096, T=8, round_scores=True)
     P.check_topk_dense_ties(dev)
 
 
@@ -129,7 +131,7 @@ def test_op_l2(dev, fused, rope):
 
 
 @pytest.mark.parametrize("B,H,N,T", [(1, 1, 1024, 4), (3, 1, 3072, 12), (1, 5, 5120, 16), (2, 3, 2048, 32), (1, 2, 7168, 64),
-                                     (1, 7, 1024, 64)])
+                                     (1, 7, 1024, 64), (1, 1, 32768, 16)])
 def test_op_l1_shapes(dev, B, H, N, T):
     """Token counts that are not powers of two (any multiple of 1024), odd batch and head counts, every
     topk the kernels take (multiples of 4 up to N/16)."""
