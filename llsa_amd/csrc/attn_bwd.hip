@@ -376,9 +376,6 @@ __device__ __forceinline__ void kside_pair(f32x4 dk[4], f32x4 dv[4], const bf16x
 // accumulator layout: 8 f32x4 registers per lane (4 channel tiles of dK, then 4 of dV).
 __device__ __forceinline__ f32x4* part_slot(f32x4* part, int64_t slot) { return part + slot * (8 * kWave); }
 
-#ifndef KS_IPW
-#define KS_IPW 1
-#endif
 template <int MODE>
 __device__ __forceinline__ void kside_item(const KSideParams& p, int bx, int bh, unsigned char* smem_raw, bf16* fold_buf) {
     constexpr int W = (MODE == MODE_FINE) ? 1 : 4;            // waves per work item = waves per workgroup
@@ -535,15 +532,7 @@ __global__ __launch_bounds__(MODE == MODE_FINE ? 64 : 256) void attn_kside_kerne
     const int lid = xcd_logical_id();
     const int bx = lid % (int)gridDim.x;
     const int bh = lid / (int)gridDim.x;
-    if (MODE == MODE_FINE) {
-        for (int rep = 0; rep < KS_IPW; rep++) {
-            kside_item<MODE>(p, bx * KS_IPW + rep, bh, smem_raw, fold_buf);
-            __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-        }
-    } else {
-        kside_item<MODE>(p, bx, bh, smem_raw, fold_buf);
-    }
+    kside_item<MODE>(p, bx, bh, smem_raw, fold_buf);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -905,7 +894,7 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
                               (a->levels >= 2) ? (const bf16*)a->dpv2 : nullptr, (const bf16*)a->freq_dk,
                               (a->levels == 3) ? (const bf16*)a->dpk3 : nullptr, (a->levels == 3) ? (const bf16*)a->dpv3 : nullptr};
         const int max_items = N1 * a->T / LLSA_CHUNK_FINE + N1;
-        hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_FINE>), dim3((max_items + KS_IPW - 1) / KS_IPW, BH), dim3(64), 0, s, p);
+        hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_FINE>), dim3(max_items, BH), dim3(64), 0, s, p);
         add_job(p, LLSA_CHUNK_FINE, N1 * a->T / LLSA_CHUNK_FINE + 1, 0);
     };
     auto run_sparse1 = [&]() {                                // level-1 pooled tokens, through the transposed coarse index
