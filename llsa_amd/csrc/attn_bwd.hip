@@ -670,8 +670,15 @@ struct ReduceParams {
     int n_jobs, H, N;
 };
 
-constexpr int kReduceSlots = 256;    // unit positions per job and (b,h) that are walked in parallel
-__host__ __device__ inline int reduce_slots(int max_units) { return max_units < kReduceSlots ? max_units : kReduceSlots; }
+// Unit positions per job and (b,h) that are walked in parallel: a quarter of the most units the job can have,
+// between 32 and 256.  Usually a few per cent of the units have several pieces, and every position beyond
+// them is a pair of workgroups that starts, reads one record and leaves (at 256 positions for a job of at
+// most 257 units that cost 4 us per launch).
+__host__ __device__ inline int reduce_slots(int max_units) {
+    if (max_units <= 32) return max_units;
+    const int q = max_units / 4;
+    return q < 32 ? 32 : (q > 256 ? 256 : q);
+}
 
 __global__ __launch_bounds__(256) void kside_reduce_kernel(ReduceParams rp) {
     // Two workgroups per unit; every thread owns one f32x4 of the unit's 8 x 64 accumulator
