@@ -40,8 +40,8 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 # WRITE_SIZE on this command, each scaled by what the same counter reads for a 256 MiB elementwise
 # copy (fetch x2.000, write x1.000); the tables they come from are profiles/step_kernels_<workload>_hbm_traffic.txt
 MEASURED_TRAFFIC = {
-    "c3": {"attn_fwd": 130031637, "bwd_dq": 249947726, "bwd_dkv": 295409617, "bwd_dpkv1_sparse": 192022090,
-           "bwd_dpkv_dense": 69261445, "pool_pyramid": 95573732},
+    "c3": {"attn_fwd": 129689497, "bwd_dq": 249972361, "bwd_dkv": 302121348, "bwd_dpkv1_sparse": 190617560,
+           "bwd_dpkv_dense": 69261766, "pool_pyramid": 95573151},
 }
 
 WORKLOADS = {
