@@ -102,7 +102,7 @@ _layouts = {}
 
 
 def _layout(lib, B, H, N, levels, T, T2, grad, T3=0):
-    key = (id(lib), B, H, N, levels, T, T2, grad, T3)
+    key = (lib.path, B, H, N, levels, T, T2, grad, T3)
     lay = _layouts.get(key)
     if lay is None:
         if len(_layouts) > 64:
