@@ -25,7 +25,7 @@ from ..kernel.hip.permute import permute_tokens
 from ..kernel.hip.rms_norm import my_rms_norm_fn
 from ..kernel.hip.rope import my_rope_fn
 from ..kernel.torch_op.flash_sparse_attention_res_1 import llsa_l1
-from ..kernel.torch_op.flash_sparse_attention_res_2 import llsa_l2
+from ..kernel.torch_op.flash_sparse_attention_res_2 import llsa_l2, llsa_l3
 from ..utils.rope_table import rope_table
 from ..utils.zorder import zorder_perm
 
@@ -101,10 +101,13 @@ class LlsaSelfAttention(nn.Module):
                 q, k = my_rms_norm_fn(q, norm[0], self.eps), my_rms_norm_fn(k, norm[1], self.eps)
             q, k = my_rope_fn(q, freq), my_rope_fn(k, freq)
             norm = rope = None
+        tk = self.sparse_topk                                   # coarsest level first, fine blocks last
         if self.levels == 1:
-            o = llsa_l1(q, k, v, self.sparse_topk[1], self.block_size, rope=rope, qk_norm=norm)
-        else:       # the reference passes (sparse_topk[1], sparse_topk[0]) as (topk1, topk2), :249-250
-            o = llsa_l2(q, k, v, self.sparse_topk[1], self.sparse_topk[0], self.block_size, rope=rope, qk_norm=norm)
+            o = llsa_l1(q, k, v, tk[-1], self.block_size, rope=rope, qk_norm=norm)
+        elif self.levels == 2:      # the reference passes (sparse_topk[1], sparse_topk[0]) as (topk1, topk2), :249-250
+            o = llsa_l2(q, k, v, tk[-1], tk[-2], self.block_size, rope=rope, qk_norm=norm)
+        else:                       # three levels: no counterpart in the reference
+            o = llsa_l3(q, k, v, tk[-1], tk[-2], tk[-3], self.block_size, rope=rope, qk_norm=norm)
         return self.to_out(o.transpose(1, 2).reshape(B, N, self.heads * self.head_dim))
 
 
@@ -136,7 +139,7 @@ class PixelDiT(nn.Module):
         super().__init__()
         dim = num_attention_heads * attention_head_dim
         if isinstance(sparse_topk, int):
-            sparse_topk = (sparse_topk, sparse_topk)
+            sparse_topk = (sparse_topk,) * max(levels, 2)
         self.sample_size, self.out_channels = sample_size, out_channels
         self.proj_in = nn.Conv2d(in_channels, dim, kernel_size=1)
         self.transformer_blocks = nn.ModuleList(
