@@ -105,6 +105,22 @@ int llsa_rmsnorm_bwd(const void* dy, const int64_t* sdy /*3*/, const void* x, co
                      float eps, void* dx, const int64_t* sdx /*3*/, float* dgamma, float* partials,
                      int B, int H, int N, void* stream);
 
+/* The same backward with the partial sums in a static device array inside the library instead of a
+ * caller-owned buffer.  It has no counterpart in the reference; it is for callers that cannot
+ * allocate device memory: a step that is being captured into a HIP graph, a tight serving loop,
+ * a harness that forbids hipMalloc.  Limits and rules:
+ *   - B * H * ceil(N / 256) * 64 <= LLSA_STATIC_PARTIALS_MAX (1 MiB of fp32), else the call is
+ *     rejected with an error that names the limit;
+ *   - the first call on a device looks up the array's address there (no allocation, but do it
+ *     once outside a graph capture); the device of `stream` must be the current device;
+ *   - every call on one GPU uses the same array: calls that overlap on one GPU (two streams,
+ *     two threads) race on it.  Calls on one stream are ordered and safe.
+ * Results are bit-identical to llsa_rmsnorm_bwd's. */
+#define LLSA_STATIC_PARTIALS_MAX 262144
+int llsa_rmsnorm_bwd_static(const void* dy, const int64_t* sdy /*3*/, const void* x, const int64_t* sx /*3*/, const float* gamma,
+                            float eps, void* dx, const int64_t* sdx /*3*/, float* dgamma,
+                            int B, int H, int N, void* stream);
+
 /* Token permutation at the model's entry and exit (models/rope_dit_transformer_2d.py:963-965,
  * 1028-1030: hidden_states[:, fwd_perm, :] and hidden_states[:, bwd_perm, :]), and the one after
  * the REPA pooling (:1020).  y[b, i, :] = x[b, index[i], :] for b < B, i < n_out; rows are

@@ -70,6 +70,8 @@ _SIGNATURES = {
     "llsa_rmsnorm_bwd_partials": (c_int64, [c_int, c_int, c_int]),
     "llsa_rmsnorm_bwd": (c_int, [c_void_p, P64, c_void_p, P64, c_void_p, c_float, c_void_p, P64, c_void_p, c_void_p,
                                  c_int, c_int, c_int, c_void_p]),
+    "llsa_rmsnorm_bwd_static": (c_int, [c_void_p, P64, c_void_p, P64, c_void_p, c_float, c_void_p, P64, c_void_p,
+                                        c_int, c_int, c_int, c_void_p]),
     "llsa_gather_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int64, c_int64, c_void_p]),
     "llsa_rope_fwd": (c_int, [c_void_p, P64, c_void_p, c_void_p, P64, c_int, c_int, c_int, c_void_p]),
     "llsa_rope_bwd": (c_int, [c_void_p, P64, c_void_p, c_void_p, P64, c_int, c_int, c_int, c_void_p]),
@@ -84,6 +86,7 @@ _SIGNATURES = {
 
 EXPORTS = tuple(_SIGNATURES)
 CHUNK_FINE, CHUNK_COARSE, CHUNK_COARSE2 = 64, 8, 1          # LLSA_CHUNK_* of include/llsa_hip.h
+STATIC_PARTIALS_MAX = 262144                                # LLSA_STATIC_PARTIALS_MAX
 
 
 class LlsaError(RuntimeError):

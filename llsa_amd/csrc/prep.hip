@@ -4,6 +4,7 @@
 #include "llsa_device.h"
 #include "llsa_host.h"
 #include "../../include/llsa_hip.h"
+#include <mutex>
 
 namespace llsa {
 
@@ -496,8 +497,8 @@ extern "C" int64_t llsa_rmsnorm_bwd_partials(int B, int H, int N) {
     return (int64_t)B * H * ((N + kNormTokens - 1) / kNormTokens) * kD;
 }
 
-extern "C" int llsa_rmsnorm_bwd(const void* dy, const int64_t* sdy, const void* x, const int64_t* sx, const float* gamma, float eps,
-                                void* dx, const int64_t* sdx, float* dgamma, float* partials, int B, int H, int N, void* stream) {
+static int rmsnorm_bwd_launch(const void* dy, const int64_t* sdy, const void* x, const int64_t* sx, const float* gamma, float eps,
+                              void* dx, const int64_t* sdx, float* dgamma, float* partials, int B, int H, int N, void* stream) {
     LLSA_REQUIRE(dy && x && gamma && dx && dgamma && partials && sdy && sx && sdx, "rmsnorm_bwd: null argument");
     LLSA_REQUIRE(B > 0 && H > 0 && N > 0 && eps >= 0.f, "rmsnorm_bwd: bad shape or eps");
     LLSA_REQUIRE(aligned16(dy) && aligned16(x) && aligned16(dx) && s3_ok(sdy) && s3_ok(sx) && s3_ok(sdx),
@@ -514,4 +515,52 @@ extern "C" int llsa_rmsnorm_bwd(const void* dy, const int64_t* sdy, const void* 
     }
     hipLaunchKernelGGL(rmsnorm_dgamma_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, (const float*)partials, dgamma, rows);
     return launch_status("rmsnorm_bwd");
+}
+
+extern "C" int llsa_rmsnorm_bwd(const void* dy, const int64_t* sdy, const void* x, const int64_t* sx, const float* gamma, float eps,
+                                void* dx, const int64_t* sdx, float* dgamma, float* partials, int B, int H, int N, void* stream) {
+    return rmsnorm_bwd_launch(dy, sdy, x, sx, gamma, eps, dx, sdx, dgamma, partials, B, H, N, stream);
+}
+
+// ---------------------------------------------------------------------------------------
+// The same backward for callers that cannot allocate (a step under HIP graph capture, a tight
+// serving loop): the per-workgroup partial sums of dgamma live in a static device array instead
+// of a buffer the caller brings.  Every GPU holds its own copy of the array at its own address;
+// the address is looked up once per device, with that device current, and the kernels receive
+// it as an ordinary pointer argument.
+// ---------------------------------------------------------------------------------------
+static __device__ __align__(256) float scratch[LLSA_STATIC_PARTIALS_MAX];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+float* g_scratch_ptr[kMaxDevices];       // device address of `scratch` per device ordinal, looked up on first use
+}  // namespace
+
+extern "C" int llsa_rmsnorm_bwd_static(const void* dy, const int64_t* sdy, const void* x, const int64_t* sx, const float* gamma,
+                                       float eps, void* dx, const int64_t* sdx, float* dgamma, int B, int H, int N, void* stream) {
+    const int64_t need = llsa_rmsnorm_bwd_partials(B, H, N);
+    LLSA_REQUIRE(need > 0, "rmsnorm_bwd_static: bad shape");
+    LLSA_REQUIRE(need <= (int64_t)LLSA_STATIC_PARTIALS_MAX,
+                 "rmsnorm_bwd_static: B*H*ceil(N/256)*64 = %lld partial sums exceed the static scratch of %lld floats; "
+                 "use llsa_rmsnorm_bwd with a caller-owned buffer",
+                 (long long)need, (long long)LLSA_STATIC_PARTIALS_MAX);
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(-102, "rmsnorm_bwd_static: hipGetDevice: %s", hipGetErrorString(e));
+    LLSA_REQUIRE(dev >= 0 && dev < kMaxDevices, "rmsnorm_bwd_static: device ordinal %d out of range", dev);
+    float* part = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (g_scratch_ptr[dev] == nullptr) {
+            void* p = nullptr;
+            e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+            if (e != hipSuccess || p == nullptr)
+                return fail(-103, "rmsnorm_bwd_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+            g_scratch_ptr[dev] = (float*)p;
+        }
+        part = g_scratch_ptr[dev];
+    }
+    // every row of the partial sums this call reads is written by its first kernel, so nothing has to be cleared
+    return rmsnorm_bwd_launch(dy, sdy, x, sx, gamma, eps, dx, sdx, dgamma, part, B, H, N, stream);
 }

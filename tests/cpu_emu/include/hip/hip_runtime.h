@@ -37,6 +37,10 @@ typedef int hipError_t;
 inline hipError_t hipGetLastError() { return hipSuccess; }
 inline hipError_t hipPeekAtLastError() { return hipSuccess; }
 inline const char* hipGetErrorString(hipError_t) { return "emu"; }
+inline hipError_t hipGetDevice(int* d) { *d = 0; return hipSuccess; }
+#define HIP_SYMBOL(x) x
+template <typename T>
+inline hipError_t hipGetSymbolAddress(void** p, T& symbol) { *p = (void*)&symbol; return hipSuccess; }
 inline hipError_t hipMemsetAsync(void* p, int v, size_t n, hipStream_t) { memset(p, v, n); return hipSuccess; }
 
 namespace emu {
