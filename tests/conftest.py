@@ -28,3 +28,16 @@ def _seed_every_test():
     import torch
     torch.manual_seed(1234)
     yield
+
+
+def pytest_sessionfinish(session, exitstatus):
+    """LLSA_PARITY_REPORT=<file>: write the errors the parity checks measured (rel-L2, max-abs per tensor and the
+    fractions of rows whose selection equals the oracle's) as JSON."""
+    path = os.environ.get("LLSA_PARITY_REPORT")
+    if not path:
+        return
+    import json
+    mod = sys.modules.get("parity_cases")
+    if mod is not None and mod.MEASURED:
+        with open(path, "w") as f:
+            json.dump(mod.MEASURED, f, indent=1)

@@ -13,12 +13,18 @@ from llsa_amd._lib import override_library_for_tests
 from llsa_amd.caller import dit as D
 
 
+_SELECTIONS = []        # with share_selection: what the device chose, one entry per attention call, in call order
+
+
 class _OracleAttn(Function):
     @staticmethod
     def forward(ctx, q, k, v, levels, t1, t2):
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
         if levels == 1:
             o, c = O.llsa_l1_fwd(q, k, v, t1, 16)
+        elif levels == 2 and _SELECTIONS:
+            idx, pidx = _SELECTIONS.pop(0)
+            o, c = O.llsa_l2_fwd(q, k, v, t1, t2, 16, indices=idx, p_indices=pidx.long())
         elif levels == 2:
             o, c = O.llsa_l2_fwd(q, k, v, t1, t2, 16)
         else:
@@ -82,7 +88,11 @@ def _loss_and_grads(model, batch, dev):
     return loss.item(), {n: p.grad.detach().float().cpu() for n, p in model.named_parameters() if p.grad is not None}
 
 
-def _compare(dev, monkeypatch, fused, **cfg):
+def _compare(dev, monkeypatch, fused, batch_size=1, share_selection=False, **cfg):
+    """share_selection: the oracle's attention takes the blocks the device selected in the same layer (deep models
+    on fresh weights have nearly uniform pooled scores in the later layers, where the bf16 GEMMs of GPU and CPU round
+    q and k differently and the two sides would otherwise attend to different blocks; the selection itself is
+    compared with the oracle's in the operator tests)."""
     torch.manual_seed(3)
     ref = D.PixelDiT(fused_prologue=False, **cfg)
     with torch.no_grad():                       # the adaLN gates start at random values: every block contributes
@@ -92,8 +102,19 @@ def _compare(dev, monkeypatch, fused, **cfg):
     got = D.PixelDiT(fused_prologue=fused, **cfg)
     got.load_state_dict(ref.state_dict())
     got.to(dev)
-    batch = _batch(1, cfg["sample_size"])
-    loss, grads = _loss_and_grads(got, batch, dev)
+    batch = _batch(batch_size, cfg["sample_size"])
+    del _SELECTIONS[:]
+    with monkeypatch.context() as mp:
+        if share_selection:
+            from llsa_amd.kernel.torch_op._fused import selection
+            real = D.llsa_l2
+
+            def recording(*a, **kw):
+                out = real(*a, **kw)
+                _SELECTIONS.append(tuple(t.cpu() for t in selection(out)))
+                return out
+            mp.setattr(D, "llsa_l2", recording)
+        loss, grads = _loss_and_grads(got, batch, dev)
     with monkeypatch.context() as mp:
         _oracle_ops(mp)
         rloss, rgrads = _loss_and_grads(ref, batch, torch.device("cpu"))
@@ -148,6 +169,15 @@ def test_step_against_oracle_ops_emulated(monkeypatch, fused):
 def test_step_against_oracle_ops_gpu(monkeypatch, fused, levels, side):
     _compare(torch.device("cuda:0"), monkeypatch, fused, num_attention_heads=2, num_layers=2, sample_size=side,
              levels=levels, sparse_topk=8)
+
+
+@pytest.mark.gpu
+def test_full_dit_s_step_against_oracle_ops_gpu(monkeypatch):
+    """The benchmark's training-step configuration at its depth and width -- 12 layers, 6 heads of 64, 128 x 128
+    pixels = 16384 tokens, llsa_l2 with topk 16/16, fused prologue -- at batch 2 (the oracle side runs on the CPU)."""
+    _compare(torch.device("cuda:0"), monkeypatch, True, batch_size=2, share_selection=True, num_attention_heads=6,
+             num_layers=12, sample_size=128, levels=2, sparse_topk=16)
+    assert not _SELECTIONS, "the oracle side made fewer attention calls than the device side"
 
 
 @pytest.mark.gpu

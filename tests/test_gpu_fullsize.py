@@ -53,6 +53,12 @@ def test_c3_full_size_against_oracle(dev):
     P.check_op_l2(dev, B=2, H=6, N=16384, T=16, T2=16, fused=True, rope=True, smooth=True)
 
 
+def test_c5_full_size_two_heads_against_oracle(dev):
+    """Benchmark configuration 5 at its shape, B=1, H=6, N=262144, topk 16/16, RoPE in the kernel (six (b,h) in the
+    split-form index transpose and the workspace strides); the oracle runs on the first and the last head."""
+    P.check_op_l2(dev, B=1, H=6, N=262144, T=16, T2=16, fused=True, rope=True, smooth=True, slices=[(0, 0), (0, 5)])
+
+
 @pytest.mark.parametrize("H,T,T2,T3,rope,qk_norm", [(1, 16, 16, 16, True, False), (2, 8, 4, 8, False, True)])
 def test_three_levels_against_oracle(dev, H, T, T2, T3, rope, qk_norm):
     """llsa_l3 (no counterpart in the reference) at its smallest size, N = 262144, against the oracle's
