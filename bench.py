@@ -85,7 +85,7 @@ def stage_profile(op, q, k, v, do, t1, t2, freq, iters, torch):
     """Runs the kernels of one forward + backward one stage at a time, the same launches the
     fused operator makes, and times each stage with events on the launch stream."""
     from llsa_amd.kernel.hip import _attention as A
-    from llsa_amd._lib import CHUNK_COARSE, CHUNK_FINE
+    from llsa_amd._lib import CHUNK_FINE
     from llsa_amd.kernel.hip.indices_transpose import transpose_indices
     from llsa_amd.kernel.hip.mean_pool import PoolSpec, pool_pyramid
     from llsa_amd.kernel.hip.topk import compute_topk_indices_sparse, gen_sparse_indices
@@ -126,7 +126,7 @@ def stage_profile(op, q, k, v, do, t1, t2, freq, iters, torch):
 
     def transposes():
         r = transpose_indices(idx, N // 16, CHUNK_FINE)
-        return r + transpose_indices(pidx, N // 256, CHUNK_COARSE) if l2 else r
+        return r + transpose_indices(pidx, N // 256, inverse=True) if l2 else r
 
     csr = transposes()
     res["transpose_indices"] = timed(transposes, iters, torch)

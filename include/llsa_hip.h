@@ -186,17 +186,22 @@ int llsa_attn_fwd(const llsa_attn_fwd_args* a, void* stream);
  * Index transpose.  Replaces transpose_indices (kernel/triton/indices_transpose.py:104-109):
  * idx (B,H,Mb,T) -> offsets (B,H,Kb+1) with offsets[0] = 0 and flat (B,H,Mb*T); segment n of
  * flat lists the query blocks that selected key block n in ASCENDING order (the reference's
- * order is whatever its atomics produce).  Rows of idx must hold distinct values.
+ * order is whatever its atomics produce).  Rows of idx must hold distinct values in [0, Kb): a
+ * value named twice in a row collapses to one list entry and leaves the tail of the segment
+ * undefined (nothing is read or written out of bounds).
+ * With `inv` (B,H,Mb,T) the inverse is written too: inv[q][t] = position in flat of the entry
+ * that (query block q, slot t) became.  llsa_attn_bwd needs it for the selections of the pooled
+ * levels (pidx, ppidx): the partial sums of a key block are stored at the positions of its list.
  * ---------------------------------------------------------------------------------------- */
 int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, int32_t* work /* or NULL */,
-                           int B, int H, int Mb, int Kb, int T, int chunk, void* stream);
+                           int32_t* inv /* or NULL */, int B, int H, int Mb, int Kb, int T, int chunk, void* stream);
 
 /* Work list for the K-side backward kernels, written by llsa_transpose_indices when `work` is
  * given: every key block's segment is cut into chunks of at most `chunk` entries, one work item
  * per chunk, so that a key block selected by very many query blocks is spread over many waves
  * (the reference walks each segment serially, sparse_attention_res_1.py:300-322).  `work` is
- * (B,H,llsa_work_list_len(Mb,Kb,T,chunk)) int32, 16-byte aligned; llsa_attn_bwd needs
- * chunk = LLSA_CHUNK_FINE for idx and chunk = LLSA_CHUNK_COARSE for pidx.  Per (b,h), in int32:
+ * (B,H,llsa_work_list_len(Mb,Kb,T,chunk)) int32, 16-byte aligned; llsa_attn_bwd needs the
+ * work list of idx with chunk = LLSA_CHUNK_FINE (the pooled levels need none).  Per (b,h), in int32:
  *   [0] items, [1] partial-sum slots, [2] key blocks with more than one chunk, [3] 0
  *   [4 + 4i ..]              item i = {key block, first entry in flat, entries, partial-sum slot or -1};
  *                            items with more than chunk/2 entries come first
@@ -205,8 +210,6 @@ int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, 
  * with max_items = Mb*T/chunk + Kb; every key block has at least one item. */
 int64_t llsa_work_list_len(int Mb, int Kb, int T, int chunk);
 #define LLSA_CHUNK_FINE 64
-#define LLSA_CHUNK_COARSE 8
-#define LLSA_CHUNK_COARSE2 1
 
 /* ------------------------------------------------------------------------------------------
  * Backward.  Replaces sparse_indices_attn_res_scatter_bwd_v2 (sparse_attention_res_1.py:403-471)
@@ -228,7 +231,7 @@ typedef struct llsa_attn_bwd_args {
     const void* pk2r; const void* pv2r;          /* R tiles of pk2, pv2 (B,H,N/4096,1024)         */
     const int32_t* idx;  const int32_t* pidx;
     const int32_t* off;  const int32_t* flat;  const int32_t* work;    /* transposed idx  (Kb = N/16)     */
-    const int32_t* poff; const int32_t* pflat; const int32_t* pwork;   /* transposed pidx (Kb = N/256)    */
+    const int32_t* poff; const int32_t* pinv;    /* transposed pidx (Kb = N/256): offsets and inverse positions */
     void* dq; int64_t sdqb, sdqh, sdqn;
     void* dk; int64_t sdkb, sdkh, sdkn;
     void* dv; int64_t sdvb, sdvh, sdvn;
@@ -250,8 +253,7 @@ typedef struct llsa_attn_bwd_args {
     /* levels == 3 (no counterpart in the reference): one more pooled level */
     const void* pk3r; const void* pv3r;          /* R tiles of pk3, pv3 (B,H,N/65536,1024)        */
     const int32_t* ppidx;                        /* (B,H,N/4096,T3) selected level-2 blocks        */
-    const int32_t* ppoff; const int32_t* ppflat; const int32_t* ppwork;  /* transposed ppidx (Kb = N/4096,
-                                                    chunk = LLSA_CHUNK_COARSE2)                    */
+    const int32_t* ppoff; const int32_t* ppinv;  /* transposed ppidx (Kb = N/4096): offsets, inverse positions */
     void* dpk3; void* dpv3;                      /* (B,H,N/4096,64) contiguous out                 */
     int32_t T3;
     float w3;

@@ -46,7 +46,7 @@ class AttnBwdArgs(C.Structure):
         + [("lse", c_void_p), ("qr", c_void_p), ("kr", c_void_p), ("vr", c_void_p),
            ("pkr", c_void_p), ("pvr", c_void_p), ("pk2r", c_void_p), ("pv2r", c_void_p),
            ("idx", c_void_p), ("pidx", c_void_p), ("off", c_void_p), ("flat", c_void_p), ("work", c_void_p),
-           ("poff", c_void_p), ("pflat", c_void_p), ("pwork", c_void_p)]
+           ("poff", c_void_p), ("pinv", c_void_p)]
         + [("dq", c_void_p), ("sdqb", c_int64), ("sdqh", c_int64), ("sdqn", c_int64),
            ("dk", c_void_p), ("sdkb", c_int64), ("sdkh", c_int64), ("sdkn", c_int64),
            ("dv", c_void_p), ("sdvb", c_int64), ("sdvh", c_int64), ("sdvn", c_int64)]
@@ -54,8 +54,8 @@ class AttnBwdArgs(C.Structure):
            ("workspace", c_void_p), ("workspace_bytes", c_int64), ("freq_dq", c_void_p), ("freq_dk", c_void_p),
            ("B", c_int32), ("H", c_int32), ("N", c_int32), ("T", c_int32), ("T2", c_int32), ("levels", c_int32),
            ("w1", c_float), ("w2", c_float), ("cgw1", c_float), ("stages", c_int32), ("fold_pooled", c_int32),
-           ("pk3r", c_void_p), ("pv3r", c_void_p), ("ppidx", c_void_p), ("ppoff", c_void_p), ("ppflat", c_void_p),
-           ("ppwork", c_void_p), ("dpk3", c_void_p), ("dpv3", c_void_p), ("T3", c_int32), ("w3", c_float)])
+           ("pk3r", c_void_p), ("pv3r", c_void_p), ("ppidx", c_void_p), ("ppoff", c_void_p), ("ppinv", c_void_p),
+           ("dpk3", c_void_p), ("dpv3", c_void_p), ("T3", c_int32), ("w3", c_float)])
 
 
 P64 = C.POINTER(c_int64)
@@ -78,14 +78,14 @@ _SIGNATURES = {
     "llsa_topk_dense": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llsa_topk_sparse": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llsa_attn_fwd": (c_int, [C.POINTER(AttnFwdArgs), c_void_p]),
-    "llsa_transpose_indices": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "llsa_transpose_indices": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llsa_work_list_len": (c_int64, [c_int, c_int, c_int, c_int]),
     "llsa_attn_bwd_workspace_bytes": (c_int64, [c_int, c_int, c_int, c_int, c_int, c_int, c_int]),
     "llsa_attn_bwd": (c_int, [C.POINTER(AttnBwdArgs), c_void_p]),
 }
 
 EXPORTS = tuple(_SIGNATURES)
-CHUNK_FINE, CHUNK_COARSE, CHUNK_COARSE2 = 64, 8, 1          # LLSA_CHUNK_* of include/llsa_hip.h
+CHUNK_FINE = 64                                             # LLSA_CHUNK_FINE of include/llsa_hip.h
 STATIC_PARTIALS_MAX = 262144                                # LLSA_STATIC_PARTIALS_MAX
 
 

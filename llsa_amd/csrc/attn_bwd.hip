@@ -245,13 +245,12 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, floa
 }
 
 // ---------------------------------------------------------------------------------------
-// K-side gradients.  A "unit" is 16 key rows (a fine K block, 16 level-1 pooled tokens of one
-// coarse block, or 16 tokens of the dense coarsest level) together with a list of query
-// blocks; the unit's waves walk the list two query blocks at a time.  attn_kside_kernel serves
-// the two list-driven passes, attn_kside_dense_kernel the dense one.
+// K-side gradients.  A "unit" is 16 key rows (a fine K block, 16 pooled tokens of one coarse
+// block, or 16 tokens of the dense coarsest level).  Three kernels: attn_kside_kernel walks the
+// transposed selection of the fine blocks (unit-major: a unit and the list of query blocks that
+// selected it), attn_kside_group_kernel the pooled levels under an ancestor's selection
+// (query-group-major), attn_kside_dense_kernel the dense coarsest level.
 // ---------------------------------------------------------------------------------------
-enum { MODE_FINE = 0, MODE_SPARSE1 = 1, MODE_SPARSE2 = 2 };   // (the dense coarsest level has a kernel of its own)
-// SPARSE1: a list entry is a parent and stands for its 16 children; SPARSE2 (three levels): a grand-parent, 256 query blocks
 
 // Optional last step of the fine dK / dV: add the pooled gradients the token's block received
 // (what the backward of the two mean pools and autograd's accumulation do in the reference:
@@ -300,17 +299,17 @@ struct KSideParams {
     const bf16* qr;  const bf16* dor;             // R tiles of q and dO, (BH, N1, 1024)
     const float* lse; const float* delta;         // (BH, N)
     const bf16* kk;  const bf16* vv;              // R tiles the unit's 16 key rows come from, (BH, n_units, 1024)
-    const int* off;  const int* flat;             // CSR of the list (FINE: per K block, SPARSE1: per coarse block)
+    const int* off;  const int* flat;             // CSR of the transposed selection (per K block)
     const int* work;                              // work list over that CSR (see transpose.hip)
-    bf16* dk; int64_t sdkb, sdkh, sdkn;           // bf16 outputs (FINE, SPARSE1)
+    bf16* dk; int64_t sdkb, sdkh, sdkn;           // bf16 outputs
     bf16* dv; int64_t sdvb, sdvh, sdvn;
-    f32x4* part;                                  // fp32 partials: slots (FINE, SPARSE1) or chunks (DENSE)
+    f32x4* part;                                  // fp32 partials: slots (fine pass) or chunks (dense pass)
     int H, N, n_units, chunk_len;
     int64_t flat_stride;                          // entries of `flat` per (b,h)
     int64_t work_stride;                          // ints of `work` per (b,h)
     int64_t slot_stride;                          // partial slots per (b,h)
     float w;
-    PoolFold fold;                                // FINE only
+    PoolFold fold;                                // fine pass only
 };
 
 // Two query blocks (g0, g1; g1 < 0: only one) against the unit's 16 key rows.  Q and dO are
@@ -318,7 +317,7 @@ struct KSideParams {
 // the registers, and they are parked in a wave-private piece of LDS (`stage`, 4096 elements)
 // from which the transposing LDS read delivers them again as T operands for dV^T += dO^T.P and
 // dK^T += Q^T.dS.
-__device__ __forceinline__ void kside_pair(f32x4 dk[4], f32x4 dv[4], const bf16x8 bk[2], const bf16x8 bv[2], float w,
+__device__ __forceinline__ void kside_pair(f32x4 dk[4], f32x4 dv[4], const bf16x8 bk[2], const bf16x8 bv[2],
                                            int g0, int g1, const bf16* qrb, const bf16* dorb, const float* lseb,
                                            const float* dlb, bf16* stage, int lane) {
     const int quad = lane >> 4;
@@ -355,7 +354,7 @@ __device__ __forceinline__ void kside_pair(f32x4 dk[4], f32x4 dv[4], const bf16x
         dp = mfma_bf16(ag[u][1], bv[1], dp);
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            float pe = exp2_fast(fmaf(s[e], kScaleLog2e, -l4[u][e] * kLog2e)) * w;
+            float pe = exp2_fast(fmaf(s[e], kScaleLog2e, -l4[u][e] * kLog2e));
             if (!valid) pe = 0.f;
             bp[u * 4 + e] = (bf16)pe;
             bds[u * 4 + e] = (bf16)(pe * (dp[e] - d4[u][e]));
@@ -376,16 +375,19 @@ __device__ __forceinline__ void kside_pair(f32x4 dk[4], f32x4 dv[4], const bf16x
 // accumulator layout: 8 f32x4 registers per lane (4 channel tiles of dK, then 4 of dV).
 __device__ __forceinline__ f32x4* part_slot(f32x4* part, int64_t slot) { return part + slot * (8 * kWave); }
 
-template <int MODE>
-__device__ __forceinline__ void kside_item(const KSideParams& p, int bx, int bh, unsigned char* smem_raw, bf16* fold_buf) {
-    constexpr int W = (MODE == MODE_FINE) ? 1 : 4;            // waves per work item = waves per workgroup
-    constexpr int kFanShift = (MODE == MODE_SPARSE2) ? 8 : 4;
+// One work item of the fine pass: a key block and a piece (at most LLSA_CHUNK_FINE entries) of its list.
+// One wave = one workgroup per item (items differ a lot in length; a wave that shared its workgroup
+// with a longer one would keep its registers and LDS allocated while idle).
+__global__ __launch_bounds__(64) void attn_kside_kernel(KSideParams p) {
+    __shared__ __align__(16) bf16 stage[4 * kTile];           // 2 query blocks x {Q, dO} R tiles
+    __shared__ __align__(16) bf16 fold_buf[kFoldElems];
+    const int lid = xcd_logical_id();
+    const int item = lid % (int)gridDim.x;
+    const int bh = lid / (int)gridDim.x;
     const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int N1 = p.N / kBlk;
     const int b = bh / p.H, h = bh % p.H;
     const int r = lane & 15, quad = lane >> 4;
-    const int sub = (MODE == MODE_FINE) ? 0 : wave;
 
     // which 16 key rows, which part of their query-block list, and where the result goes
     int unit, start, cnt;
@@ -395,21 +397,19 @@ __device__ __forceinline__ void kside_item(const KSideParams& p, int bx, int bh,
         // the item's record is fetched together with the count it is checked against (the grid never
         // exceeds the list's storage): the wave knows its key rows and entries after one round trip
         const int* work = p.work + (int64_t)bh * p.work_stride;
-        const int item = bx;
         const int n_items = work[0];
         const int* rec = work + 4 + 4 * item;
         unit = rec[0];
         start = rec[1];
         cnt = rec[2];
         const int sl = rec[3];
-        if (item >= n_items) return;                          // uniform over the item's waves
-        if (MODE != MODE_FINE) cnt <<= kFanShift;             // every entry stands for its children
+        if (item >= n_items) return;
         if (sl >= 0) slot = (int64_t)bh * p.slot_stride + sl;
         fl = p.flat + (int64_t)bh * p.flat_stride;
     }
     // What the fold on the way out needs (the unit's pooled-gradient rows, its tokens' RoPE entries)
     // is copied into LDS now, without registers, so that no load waits at the end of the wave.
-    const bool folding = MODE == MODE_FINE && p.fold.g1k != nullptr && slot < 0;
+    const bool folding = p.fold.g1k != nullptr && slot < 0;
     if (folding) {
         const int row = lane >> 3, piece = lane & 7;          // rows: dpk, dpv, dpk2, dpv2, dpk3, dpv3 of the unit; 8 x 16 bytes each
         const int deep = p.fold.g3k != nullptr ? 3 : p.fold.g2k != nullptr ? 2 : 1;
@@ -427,14 +427,10 @@ __device__ __forceinline__ void kside_item(const KSideParams& p, int bx, int bh,
             copy16_global_to_lds(fr + 512 + lane * 8, fold_buf + kFoldRows + 512);
         }
     }
-    // The item's list entries (FINE: at most 32 query blocks) are fetched once, entry i into
-    // lane i, and handed out with readlane: the walk below then has no load that depends on a load.
-    int mine = 0;
-    if (MODE == MODE_FINE) mine = (lane < cnt) ? fl[start + lane] : 0;
-    auto entry = [&](int i) -> int {                          // i-th query block of this item (i is wave-uniform)
-        if (MODE == MODE_FINE) return clampi(__builtin_amdgcn_readlane(mine, i), 0, N1 - 1);
-        return (clampi(fl[start + (i >> kFanShift)], 0, (N1 >> kFanShift) - 1) << kFanShift) + (i & ((1 << kFanShift) - 1));
-    };
+    // The item's list entries (at most 64 query blocks) are fetched once, entry i into lane i, and
+    // handed out with readlane: the walk below then has no load that depends on a load.
+    const int mine = (lane < cnt) ? fl[start + lane] : 0;
+    auto entry = [&](int i) -> int { return clampi(__builtin_amdgcn_readlane(mine, i), 0, N1 - 1); };   // i is wave-uniform
 
     f32x4 dk[4], dv[4];
 #pragma unroll
@@ -454,154 +450,129 @@ __device__ __forceinline__ void kside_item(const KSideParams& p, int bx, int bh,
         const bf16* dorb = p.dor + (int64_t)bh * N1 * kTile;
         const float* lseb = p.lse + (int64_t)bh * p.N;
         const float* dlb = p.delta + (int64_t)bh * p.N;
-        bf16* stage = reinterpret_cast<bf16*>(smem_raw) + wave * (4 * kTile);
-        for (int i = 2 * sub; i < cnt; i += 2 * W) {
+        for (int i = 0; i < cnt; i += 2) {
             const int g0 = entry(i);
             const int g1 = (i + 1 < cnt) ? entry(i + 1) : -1;
-            kside_pair(dk, dv, bk, bv, p.w, g0, g1, qrb, dorb, lseb, dlb, stage, lane);
+            kside_pair(dk, dv, bk, bv, g0, g1, qrb, dorb, lseb, dlb, stage, lane);
         }
     }
 
-    if (MODE == MODE_FINE) {
-        if (slot >= 0) {
-            f32x4* ps = part_slot(p.part, slot);
-#pragma unroll
-            for (int dt = 0; dt < 4; dt++) {
-                ps[dt * kWave + lane] = dk[dt];
-                ps[(4 + dt) * kWave + lane] = dv[dt];
-            }
-            return;
-        }
-        bf16* kp = p.dk + b * p.sdkb + h * p.sdkh + (int64_t)(unit * kBlk + r) * p.sdkn + quad * 4;
-        bf16* vp = p.dv + b * p.sdvb + h * p.sdvh + (int64_t)(unit * kBlk + r) * p.sdvn + quad * 4;
-        if (folding) wait_vm0();                              // the copies into fold_buf (long since done)
+    if (slot >= 0) {
+        f32x4* ps = part_slot(p.part, slot);
 #pragma unroll
         for (int dt = 0; dt < 4; dt++) {
-            bf16x4 ok = cvt4(dk[dt] * kScale), ov = cvt4(dv[dt]);
-            if (folding) {
-                const int c0 = dt * 16 + quad * 4;
-                const bool two = p.fold.g2k != nullptr, three = p.fold.g3k != nullptr, rot = p.fold.freq != nullptr;
-                ok = fold_math(ok, lds_ld8(fold_buf + c0), two, lds_ld8(fold_buf + 2 * kD + c0), rot,
-                               lds_ld8(fold_buf + kFoldRows + r * kD + c0), three, lds_ld8(fold_buf + 4 * kD + c0));
-                ov = fold_math(ov, lds_ld8(fold_buf + kD + c0), two, lds_ld8(fold_buf + 3 * kD + c0), false, ov, three,
-                               lds_ld8(fold_buf + 5 * kD + c0));
-            }
-            st8(kp + dt * 16, ok);
-            st8(vp + dt * 16, ov);
+            ps[dt * kWave + lane] = dk[dt];
+            ps[(4 + dt) * kWave + lane] = dv[dt];
         }
         return;
     }
-    // four waves per item: reduce through LDS, wave w finishes channel tile w
-    __syncthreads();                                          // everyone is done with the staging area
-    f32x4 (*red)[8][kWave] = reinterpret_cast<f32x4 (*)[8][kWave]>(smem_raw);
-    static_assert(MODE == MODE_FINE || W * 4 * kTile * sizeof(bf16) >= 4 * 8 * kWave * sizeof(f32x4), "reduction buffer must fit the staging area");
+    bf16* kp = p.dk + b * p.sdkb + h * p.sdkh + (int64_t)(unit * kBlk + r) * p.sdkn + quad * 4;
+    bf16* vp = p.dv + b * p.sdvb + h * p.sdvh + (int64_t)(unit * kBlk + r) * p.sdvn + quad * 4;
+    if (folding) wait_vm0();                                  // the copies into fold_buf (long since done)
 #pragma unroll
     for (int dt = 0; dt < 4; dt++) {
-        red[wave][dt][lane] = dk[dt];
-        red[wave][4 + dt][lane] = dv[dt];
+        bf16x4 ok = cvt4(dk[dt] * kScale), ov = cvt4(dv[dt]);
+        if (folding) {
+            const int c0 = dt * 16 + quad * 4;
+            const bool two = p.fold.g2k != nullptr, three = p.fold.g3k != nullptr, rot = p.fold.freq != nullptr;
+            ok = fold_math(ok, lds_ld8(fold_buf + c0), two, lds_ld8(fold_buf + 2 * kD + c0), rot,
+                           lds_ld8(fold_buf + kFoldRows + r * kD + c0), three, lds_ld8(fold_buf + 4 * kD + c0));
+            ov = fold_math(ov, lds_ld8(fold_buf + kD + c0), two, lds_ld8(fold_buf + 3 * kD + c0), false, ov, three,
+                           lds_ld8(fold_buf + 5 * kD + c0));
+        }
+        st8(kp + dt * 16, ok);
+        st8(vp + dt * 16, ov);
     }
-    __syncthreads();
-    const int dt = wave;
-    f32x4 sk = red[0][dt][lane], sv = red[0][4 + dt][lane];
-#pragma unroll
-    for (int w = 1; w < 4; w++) {
-        sk += red[w][dt][lane];
-        sv += red[w][4 + dt][lane];
-    }
-    if (slot >= 0) {
-        f32x4* ps = part_slot(p.part, slot);
-        ps[dt * kWave + lane] = sk;
-        ps[(4 + dt) * kWave + lane] = sv;
-    } else {
-        bf16* kp = p.dk + b * p.sdkb + h * p.sdkh + (int64_t)(unit * kBlk + r) * p.sdkn + quad * 4 + dt * 16;
-        bf16* vp = p.dv + b * p.sdvb + h * p.sdvh + (int64_t)(unit * kBlk + r) * p.sdvn + quad * 4 + dt * 16;
-        st8(kp, cvt4(sk * kScale));
-        st8(vp, cvt4(sv));
-    }
-}
-
-template <int MODE>
-__global__ __launch_bounds__(MODE == MODE_FINE ? 64 : 256) void attn_kside_kernel(KSideParams p) {
-    // FINE: one wave per work item and per workgroup (items differ a lot in length; a wave that
-    // shares its workgroup with a longer one would keep its registers and LDS allocated while idle).
-    // Others: four waves per work item.
-    constexpr int W = (MODE == MODE_FINE) ? 1 : 4;
-    // per wave 2 query blocks x {Q, dO} R tiles; reused for the cross-wave reduction
-    __shared__ __align__(16) unsigned char smem_raw[W * 4 * kTile * sizeof(bf16)];
-    __shared__ __align__(16) bf16 fold_buf[MODE == MODE_FINE ? kFoldElems : 8];
-    const int lid = xcd_logical_id();
-    const int bx = lid % (int)gridDim.x;
-    const int bh = lid / (int)gridDim.x;
-    kside_item<MODE>(p, bx, bh, smem_raw, fold_buf);
 }
 
 // ---------------------------------------------------------------------------------------
 // Dense coarsest level.  Every unit (16 pooled tokens) meets every query block, so the Q / dO
-// tiles are the same for all units: a workgroup takes four units (one per wave) and one piece
-// of the query range, and the tiles of each pair of query blocks are copied into LDS once for
-// the four of them (two 8 KB buffers: the copy of pair t+1 runs during the arithmetic of pair t).
-// Each wave ends with the partial sum of its unit over this piece of the range.
+// tiles are the same for all units: a workgroup takes 4 * UPW units (UPW per wave) and one piece
+// of the query range and streams that piece through LDS, a pair of query blocks (8 KB) per
+// round, once for all of its units.  The more units a workgroup holds, the fewer times the whole
+// of Q and dO is streamed through the chip: with many coarsest tokens (long sequences) that
+// stream is what the pass costs.
+// The stream is three rounds deep: the tiles of round t + 3 are requested from memory (every wave a
+// quarter, into registers) while those of round t + 1 move from registers into the other LDS buffer
+// and round t is worked on, so a tile has two rounds of arithmetic to arrive.  (Copies straight
+// into LDS cannot be run ahead like that: the compiler waits for all of them before any LDS read.)
+// Each wave ends with the partial sums of its units over this piece of the range.
 // ---------------------------------------------------------------------------------------
-constexpr int kDenseUnits = 4;                    // units (= waves) per workgroup
+constexpr int kDenseWaves = 4;                    // waves per workgroup
 
-__global__ __launch_bounds__(64 * kDenseUnits) void attn_kside_dense_kernel(KSideParams p) {
+template <int UPW>
+__global__ __launch_bounds__(64 * kDenseWaves) void attn_kside_dense_kernel(KSideParams p) {
     __shared__ __align__(16) bf16 sh[2][4 * kTile];           // per pair: Q0, dO0, Q1, dO1 as R tiles
+    __shared__ __align__(16) float sh_stats[2][64];           // per pair: lse of its 32 queries, then delta
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int quad = lane >> 4;
     const int N1 = p.N / kBlk;
-    const int bh = blockIdx.y;
-    const int unit = blockIdx.x * kDenseUnits + wave;         // < n_units: the host checks n_units % kDenseUnits == 0
-    const int start = blockIdx.z * p.chunk_len;
+    // Workgroups that stream the same piece of the query range (one per group of units) get neighbouring logical ids,
+    // which xcd_logical_id keeps on one XCD: the piece then comes out of that XCD's L2 for all but the first of them.
+    const int unit_groups = p.n_units / (kDenseWaves * UPW);
+    const int lid = xcd_logical_id();                          // grid: (unit_groups * chunks, BH)
+    const int piece = (lid % (int)gridDim.x) / unit_groups;
+    const int bh = lid / (int)gridDim.x;
+    const int unit0 = (((lid % (int)gridDim.x) % unit_groups) * kDenseWaves + wave) * UPW;   // + UPW <= n_units (the plan sees to it)
+    const int start = piece * p.chunk_len;
     const int n_pairs = min(p.chunk_len, N1 - start) / 2;     // chunk_len and N1 are even
+    if (n_pairs <= 0) return;                                 // uniform over the workgroup
     const bf16* qrb = p.qr + ((int64_t)bh * N1 + start) * kTile;
     const bf16* dorb = p.dor + ((int64_t)bh * N1 + start) * kTile;
     const float* lseb = p.lse + (int64_t)bh * p.N + start * kBlk;
     const float* dlb = p.delta + (int64_t)bh * p.N + start * kBlk;
 
-    // wave w copies tile w of the pair's four (query block w/2; Q for even w, dO for odd w)
-    auto issue = [=](int t) __attribute__((always_inline)) {
+    // wave w moves tile w of a pair's four (query block w/2; Q for even w, dO for odd w); the first 16 lanes of wave 0
+    // also its 64 statistics.  Rounds past the end re-read the last pair (no branch around loads).
+    struct Stage { bf16x8 a, b; f32x4 s; };
+    const bool stat_lane = wave == 0 && lane < 16;
+    auto request = [=](int t, Stage& st) __attribute__((always_inline)) {
+        t = min(t, n_pairs - 1);
         const bf16* src = ((wave & 1) ? dorb : qrb) + (int64_t)(2 * t + (wave >> 1)) * kTile;
+        st.a = ld16(src + lane * 8);
+        st.b = ld16(src + 512 + lane * 8);
+        if (stat_lane) st.s = *reinterpret_cast<const f32x4*>((lane < 8 ? lseb : dlb) + 2 * t * kBlk + (lane & 7) * 4);
+    };
+    auto deposit = [&](int t, const Stage& st) __attribute__((always_inline)) {
         bf16* dst = &sh[t & 1][wave * kTile];
-        copy16_global_to_lds(src + lane * 8, dst);
-        copy16_global_to_lds(src + 512 + lane * 8, dst + 512);
+        st16(dst + lane * 8, st.a);
+        st16(dst + 512 + lane * 8, st.b);
+        if (stat_lane) *reinterpret_cast<f32x4*>(&sh_stats[t & 1][lane * 4]) = st.s;
     };
-    struct Stats { f32x4 l[2], d[2]; };
-    auto load_stats = [=](int t, Stats& st) __attribute__((always_inline)) {
+    Stage s0, s1;
+    s0.s = s1.s = f32x4{0.f, 0.f, 0.f, 0.f};
+    request(0, s0);
+    request(1, s1);
+    bf16x8 bk[UPW][2], bv[UPW][2];
 #pragma unroll
-        for (int u = 0; u < 2; u++) {
-            st.l[u] = *reinterpret_cast<const f32x4*>(lseb + (2 * t + u) * kBlk + quad * 4);
-            st.d[u] = *reinterpret_cast<const f32x4*>(dlb + (2 * t + u) * kBlk + quad * 4);
+    for (int j = 0; j < UPW; j++) {
+        const bf16* kp = p.kk + ((int64_t)bh * p.n_units + unit0 + j) * kTile + lane * 8;
+        const bf16* vp = p.vv + ((int64_t)bh * p.n_units + unit0 + j) * kTile + lane * 8;
+        bk[j][0] = ld16(kp);
+        bk[j][1] = ld16(kp + 512);
+        bv[j][0] = ld16(vp);
+        bv[j][1] = ld16(vp + 512);
+    }
+    deposit(0, s0);
+    request(2, s0);
+    f32x4 dk[UPW][4], dv[UPW][4];
+#pragma unroll
+    for (int j = 0; j < UPW; j++)
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+            dk[j][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            dv[j][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
         }
-    };
-    if (n_pairs > 0) issue(0);
-    bf16x8 bk[2], bv[2];
-    {
-        const bf16* kp = p.kk + ((int64_t)bh * p.n_units + unit) * kTile + lane * 8;
-        const bf16* vp = p.vv + ((int64_t)bh * p.n_units + unit) * kTile + lane * 8;
-        bk[0] = ld16(kp);
-        bk[1] = ld16(kp + 512);
-        bv[0] = ld16(vp);
-        bv[1] = ld16(vp + 512);
-    }
-    Stats sa, sb;
-    if (n_pairs > 0) load_stats(0, sa);
-    f32x4 dk[4], dv[4];
-#pragma unroll
-    for (int dt = 0; dt < 4; dt++) {
-        dk[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-        dv[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
-    }
-    // One round per pair.  The barrier at its top says: the pair's tiles have landed (every wave
-    // waited for its own copies) and everybody is done reading the other buffer.  All LDS reads of
-    // the round come before the next copies are issued (the compiler makes an LDS read wait for
-    // every copy into LDS issued before it).
-    auto round = [&](int t, const Stats& cur, Stats& nxt) __attribute__((always_inline)) {
-        wait_vm0();
+    // Round t.  The barrier at its top says: buffer t & 1 is filled (every wave deposited its part during round t - 1)
+    // and everybody is done reading the other buffer, which this round refills for round t + 1 out of the registers
+    // `nxt` -- which then take the request for round t + 3.
+    auto round = [&](int t, Stage& nxt) __attribute__((always_inline)) {
         __syncthreads();
         const bf16* b = &sh[t & 1][0];
         bf16x8 aq[2][2], ag[2][2];
         bf16x4 tq[2][4], tg[2][4];
+        f32x4 l4[2], d4[2];
 #pragma unroll
         for (int u = 0; u < 2; u++) {
             aq[u][0] = lds_ld16(b + (2 * u) * kTile + lane * 8);
@@ -613,41 +584,258 @@ __global__ __launch_bounds__(64 * kDenseUnits) void attn_kside_dense_kernel(KSid
                 tq[u][dt] = lds_t_operand(b + (2 * u) * kTile, dt, lane);
                 tg[u][dt] = lds_t_operand(b + (2 * u + 1) * kTile, dt, lane);
             }
+            l4[u] = *reinterpret_cast<const f32x4*>(&sh_stats[t & 1][u * kBlk + quad * 4]);
+            d4[u] = *reinterpret_cast<const f32x4*>(&sh_stats[t & 1][32 + u * kBlk + quad * 4]);
         }
-        if (t + 1 < n_pairs) {
-            issue(t + 1);
-            load_stats(t + 1, nxt);
-        }
-        bf16x8 bp, bds;
+        deposit(t + 1, nxt);
+        request(t + 3, nxt);
+        float nl[2][4];
 #pragma unroll
-        for (int u = 0; u < 2; u++) {
-            f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
-            s = mfma_bf16(aq[u][0], bk[0], s);
-            s = mfma_bf16(aq[u][1], bk[1], s);
-            dp = mfma_bf16(ag[u][0], bv[0], dp);
-            dp = mfma_bf16(ag[u][1], bv[1], dp);
+        for (int u = 0; u < 2; u++)
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const float pe = exp2_fast(fmaf(s[e], kScaleLog2e, -cur.l[u][e] * kLog2e)) * p.w;
-                bp[u * 4 + e] = (bf16)pe;
-                bds[u * 4 + e] = (bf16)(pe * (dp[e] - cur.d[u][e]));
+            for (int e = 0; e < 4; e++) nl[u][e] = -l4[u][e] * kLog2e;
+#pragma unroll
+        for (int j = 0; j < UPW; j++) {
+            bf16x8 bp, bds;
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
+                s = mfma_bf16(aq[u][0], bk[j][0], s);
+                s = mfma_bf16(aq[u][1], bk[j][1], s);
+                dp = mfma_bf16(ag[u][0], bv[j][0], dp);
+                dp = mfma_bf16(ag[u][1], bv[j][1], dp);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float pe = exp2_fast(fmaf(s[e], kScaleLog2e, nl[u][e]));
+                    bp[u * 4 + e] = (bf16)pe;
+                    bds[u * 4 + e] = (bf16)(pe * (dp[e] - d4[u][e]));
+                }
             }
-        }
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++) {
-            dv[dt] = mfma_bf16(cat(tg[0][dt], tg[1][dt]), bp, dv[dt]);
-            dk[dt] = mfma_bf16(cat(tq[0][dt], tq[1][dt]), bds, dk[dt]);
+            for (int dt = 0; dt < 4; dt++) {
+                dv[j][dt] = mfma_bf16(cat(tg[0][dt], tg[1][dt]), bp, dv[j][dt]);
+                dk[j][dt] = mfma_bf16(cat(tq[0][dt], tq[1][dt]), bds, dk[j][dt]);
+            }
         }
     };
     for (int t = 0; t < n_pairs; t += 2) {
-        round(t, sa, sb);
-        if (t + 1 < n_pairs) round(t + 1, sb, sa);
+        round(t, s1);
+        if (t + 1 < n_pairs) round(t + 1, s0);
     }
-    f32x4* ps = part_slot(p.part, ((int64_t)blockIdx.z * gridDim.y + bh) * p.n_units + unit);
 #pragma unroll
-    for (int dt = 0; dt < 4; dt++) {
-        ps[dt * kWave + lane] = dk[dt];
-        ps[(4 + dt) * kWave + lane] = dv[dt];
+    for (int j = 0; j < UPW; j++) {
+        f32x4* ps = part_slot(p.part, ((int64_t)piece * gridDim.y + bh) * p.n_units + unit0 + j);
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+            ps[dt * kWave + lane] = dk[j][dt] * p.w;         // (the weight, left out of the exponentials)
+            ps[(4 + dt) * kWave + lane] = dv[j][dt] * p.w;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------
+// Pooled levels whose keys come from an ancestor's selection (the level-1 pooled tokens of
+// llsa_l2 / llsa_l3 under the parent's coarse blocks, the level-2 pooled tokens of llsa_l3 under
+// the grand-parent's), "group-major": a workgroup owns one group of 16 consecutive query blocks
+// -- the children of one parent, which all read the same pooled key blocks -- copies their Q and
+// dO tiles into LDS once (64 KB) and meets every key block of the group's lists there; a wave
+// takes its share of the key blocks, two at a time, and ends each with that block's dK / dV summed
+// over the group's 256 queries.  A key block selected by several ancestors receives one such
+// partial sum per selecting group, written where kside_reduce_kernel finds the partial sums of a
+// key block side by side: at the position the transposed selection gives the (ancestor, entry)
+// pair.  Walking the transposed lists instead (key block major, the reference's order,
+// sparse_attention_res_2.py:492-575) fetches the 64 KB of a group once per key block that
+// selected it, T2 times in all.
+// With few tokens on the dense coarsest level its blocks are appended to the lists (every group
+// meets all of them), which saves that level a pass of its own over Q and dO.
+// ---------------------------------------------------------------------------------------
+constexpr int kGroupWaves = 4;
+constexpr int kGroupSegs = 3;
+constexpr int kGroupMaxBlocks = 64;               // key blocks per group over all its lists (their ids live in one lane each)
+constexpr int kGroupDenseMax = 8;                 // dense blocks are appended up to this many
+
+struct GroupSeg {
+    const bf16* kk; const bf16* vv;               // R tiles of this level's pooled k, v: (BH, n_units, 1024)
+    const int* sel;                               // (BH, n_groups >> owner_shift, cnt) blocks selected by the group's ancestor;
+                                                  // nullptr: blocks 0..cnt-1 (dense level)
+    const int* inv;                               // (BH, n_groups >> owner_shift, cnt) position of each entry in the transposed selection
+    f32x4* part;                                  // partial sums
+    int n_units, owner_shift, cnt;
+    int64_t slots;                                // partial slots per (b,h) (sparse) -- positions are clamped into them
+    float w;
+};
+struct GroupParams {
+    const bf16* qr; const bf16* dor;              // R tiles of q and dO, (BH, N1, 1024)
+    const float* lse; const float* delta;         // (BH, N)
+    int H, N, n_segs, n_blocks;
+    GroupSeg seg[kGroupSegs];
+};
+
+struct GroupStats { f32x4 l[2], d[2]; };
+
+// UPW key blocks against the group's 16 query blocks, two query blocks per step, operands out of LDS.
+template <int UPW>
+__device__ __forceinline__ void group_pass(const bf16x8 (&bk)[2][2], const bf16x8 (&bv)[2][2], const float (&w)[2], f32x4* const (&dst)[2],
+                                           const bf16* shq, const bf16* shg, const float* lseb, const float* dlb, int lane) {
+    const int quad = lane >> 4;
+    f32x4 dk[UPW][4], dv[UPW][4];
+#pragma unroll
+    for (int j = 0; j < UPW; j++)
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+            dk[j][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+            dv[j][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+    auto load_stats = [=](int t, GroupStats& st) __attribute__((always_inline)) {
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            st.l[u] = *reinterpret_cast<const f32x4*>(lseb + (2 * t + u) * kBlk + quad * 4);
+            st.d[u] = *reinterpret_cast<const f32x4*>(dlb + (2 * t + u) * kBlk + quad * 4);
+        }
+    };
+    auto step = [&](int t, const GroupStats& cur) __attribute__((always_inline)) {
+        bf16x8 aq[2][2], ag[2][2];
+        bf16x4 tq[2][4], tg[2][4];
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const bf16* q = shq + (2 * t + u) * kTile;
+            const bf16* g = shg + (2 * t + u) * kTile;
+            aq[u][0] = lds_ld16(q + lane * 8);
+            aq[u][1] = lds_ld16(q + 512 + lane * 8);
+            ag[u][0] = lds_ld16(g + lane * 8);
+            ag[u][1] = lds_ld16(g + 512 + lane * 8);
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) {
+                tq[u][dt] = lds_t_operand(q, dt, lane);
+                tg[u][dt] = lds_t_operand(g, dt, lane);
+            }
+        }
+        float nl[2][4];
+#pragma unroll
+        for (int u = 0; u < 2; u++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) nl[u][e] = -cur.l[u][e] * kLog2e;
+#pragma unroll
+        for (int j = 0; j < UPW; j++) {
+            bf16x8 bp, bds;
+#pragma unroll
+            for (int u = 0; u < 2; u++) {
+                f32x4 sc = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
+                sc = mfma_bf16(aq[u][0], bk[j][0], sc);
+                sc = mfma_bf16(aq[u][1], bk[j][1], sc);
+                dp = mfma_bf16(ag[u][0], bv[j][0], dp);
+                dp = mfma_bf16(ag[u][1], bv[j][1], dp);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float pe = exp2_fast(fmaf(sc[e], kScaleLog2e, nl[u][e]));   // (the weight multiplies the sums below)
+                    bp[u * 4 + e] = (bf16)pe;
+                    bds[u * 4 + e] = (bf16)(pe * (dp[e] - cur.d[u][e]));
+                }
+            }
+#pragma unroll
+            for (int dt = 0; dt < 4; dt++) {
+                dv[j][dt] = mfma_bf16(cat(tg[0][dt], tg[1][dt]), bp, dv[j][dt]);
+                dk[j][dt] = mfma_bf16(cat(tq[0][dt], tq[1][dt]), bds, dk[j][dt]);
+            }
+        }
+    };
+    GroupStats sa, sb;
+    load_stats(0, sa);
+#pragma unroll 1
+    for (int t = 0; t < kBlk / 2; t += 2) {
+        load_stats(t + 1, sb);
+        step(t, sa);
+        load_stats((t + 2) & (kBlk / 2 - 1), sa);             // (the last one re-reads step 0: no branch around loads)
+        step(t + 1, sb);
+    }
+#pragma unroll
+    for (int j = 0; j < UPW; j++)
+#pragma unroll
+        for (int dt = 0; dt < 4; dt++) {
+            dst[j][dt * kWave + lane] = dk[j][dt] * w[j];
+            dst[j][(4 + dt) * kWave + lane] = dv[j][dt] * w[j];
+        }
+}
+
+__global__ __launch_bounds__(64 * kGroupWaves, 2) void attn_kside_group_kernel(GroupParams p) {
+    __shared__ __align__(16) bf16 sh[2][kBlk * kTile];        // R tiles of the group's 16 query blocks: Q, then dO
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int N1 = p.N / kBlk;
+    const int lid = xcd_logical_id();
+    const int G = lid % (int)gridDim.x;                        // group of query blocks 16 G .. 16 G + 15
+    const int bh = lid / (int)gridDim.x;
+    const int n_groups = (int)gridDim.x;
+
+    {   // 32 KB of Q tiles and 32 KB of dO tiles, contiguous in memory, 1 KB per wave and copy
+        const bf16* qsrc = p.qr + ((int64_t)bh * N1 + (int64_t)G * kBlk) * kTile;
+        const bf16* gsrc = p.dor + ((int64_t)bh * N1 + (int64_t)G * kBlk) * kTile;
+#pragma unroll
+        for (int i = 0; i < 2 * kBlk / kGroupWaves; i++) {
+            const int piece = i * kGroupWaves + wave;
+            copy16_global_to_lds(qsrc + piece * 512 + lane * 8, &sh[0][piece * 512]);
+            copy16_global_to_lds(gsrc + piece * 512 + lane * 8, &sh[1][piece * 512]);
+        }
+    }
+    // Key block j of the group's lists lives in lane j: which tile, which weight, where its partial sum goes.
+    int my_unit = 0, my_seg = 0;
+    int64_t my_slot = 0;
+    {
+        int j = lane, sgi = 0;
+        while (sgi < p.n_segs - 1 && j >= p.seg[sgi].cnt) {
+            j -= p.seg[sgi].cnt;
+            sgi++;
+        }
+        const GroupSeg& sg = p.seg[sgi];
+        if (lane < p.n_blocks) {
+            my_seg = sgi;
+            if (sg.sel != nullptr) {
+                const int64_t e = ((int64_t)bh * (n_groups >> sg.owner_shift) + (G >> sg.owner_shift)) * sg.cnt + j;
+                my_unit = clampi(sg.sel[e], 0, sg.n_units - 1);
+                const int64_t pos = ((int64_t)clampi(sg.inv[e], 0, (int)((sg.slots >> sg.owner_shift) - 1)) << sg.owner_shift) +
+                                    (G & ((1 << sg.owner_shift) - 1));
+                my_slot = (int64_t)bh * sg.slots + pos;
+            } else {
+                my_unit = j;
+                my_slot = ((int64_t)G * gridDim.y + bh) * sg.n_units + j;      // [group][bh][unit]: what the dense reduction walks
+            }
+        }
+    }
+    const float* lseb = p.lse + (int64_t)bh * p.N + (int64_t)G * kBlk * kBlk;
+    const float* dlb = p.delta + (int64_t)bh * p.N + (int64_t)G * kBlk * kBlk;
+    // this wave's key blocks: a contiguous share, taken two at a time (the last alone if the share is odd)
+    const int per = (p.n_blocks + kGroupWaves - 1) / kGroupWaves;
+    const int lo = min(wave * per, p.n_blocks), hi = min(lo + per, p.n_blocks);
+
+    bf16x8 bk[2][2], bv[2][2];
+    float w[2];
+    f32x4* dst[2];
+    auto fetch = [&](int j, int u) __attribute__((always_inline)) {    // K, V tiles of key block j into register set u
+        const int sgi = __builtin_amdgcn_readlane(my_seg, j);
+        const int unit = __builtin_amdgcn_readlane(my_unit, j);
+        const int slo = __builtin_amdgcn_readlane((int)(my_slot & 0xffffffff), j), shi = __builtin_amdgcn_readlane((int)(my_slot >> 32), j);
+        const GroupSeg& sg = p.seg[sgi];
+        const bf16* kp = sg.kk + ((int64_t)bh * sg.n_units + unit) * kTile + lane * 8;
+        const bf16* vp = sg.vv + ((int64_t)bh * sg.n_units + unit) * kTile + lane * 8;
+        bk[u][0] = ld16(kp);
+        bk[u][1] = ld16(kp + 512);
+        bv[u][0] = ld16(vp);
+        bv[u][1] = ld16(vp + 512);
+        w[u] = sg.w;
+        dst[u] = part_slot(sg.part, ((int64_t)(unsigned)slo) | ((int64_t)shi << 32));
+    };
+    if (lo < hi) fetch(lo, 0);
+    if (lo + 1 < hi) fetch(lo + 1, 1);
+    wait_vm0();
+    __syncthreads();                                          // the copies into LDS are everybody's
+    for (int j = lo; j < hi; j += 2) {
+        const bool two = j + 1 < hi;
+        if (j != lo) {
+            fetch(j, 0);
+            if (two) fetch(j + 1, 1);
+        }
+        if (two) group_pass<2>(bk, bv, w, dst, &sh[0][0], &sh[1][0], lseb, dlb, lane);
+        else group_pass<1>(bk, bv, w, dst, &sh[0][0], &sh[1][0], lseb, dlb, lane);
     }
 }
 
@@ -656,8 +844,10 @@ __global__ __launch_bounds__(64 * kDenseUnits) void attn_kside_dense_kernel(KSid
 // serves the three K-side passes.
 struct ReduceJob {
     const f32x4* part;
-    const int* off;          // CSR offsets (sparse jobs) or nullptr (dense job)
-    const int* work;         // work list (sparse jobs)
+    const int* off;          // CSR offsets (list-driven jobs) or nullptr (dense job)
+    const int* work;         // work list (fine job); nullptr with `off`: the partial sums of unit u are slots
+                             // [off[u] << csr_shift, off[u + 1] << csr_shift) (group-major pooled jobs)
+    int csr_shift;
     bf16* dk; int64_t sdkb, sdkh, sdkn;
     bf16* dv; int64_t sdvb, sdvh, sdvn;
     int n_units, chunk, max_units;       // max_units: upper bound of units this job can have per (b,h)
@@ -725,6 +915,13 @@ __global__ __launch_bounds__(256) void kside_reduce_kernel(ReduceParams rp) {
             n = rec_n;
             first = (int64_t)bh * jb.slot_stride + rec_first;
             stride = 1;
+        } else if (jb.off != nullptr) {
+            const int* o = jb.off + (int64_t)bh * (jb.n_units + 1) + u;
+            const int o0 = o[0], o1 = o[1];
+            unit = u;
+            n = (o1 - o0) << jb.csr_shift;
+            first = (int64_t)bh * jb.slot_stride + ((int64_t)o0 << jb.csr_shift);
+            stride = 1;
         } else {
             unit = u;
             n = jb.n_chunks;
@@ -752,22 +949,37 @@ __global__ __launch_bounds__(256) void kside_reduce_kernel(ReduceParams rp) {
 
 struct DensePlan {
     int n_tok;       // tokens of the dense coarsest level per (b,h)
+    int upw;         // units per wave (1 or 2): a workgroup holds 4 * upw units
     int chunks;      // query range split
     int chunk_len;   // query blocks per chunk (even)
+    bool merged;     // the dense blocks ride on the group-major pass (one partial sum per group of 16 query blocks)
 };
 
 static DensePlan dense_plan(int B, int H, int N, int levels) {
     const int N1 = N / 16;
     DensePlan d;
     d.n_tok = (levels == 3) ? N1 / 256 : (levels == 2) ? N1 / 16 : N1;
-    const int groups = (d.n_tok / 16 / 4) * B * H;            // workgroups per piece of the query range (4 units each)
-    int chunks = (512 + groups - 1) / groups;                 // aim at two workgroups per CU
+    const int n_units = d.n_tok / 16;
+    // Q and dO are streamed n_units / (4 * upw) times (mostly out of an L2: see the kernel); four units per wave would
+    // halve that again but leave one wave per SIMD, which measured slower (1.07 ms against 0.93 ms at N = 262144)
+    d.upw = (n_units % 8 == 0 && n_units >= 16) ? 2 : 1;
+    const int groups = (n_units / (kDenseWaves * d.upw)) * B * H;   // workgroups per piece of the query range
+    // The query range is cut so that the workgroups fill the chip's resident slots (256 CUs x the workgroups the
+    // registers allow per CU) a whole number of times, three if there is that much work: a count just above a
+    // multiple of the slots leaves a last round in which a few workgroups run alone.
+    const int slots = 256 * (d.upw == 2 ? 2 : 3);
+    int chunks = 3 * slots / groups;
     if (chunks > N1 / 16) chunks = N1 / 16;
     if (chunks < 1) chunks = 1;
     int len = (N1 + chunks - 1) / chunks;
     len += len & 1;
     d.chunk_len = len;
     d.chunks = (N1 + len - 1) / len;
+    d.merged = levels >= 2 && n_units <= kGroupDenseMax;
+    if (d.merged) {
+        d.chunks = N1 / 16;
+        d.chunk_len = 16;
+    }
     return d;
 }
 
@@ -780,14 +992,15 @@ struct BwdWorkspace {
 };
 
 static BwdWorkspace bwd_workspace(int B, int H, int N, int T, int T2, int T3, int levels) {
-    const int64_t BH = (int64_t)B * H, N1 = N / 16, N2 = N1 / 16, N3 = N2 / 16;
+    const int64_t BH = (int64_t)B * H, N1 = N / 16, N2 = N1 / 16;
     const DensePlan d = dense_plan(B, H, N, levels);
     BwdWorkspace w;
     // a key block has several chunks only if it has more than `chunk` entries, so at most
     // E/chunk such blocks with at most E/chunk + E/chunk chunks in total
     w.slots_fine = 2 * (N1 * T / LLSA_CHUNK_FINE) + 2;
-    w.slots_coarse = (levels >= 2) ? 2 * (N2 * T2 / LLSA_CHUNK_COARSE) + 2 : 0;
-    w.slots_coarse2 = (levels == 3) ? 2 * (N3 * T3 / LLSA_CHUNK_COARSE2) + 2 : 0;
+    // group-major pooled passes: one partial sum per (group of 16 query blocks, entry of its ancestor's list)
+    w.slots_coarse = (levels >= 2) ? N2 * T2 : 0;
+    w.slots_coarse2 = (levels == 3) ? N2 * T3 : 0;
     int64_t o = 0;
     w.delta = o;        o += align256(BH * N * 4);
     w.dor = o;          o += align256(BH * N * 64 * 2);
@@ -822,12 +1035,12 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     } else {
         LLSA_REQUIRE(a->N % (a->levels == 3 ? 262144 : 16384) == 0, "attn_bwd: %d levels need N %% %d == 0 (N=%d)", a->levels,
                      a->levels == 3 ? 262144 : 16384, a->N);
-        LLSA_REQUIRE(a->pk2r && a->pv2r && a->pidx && a->poff && a->pflat && a->dpk2 && a->dpv2, "attn_bwd: level-2 tensors missing");
+        LLSA_REQUIRE(a->pk2r && a->pv2r && a->pidx && a->poff && a->pinv && a->dpk2 && a->dpv2, "attn_bwd: level-2 tensors missing");
         LLSA_REQUIRE(a->T2 >= 4 && a->T2 % 4 == 0 && a->T2 <= a->N / 256, "attn_bwd: topk2=%d must be a multiple of 4 and <= N/256", a->T2);
         LLSA_REQUIRE(a->w2 > 0.f, "attn_bwd: token_weight_2 must be > 0");
     }
     if (a->levels == 3) {
-        LLSA_REQUIRE(a->pk3r && a->pv3r && a->ppidx && a->ppoff && a->ppflat && a->ppwork && a->dpk3 && a->dpv3, "attn_bwd: level-3 tensors missing");
+        LLSA_REQUIRE(a->pk3r && a->pv3r && a->ppidx && a->ppoff && a->ppinv && a->dpk3 && a->dpv3, "attn_bwd: level-3 tensors missing");
         LLSA_REQUIRE(a->T3 >= 4 && a->T3 % 4 == 0 && a->T3 <= a->N / 4096, "attn_bwd: topk3=%d must be a multiple of 4 and <= N/4096", a->T3);
         LLSA_REQUIRE(a->w3 > 0.f, "attn_bwd: token_weight_3 must be > 0");
     }
@@ -841,7 +1054,9 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     const BwdWorkspace wsp = bwd_workspace(a->B, a->H, a->N, a->T, a->T2, a->T3, a->levels);
     LLSA_REQUIRE(a->workspace_bytes >= wsp.total, "attn_bwd: workspace too small (%lld < %lld)", (long long)a->workspace_bytes,
                  (long long)wsp.total);
-    LLSA_REQUIRE(a->work != nullptr && (a->levels == 1 || a->pwork != nullptr), "attn_bwd: work lists missing");
+    LLSA_REQUIRE(a->work != nullptr, "attn_bwd: work list missing");
+    LLSA_REQUIRE(a->levels == 1 || a->T2 + (a->levels == 3 ? a->T3 : 0) + kGroupDenseMax <= kGroupMaxBlocks,
+                 "attn_bwd: topk2 + topk3 must not exceed %d", kGroupMaxBlocks - kGroupDenseMax);
 
     hipStream_t s = (hipStream_t)stream;
     const int B = a->B, H = a->H, N = a->N, N1 = N / 16, N2 = N1 / 16, N3 = N2 / 16, BH = B * H;
@@ -862,7 +1077,7 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     rp.N = N;
     auto add_job = [&](const KSideParams& p, int chunk, int max_units, int n_chunks) {
         ReduceJob& j = rp.job[rp.n_jobs++];
-        j.part = p.part; j.off = p.off; j.work = p.work;
+        j.part = p.part; j.off = p.off; j.work = p.work; j.csr_shift = 0;
         j.dk = p.dk; j.sdkb = p.sdkb; j.sdkh = p.sdkh; j.sdkn = p.sdkn;
         j.dv = p.dv; j.sdvb = p.sdvb; j.sdvh = p.sdvh; j.sdvn = p.sdvn;
         j.n_units = p.n_units; j.chunk = chunk; j.max_units = max_units;
@@ -901,36 +1116,40 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
                               (a->levels >= 2) ? (const bf16*)a->dpv2 : nullptr, (const bf16*)a->freq_dk,
                               (a->levels == 3) ? (const bf16*)a->dpk3 : nullptr, (a->levels == 3) ? (const bf16*)a->dpv3 : nullptr};
         const int max_items = N1 * a->T / LLSA_CHUNK_FINE + N1;
-        hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_FINE>), dim3(max_items, BH), dim3(64), 0, s, p);
+        hipLaunchKernelGGL(attn_kside_kernel, dim3(max_items, BH), dim3(64), 0, s, p);
         add_job(p, LLSA_CHUNK_FINE, N1 * a->T / LLSA_CHUNK_FINE + 1, 0);
     };
-    auto run_sparse1 = [&]() {                                // level-1 pooled tokens, through the transposed coarse index
+    // pooled levels under an ancestor's selection, group-major (one launch for all of them, plus the dense level when it is small)
+    auto run_groups = [&]() {
         if (a->levels < 2 || !(stages & LLSA_BWD_DPKV1)) return;
-        KSideParams p = base;
-        p.kk = (const bf16*)a->pkr; p.vv = (const bf16*)a->pvr;
-        p.off = a->poff; p.flat = a->pflat; p.flat_stride = (int64_t)N2 * a->T2;
-        p.work = a->pwork; p.work_stride = llsa_work_list_len(N2, N2, a->T2, LLSA_CHUNK_COARSE);
-        p.part = (f32x4*)(ws + wsp.part_coarse); p.slot_stride = wsp.slots_coarse;
-        p.dk = (bf16*)a->dpk; p.sdkb = s1b; p.sdkh = s1h; p.sdkn = 64;
-        p.dv = (bf16*)a->dpv; p.sdvb = s1b; p.sdvh = s1h; p.sdvn = 64;
-        p.n_units = N2; p.w = a->cgw1;
-        const int max_items = N2 * a->T2 / LLSA_CHUNK_COARSE + N2;
-        hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_SPARSE1>), dim3(max_items, BH), dim3(256), 0, s, p);
-        add_job(p, LLSA_CHUNK_COARSE, N2 * a->T2 / LLSA_CHUNK_COARSE + 1, 0);
-    };
-    auto run_sparse2 = [&]() {                                // (l3) level-2 pooled tokens, through the transposed level-3 selection:
-        if (a->levels != 3 || !(stages & LLSA_BWD_DPKV1)) return;   // an entry is a grand-parent, 256 query blocks
-        KSideParams p = base;
-        p.kk = (const bf16*)a->pk2r; p.vv = (const bf16*)a->pv2r;
-        p.off = a->ppoff; p.flat = a->ppflat; p.flat_stride = (int64_t)N3 * a->T3;
-        p.work = a->ppwork; p.work_stride = llsa_work_list_len(N3, N3, a->T3, LLSA_CHUNK_COARSE2);
-        p.part = (f32x4*)(ws + wsp.part_coarse2); p.slot_stride = wsp.slots_coarse2;
-        p.dk = (bf16*)a->dpk2; p.sdkb = s2b; p.sdkh = s2h; p.sdkn = 64;
-        p.dv = (bf16*)a->dpv2; p.sdvb = s2b; p.sdvh = s2h; p.sdvn = 64;
-        p.n_units = N3; p.w = a->w2;
-        const int max_items = N3 * a->T3 / LLSA_CHUNK_COARSE2 + N3;
-        hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_kernel<MODE_SPARSE2>), dim3(max_items, BH), dim3(256), 0, s, p);
-        add_job(p, LLSA_CHUNK_COARSE2, N3 * a->T3 / LLSA_CHUNK_COARSE2 + 1, 0);
+        GroupParams g;
+        g.qr = (const bf16*)a->qr; g.dor = dor; g.lse = a->lse; g.delta = delta;
+        g.H = H; g.N = N; g.n_segs = 0; g.n_blocks = 0;
+        auto add_seg = [&](const void* kk, const void* vv, const int* sel, const int* inv, int64_t part_off, int n_units, int shift,
+                           int cnt, int64_t slots, float w) {
+            GroupSeg& sgm = g.seg[g.n_segs++];
+            sgm.kk = (const bf16*)kk; sgm.vv = (const bf16*)vv; sgm.sel = sel; sgm.inv = inv;
+            sgm.part = (f32x4*)(ws + part_off); sgm.n_units = n_units; sgm.owner_shift = shift; sgm.cnt = cnt; sgm.slots = slots; sgm.w = w;
+            g.n_blocks += cnt;
+        };
+        add_seg(a->pkr, a->pvr, a->pidx, a->pinv, wsp.part_coarse, N2, 0, a->T2, wsp.slots_coarse, a->cgw1);
+        if (a->levels == 3) add_seg(a->pk2r, a->pv2r, a->ppidx, a->ppinv, wsp.part_coarse2, N3, 4, a->T3, wsp.slots_coarse2, a->w2);
+        if (d.merged && (stages & LLSA_BWD_DENSE)) {
+            if (a->levels == 3) add_seg(a->pk3r, a->pv3r, nullptr, nullptr, wsp.part_dense, d.n_tok / 16, 0, d.n_tok / 16, 0, a->w3);
+            else add_seg(a->pk2r, a->pv2r, nullptr, nullptr, wsp.part_dense, d.n_tok / 16, 0, d.n_tok / 16, 0, a->w2);
+        }
+        hipLaunchKernelGGL(attn_kside_group_kernel, dim3(N2, BH), dim3(64 * kGroupWaves), 0, s, g);
+        auto add_csr_job = [&](const GroupSeg& sgm, const int* off, void* dk, void* dv, int64_t sb, int64_t sh) {
+            ReduceJob& j = rp.job[rp.n_jobs++];
+            j.part = sgm.part; j.off = off; j.work = nullptr; j.csr_shift = sgm.owner_shift;
+            j.dk = (bf16*)dk; j.sdkb = sb; j.sdkh = sh; j.sdkn = 64;
+            j.dv = (bf16*)dv; j.sdvb = sb; j.sdvh = sh; j.sdvn = 64;
+            j.n_units = sgm.n_units; j.chunk = 1; j.max_units = sgm.n_units;
+            j.work_stride = 0; j.slot_stride = sgm.slots; j.n_chunks = 0;
+            j.fold = PoolFold{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
+        };
+        add_csr_job(g.seg[0], a->poff, a->dpk, a->dpv, s1b, s1h);
+        if (a->levels == 3) add_csr_job(g.seg[1], a->ppoff, a->dpk2, a->dpv2, s2b, s2h);
     };
     // dense coarsest level: every unit (16 pooled tokens) meets every query block; the query
     // range is cut into d.chunks pieces whose partial sums are added afterwards
@@ -957,22 +1176,26 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
         p.off = nullptr; p.flat = nullptr; p.flat_stride = 0; p.work = nullptr; p.work_stride = 0; p.slot_stride = 0;
         p.part = (f32x4*)(ws + wsp.part_dense);
         p.n_units = d.n_tok / 16; p.chunk_len = d.chunk_len;
-        hipLaunchKernelGGL(attn_kside_dense_kernel, dim3(p.n_units / kDenseUnits, BH, d.chunks), dim3(64 * kDenseUnits), 0, s, p);
+        if (d.merged) {                                       // the group-major pass has written one partial sum per group
+            add_job(p, 1, p.n_units, d.chunks);
+            return;
+        }
+        const dim3 grid(p.n_units / (kDenseWaves * d.upw) * d.chunks, BH), block(64 * kDenseWaves);
+        if (d.upw == 2) hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_dense_kernel<2>), grid, block, 0, s, p);
+        else hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_kside_dense_kernel<1>), grid, block, 0, s, p);
         add_job(p, 1, p.n_units, d.chunks);
     };
 
     if (fold) {
         // the fine pass adds the finished pooled gradients on its way out, so they come first
-        run_sparse1();
-        run_sparse2();
+        run_groups();
         run_dense();
         run_reduce();
         run_fine();
         run_reduce();
     } else {
         run_fine();
-        run_sparse1();
-        run_sparse2();
+        run_groups();
         run_dense();
         run_reduce();
     }

@@ -256,6 +256,28 @@ __global__ __launch_bounds__(256) void sort_segments_kernel(const int* __restric
     }
 }
 
+// The inverse of the sorted lists: entry (query block q, slot t) of idx names key block n, and q sits somewhere in
+// n's ascending segment of flat -- one thread per entry finds where by bisection.  (A row that names a key block
+// twice owns one position only; both slots receive it.)
+__global__ __launch_bounds__(256) void inverse_positions_kernel(const int* __restrict__ idx, const int* __restrict__ offsets,
+                                                                const int* __restrict__ flat, int* __restrict__ inv, int Mb, int Kb,
+                                                                int T) {
+    const int e = blockIdx.x * 256 + threadIdx.x, bh = blockIdx.y;
+    const int E = Mb * T;
+    if (e >= E) return;
+    const int q = e / T;
+    const int n = clampi(idx[(int64_t)bh * E + e], 0, Kb - 1);
+    const int* o = offsets + (int64_t)bh * (Kb + 1) + n;
+    const int* f = flat + (int64_t)bh * E;
+    int lo = o[0], hi = o[1] - 1;                             // the segment holds q: it is never empty
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (f[mid] < q) lo = mid + 1;
+        else hi = mid;
+    }
+    inv[(int64_t)bh * E + e] = clampi(lo, 0, E - 1);
+}
+
 }  // namespace llsa
 
 using namespace llsa;
@@ -266,8 +288,8 @@ extern "C" int64_t llsa_work_list_len(int Mb, int Kb, int T, int chunk) {
     return 4 + 4 * (e / chunk + Kb) + 4 * (e / chunk + 1) + work_tail_len(Kb);
 }
 
-extern "C" int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, int32_t* work, int B, int H, int Mb,
-                                      int Kb, int T, int chunk, void* stream) {
+extern "C" int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, int32_t* work, int32_t* inv, int B, int H,
+                                      int Mb, int Kb, int T, int chunk, void* stream) {
     LLSA_REQUIRE(idx && offsets && flat, "transpose_indices: null argument");
     LLSA_REQUIRE(B > 0 && H > 0 && Mb > 0 && Kb > 0 && T > 0, "transpose_indices: bad shape");
     LLSA_REQUIRE(work == nullptr || chunk >= 1, "transpose_indices: work list needs chunk >= 1");
@@ -300,5 +322,8 @@ extern "C" int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int3
     }
     hipLaunchKernelGGL(sort_segments_kernel, dim3((Kb + 3) / 4, B * H), dim3(256), lds_sort, (hipStream_t)stream,
                        (const int*)offsets, flat, Mb, Kb, T);
+    if (inv != nullptr)
+        hipLaunchKernelGGL(inverse_positions_kernel, dim3((unsigned)((E + 255) / 256), B * H), dim3(256), 0, (hipStream_t)stream, idx,
+                           (const int*)offsets, (const int*)flat, inv, Mb, Kb, T);
     return launch_status("transpose_indices");
 }

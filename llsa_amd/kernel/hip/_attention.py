@@ -6,7 +6,7 @@ from typing import Optional
 
 import torch
 
-from ..._lib import CHUNK_COARSE, CHUNK_FINE, AttnBwdArgs, AttnFwdArgs
+from ..._lib import CHUNK_FINE, AttnBwdArgs, AttnFwdArgs
 from ._common import BLOCK, as_rows, lib_for, ptr, require_bf16, require_head_dim, s3, stream_of
 from .indices_transpose import transpose_indices
 
@@ -111,14 +111,14 @@ def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_wei
     idx = indices.to(torch.int32).contiguous()
     if levels == 2:
         pidx = p_indices.to(torch.int32).contiguous()
-    if csr is not None:                       # (off, flat, work[, poff, pflat, pwork]) from transpose_indices
+    if csr is not None:                       # (off, flat, work[, poff, pflat, pinv]) from transpose_indices
         off, flat, work = csr[:3]
         if levels == 2:
-            poff, pflat, pwork = csr[3:6]
+            poff, _, pinv = csr[3:6]
     else:
         off, flat, work = transpose_indices(idx, N // BLOCK, CHUNK_FINE)
         if levels == 2:
-            poff, pflat, pwork = transpose_indices(pidx, N // (BLOCK * BLOCK), CHUNK_COARSE)
+            poff, _, pinv = transpose_indices(pidx, N // (BLOCK * BLOCK), inverse=True)
     mk = lambda t: torch.empty_like(t) if rows_ok8(t) else torch.empty(t.shape, device=t.device, dtype=t.dtype)
     dq, dk, dv = mk(q), mk(k), mk(v)
     dpk, dpv = torch.empty_like(pk, memory_format=torch.contiguous_format), torch.empty_like(pv, memory_format=torch.contiguous_format)
@@ -142,7 +142,7 @@ def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_wei
         dpv2 = torch.empty_like(pv2, memory_format=torch.contiguous_format)
         for n in ("pk2r", "pv2r"):
             setattr(a, n, tl[n].data_ptr())
-        a.pidx, a.poff, a.pflat, a.pwork = pidx.data_ptr(), poff.data_ptr(), pflat.data_ptr(), pwork.data_ptr()
+        a.pidx, a.poff, a.pinv = pidx.data_ptr(), poff.data_ptr(), pinv.data_ptr()
         a.dpk2, a.dpv2 = dpk2.data_ptr(), dpv2.data_ptr()
         outs += [dpk2, dpv2]
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws_bytes

@@ -21,7 +21,7 @@ import ctypes as C
 import torch
 from torch.autograd import Function
 
-from ..._lib import CHUNK_COARSE, CHUNK_COARSE2, CHUNK_FINE, AttnBwdArgs, AttnFwdArgs, PoolItem, current_lib
+from ..._lib import CHUNK_FINE, AttnBwdArgs, AttnFwdArgs, PoolItem, current_lib
 
 _side = {}          # device -> (second stream, two events)
 _SIDE_STREAM_MIN_TOKENS = 1 << 17
@@ -77,14 +77,12 @@ class _Layout:
             return at
 
         self.wl_f = lib.work_list_len(n1, n1, T, CHUNK_FINE)
-        self.wl_c = lib.work_list_len(n2, n2, T2, CHUNK_COARSE) if l2 else 0
-        self.wl_c2 = lib.work_list_len(n3, n3, T3, CHUNK_COARSE2) if l3 else 0
         self.idx, self.pidx, self.ppidx = take_i(n1 * T), take_i(n2 * T2, l2), take_i(n3 * T3, l3)
         self.off, self.flat, self.work = take_i(n1 + 1, grad), take_i(n1 * T, grad), take_i(self.wl_f, grad)
-        self.poff, self.pflat, self.pwork = (take_i(n2 + 1, grad and l2), take_i(n2 * T2, grad and l2),
-                                             take_i(self.wl_c, grad and l2))
-        self.ppoff, self.ppflat, self.ppwork = (take_i(n3 + 1, grad and l3), take_i(n3 * T3, grad and l3),
-                                                take_i(self.wl_c2, grad and l3))
+        self.poff, self.pflat, self.pinv = (take_i(n2 + 1, grad and l2), take_i(n2 * T2, grad and l2),
+                                            take_i(n2 * T2, grad and l2))
+        self.ppoff, self.ppflat, self.ppinv = (take_i(n3 + 1, grad and l3), take_i(n3 * T3, grad and l3),
+                                               take_i(n3 * T3, grad and l3))
         self.n_i32 = o
         # backward arena (bytes): pooled gradients, then the kernels' workspace
         self.ws_bytes = lib.attn_bwd_workspace_bytes(B, H, N, T, T2, T3, levels)
@@ -235,14 +233,14 @@ class LlsaFused(Function):
             if side is not None:
                 side.wait_event(ev_idx)         # (the arena is older than the selection, so this covers it too)
                 s_lists = C.c_void_p(side.cuda_stream)
-            _check(lib, lib.transpose_indices(pi(lay.idx), pi(lay.off), pi(lay.flat), pi(lay.work), B, H, n1, n1, T, CHUNK_FINE,
+            _check(lib, lib.transpose_indices(pi(lay.idx), pi(lay.off), pi(lay.flat), pi(lay.work), None, B, H, n1, n1, T, CHUNK_FINE,
                                               s_lists), "transpose_indices")
             if l2:
-                _check(lib, lib.transpose_indices(pi(lay.pidx), pi(lay.poff), pi(lay.pflat), pi(lay.pwork), B, H, n2, n2, T2,
-                                                  CHUNK_COARSE, s_lists), "transpose_indices (coarse)")
+                _check(lib, lib.transpose_indices(pi(lay.pidx), pi(lay.poff), pi(lay.pflat), None, pi(lay.pinv), B, H, n2, n2, T2,
+                                                  1, s_lists), "transpose_indices (coarse)")
             if l3:
-                _check(lib, lib.transpose_indices(pi(lay.ppidx), pi(lay.ppoff), pi(lay.ppflat), pi(lay.ppwork), B, H, n3, n3, T3,
-                                                  CHUNK_COARSE2, s_lists), "transpose_indices (level 3)")
+                _check(lib, lib.transpose_indices(pi(lay.ppidx), pi(lay.ppoff), pi(lay.ppflat), None, pi(lay.ppinv), B, H, n3, n3, T3,
+                                                  1, s_lists), "transpose_indices (level 3)")
             if side is not None:
                 ev_lists.record(side)
                 cur.wait_event(ev_lists)
@@ -283,7 +281,7 @@ class LlsaFused(Function):
         a.pk2r, a.pv2r = pa(lay.pk2r), pa(lay.pv2r)
         a.idx, a.pidx = pi(lay.idx), pi(lay.pidx)
         a.off, a.flat, a.work = pi(lay.off), pi(lay.flat), pi(lay.work)
-        a.poff, a.pflat, a.pwork = pi(lay.poff), pi(lay.pflat), pi(lay.pwork)
+        a.poff, a.pinv = pi(lay.poff), pi(lay.pinv)
         a.dq, a.sdqb, a.sdqh, a.sdqn = dq.data_ptr(), dq.stride(0), dq.stride(1), dq.stride(2)
         a.dk, a.sdkb, a.sdkh, a.sdkn = dk.data_ptr(), dk.stride(0), dk.stride(1), dk.stride(2)
         a.dv, a.sdvb, a.sdvh, a.sdvn = dv.data_ptr(), dv.stride(0), dv.stride(1), dv.stride(2)
@@ -292,7 +290,7 @@ class LlsaFused(Function):
             a.dpk2, a.dpv2 = w0 + lay.dpk2, w0 + lay.dpv2
         if levels == 3:
             a.pk3r, a.pv3r, a.ppidx = pa(lay.pk3r), pa(lay.pv3r), pi(lay.ppidx)
-            a.ppoff, a.ppflat, a.ppwork = pi(lay.ppoff), pi(lay.ppflat), pi(lay.ppwork)
+            a.ppoff, a.ppinv = pi(lay.ppoff), pi(lay.ppinv)
             a.dpk3, a.dpv3, a.T3, a.w3 = w0 + lay.dpk3, w0 + lay.dpv3, T3, 4096.0
         a.workspace, a.workspace_bytes = w0 + lay.ws, lay.ws_bytes
         if freq is not None:

@@ -194,10 +194,16 @@ def check_transpose(dev, B=2, H=2, Mb=64, T=8, Kb=None, chunk=0):
     g = torch.Generator().manual_seed(12)
     kb = Kb or Mb
     idx = torch.stack([torch.randperm(kb, generator=g)[:T] for _ in range(B * H * Mb)]).reshape(B, H, Mb, T).int()
-    off, flat = transpose_indices(idx.to(dev), Kb, chunk)[:2]
+    res = transpose_indices(idx.to(dev), Kb, chunk, inverse=True)
+    off, flat, inv = res[0], res[1], res[-1].cpu().long()
     ro, rf = O.transpose_indices(idx.long(), Kb)
     assert torch.equal(off.cpu().long(), ro), "offsets differ"
     assert torch.equal(flat.cpu().long(), rf), "flat list differs"
+    # the inverse: entry (q, t) sits at a position of the segment of key block idx[q, t], and that position holds q
+    qid = torch.arange(Mb).view(1, 1, Mb, 1).expand(B, H, Mb, T)
+    assert torch.equal(torch.gather(rf, -1, inv.reshape(B, H, -1)).reshape(B, H, Mb, T), qid), "inverse positions do not hold their query block"
+    lo, hi = torch.gather(ro, -1, idx.long().reshape(B, H, -1)), torch.gather(ro, -1, idx.long().reshape(B, H, -1) + 1)
+    assert ((inv.reshape(B, H, -1) >= lo) & (inv.reshape(B, H, -1) < hi)).all(), "inverse position outside its key block's segment"
 
 
 def check_transpose_hot_block(dev):
