@@ -516,7 +516,7 @@ __global__ __launch_bounds__(64 * kDenseWaves) void attn_kside_dense_kernel(KSid
     const int bh = lid / (int)gridDim.x;
     const int unit0 = (((lid % (int)gridDim.x) % unit_groups) * kDenseWaves + wave) * UPW;   // + UPW <= n_units (the plan sees to it)
     const int start = piece * p.chunk_len;
-    const int n_pairs = min(p.chunk_len, N1 - start) / 2;     // chunk_len and N1 are even
+    const int n_pairs = min(p.chunk_len, N1 - start) / 2;     // even: chunk_len and N1 are multiples of 4
     if (n_pairs <= 0) return;                                 // uniform over the workgroup
     const bf16* qrb = p.qr + ((int64_t)bh * N1 + start) * kTile;
     const bf16* dorb = p.dor + ((int64_t)bh * N1 + start) * kTile;
@@ -532,7 +532,10 @@ __global__ __launch_bounds__(64 * kDenseWaves) void attn_kside_dense_kernel(KSid
         const bf16* src = ((wave & 1) ? dorb : qrb) + (int64_t)(2 * t + (wave >> 1)) * kTile;
         st.a = ld16(src + lane * 8);
         st.b = ld16(src + 512 + lane * 8);
-        if (stat_lane) st.s = *reinterpret_cast<const f32x4*>((lane < 8 ? lseb : dlb) + 2 * t * kBlk + (lane & 7) * 4);
+        // (every lane of every wave loads, lanes 16.. the same as lane % 16: a load inside a branch makes the compiler lose
+        // count of the loads in flight, after which it waits for all of them in every round)
+        const int sl = lane & 15;
+        st.s = *reinterpret_cast<const f32x4*>((sl < 8 ? lseb : dlb) + 2 * t * kBlk + (sl & 7) * 4);
     };
     auto deposit = [&](int t, const Stage& st) __attribute__((always_inline)) {
         bf16* dst = &sh[t & 1][wave * kTile];
@@ -618,9 +621,11 @@ __global__ __launch_bounds__(64 * kDenseWaves) void attn_kside_dense_kernel(KSid
             }
         }
     };
+    // (two rounds per trip without a branch between them: n_pairs is even, and with a conditional second round the
+    // compiler loses count of the loads in flight where the loop closes and waits for all of them)
     for (int t = 0; t < n_pairs; t += 2) {
         round(t, s1);
-        if (t + 1 < n_pairs) round(t + 1, s0);
+        round(t + 1, s0);
     }
 #pragma unroll
     for (int j = 0; j < UPW; j++) {
@@ -951,7 +956,7 @@ struct DensePlan {
     int n_tok;       // tokens of the dense coarsest level per (b,h)
     int upw;         // units per wave (1 or 2): a workgroup holds 4 * upw units
     int chunks;      // query range split
-    int chunk_len;   // query blocks per chunk (even)
+    int chunk_len;   // query blocks per chunk (a multiple of 4)
     bool merged;     // the dense blocks ride on the group-major pass (one partial sum per group of 16 query blocks)
 };
 
@@ -972,7 +977,7 @@ static DensePlan dense_plan(int B, int H, int N, int levels) {
     if (chunks > N1 / 16) chunks = N1 / 16;
     if (chunks < 1) chunks = 1;
     int len = (N1 + chunks - 1) / chunks;
-    len += len & 1;
+    len = (len + 3) & ~3;
     d.chunk_len = len;
     d.chunks = (N1 + len - 1) / len;
     d.merged = levels >= 2 && n_units <= kGroupDenseMax;
