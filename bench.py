@@ -10,11 +10,17 @@ applied in-kernel, smooth-field inputs, dO ~ N(0,1).
 
 One JSON line is printed:
   value        effective TFLOP/s = 14*B*H*N*D*n_kv / step time (algorithmic FLOPs: forward 4, backward 10)
-  ms_per_step  forward + backward wall time per step
-  roofline     the dominant kernel of the step, timed with HIP events on the launch stream in a
-               second pass that runs the same kernels stage by stage
-  cpu_baseline the CPU oracle (plain PyTorch restatement) on the host cores, same workload in fp32
-  kernels      per-stage times of that second pass (ms), with the achieved rate of each
+  ms_per_step  forward + backward wall time per step (K steps between two synchronisations)
+  step_event_times  median and 20 % / 80 % quantiles of per-step HIP-event times (>= 50 steps), the statistics
+               the reference's harness reports
+  roofline     the slowest MFMA kernel of the step, timed with HIP events on the launch stream in a
+               second pass that runs the same kernels stage by stage; `traffic` = its HBM-side bytes per
+               launch as the committed rocprofv3 summary named in `traffic_source` holds them
+  roofline_hbm the pooling pyramid (the q, k, v launch) against the HBM peak, on its algorithmic bytes
+  cpu_baseline the CPU oracle (plain PyTorch restatement) on the host cores, same workload in fp32, and
+               under `c1` benchmark configuration 1 (llsa_l1 forward, fp32, N = 1024), median of 10
+  kernels      per-stage times of that second pass (ms), with the achieved rate of each (TFLOP/s on
+               algorithmic FLOPs for the attention kernels, GB/s on algorithmic bytes for the others)
   dense_sdpa   F.scaled_dot_product_attention forward+backward on the same shapes, same GPU
 
 --workload c4 times something else, one training step of the operator's caller (a pixel DiT-S with
@@ -36,13 +42,34 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 
-# HBM-side bytes per launch (L2 <-> fabric reads + writes) measured with rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE on this command, each scaled by what the same counter reads for a 256 MiB elementwise
-# copy (fetch x2.000, write x1.000); the tables they come from are profiles/step_kernels_<workload>_hbm_traffic.txt
-MEASURED_TRAFFIC = {
-    "c3": {"attn_fwd": 129689497, "bwd_dq": 249972361, "bwd_dkv": 302121348, "bwd_dpkv1_sparse": 190617560,
-           "bwd_dpkv_dense": 69261766, "pool_pyramid": 95573151},
-}
+# HBM-side bytes per launch (L2 <-> fabric, reads + writes) come from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# summaries under profiles/ (each counter scaled by what it reads for a 256 MiB elementwise copy; the files say how):
+# the table of the workload is parsed at run time, so the figure printed is the one the committed profile holds.
+TRAFFIC_KERNELS = {"attn_fwd": "attn_fwd_kernel", "bwd_dq": "attn_dq_kernel", "bwd_dkv": "attn_kside_kernel",
+                   "bwd_pooled_groups": "attn_kside_group_kernel", "bwd_dpkv_dense": "attn_kside_dense_kernel",
+                   "pool_pyramid": "pool_pyramid_kernel", "topk_sparse": "topk_sparse_kernel", "topk_dense": "topk_dense_radix_kernel"}
+
+
+def measured_traffic(workload):
+    """{stage: bytes per launch} and the file they were read from (None, None if the profile is missing)."""
+    path = os.path.join(ROOT, "profiles", f"step_kernels_{workload}_hbm_traffic.txt")
+    if not os.path.exists(path):
+        return {}, None
+    rows = {}
+    for line in open(path):
+        parts = line.split()
+        if len(parts) >= 7 and parts[0].startswith("llsa::"):
+            try:
+                rows[parts[0]] = (float(parts[-3]) + float(parts[-2])) * 1e6       # read_MB + write_MB
+            except ValueError:
+                pass
+    out = {}
+    for stage, kern in TRAFFIC_KERNELS.items():
+        for name, val in rows.items():
+            if name.split("<")[0] == "llsa::" + kern or name.startswith("llsa::" + kern + "<"):
+                out.setdefault(stage, val)        # (the first row of a kernel is its largest dispatch shape)
+    return out, os.path.relpath(path, ROOT)
+
 
 WORKLOADS = {
     # name: (op, B, H, N, topk1, topk2, rope)
@@ -134,18 +161,21 @@ def stage_profile(op, q, k, v, do, t1, t2, freq, iters, torch):
     # as the fused operator calls it: pooled gradients folded into dk / dv by the fine pass
     run = lambda st: A.attn_bwd(do, q, k, v, pk, pv, o, lse, idx, 16.0, cgw, stages=st, freq_dq=freq, fold_pooled=True,
                                 freq_dk=freq, **bkw)
-    run(2)
+    run(0)
     NO_REDUCE = 32
-    for name, st in (("bwd_dq", 2), ("bwd_dpkv1_sparse", 8 | NO_REDUCE), ("bwd_dpkv_dense", 16 | NO_REDUCE),
-                     ("bwd_dkv", 4 | NO_REDUCE)):
-        if (st & 8) and not l2:
-            continue
-        # a stage run alone reads whatever workspace the allocator hands back (the block the dq stage
-        # just filled with delta and the dO tiles); only its duration is used
+    # l2 at this size: the dense coarsest level rides on the group-major pass of the pooled levels (stage bits 8 | 16)
+    merged = l2 and (N // 4096) <= 8
+    stages = [("bwd_dq", 2), ("bwd_dkv", 4 | NO_REDUCE)]
+    if l2:
+        stages.append(("bwd_pooled_groups", (8 | 16 | NO_REDUCE) if merged else (8 | NO_REDUCE)))
+    if not merged:
+        stages.append(("bwd_dpkv_dense", 16 | NO_REDUCE))
+    for name, st in stages:
+        # a stage run alone reads whatever workspace the allocator hands back (the block the complete call
+        # above filled with delta and the dO tiles); only its duration is used
         res[name] = timed(lambda: run(st), iters, torch)
-    # the two launches that add up the partial sums of the K-side passes
-    res["bwd_reduce"] = max(0.0, timed(lambda: run(4 | 8 | 16), iters, torch) - res["bwd_dkv"] - res["bwd_dpkv_dense"]
-                            - res.get("bwd_dpkv1_sparse", 0.0))
+    # the K-side passes with the launches that add up their partial sums, in one piece (no difference of timings)
+    res["bwd_kside_all_with_reductions"] = timed(lambda: run(4 | 8 | 16), iters, torch)
     return res
 
 
@@ -182,7 +212,29 @@ def cpu_baseline(op, B, H, N, D, t1, t2, rope):
     flops = 14.0 * Bs * Hs * N * D * n_kv(op, N, t1, t2)
     return {"value": flops / t_best / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"oracle llsa_{op} fwd+bwd fp32, B={Bs} H={Hs} N={N} (best of {reps}), {t_best * 1e3:.0f} ms",
-            "ms": t_best * 1e3}
+            "ms": t_best * 1e3, "c1": cpu_baseline_c1()}
+
+
+def cpu_baseline_c1():
+    """Benchmark configuration 1, the reference's own CPU-runnable case: llsa_l1 forward in fp32, B=1, H=6, N=1024
+    (32 x 32 tokens in Z-order), D=64, block_size 16, topk 8, q, k, v ~ N(0,1) from seed 0; median of 10 runs of the
+    oracle on the host cores.  (Of the reference only gen_sparse_indices, topk.py:6-9, is plain PyTorch; the oracle
+    restates the rest of the path.)"""
+    import torch
+    from oracle import llsa_oracle as O
+    g = torch.Generator().manual_seed(0)
+    q, k, v = (torch.randn(1, 6, 1024, 64, generator=g) for _ in range(3))
+    O.llsa_l1_fwd(q, k, v, 8, 16)
+    times = []
+    for _ in range(10):
+        t0 = time.perf_counter()
+        O.llsa_l1_fwd(q, k, v, 8, 16)
+        times.append((time.perf_counter() - t0) * 1e3)
+    times.sort()
+    med = 0.5 * (times[4] + times[5])
+    flops = 4.0 * 6 * 1024 * 64 * n_kv("l1", 1024, 8, 0)
+    return {"workload": "c1: llsa_l1 forward fp32 B=1 H=6 N=1024 D=64 topk=8, N(0,1) seed 0", "ms_median_of_10": med,
+            "ms_min": times[0], "gflops": flops / (med * 1e-3) / 1e9, "cores": torch.get_num_threads(), "kind": "port"}
 
 
 def bench_dit(args):
@@ -306,9 +358,6 @@ def main():
     ap.add_argument("--workload", default="c3", choices=sorted(WORKLOADS) + ["c4", "fwd_sweep"])
     ap.add_argument("--no-extras", action="store_true", help="skip stage profile, CPU baseline and dense SDPA")
     ap.add_argument("--unfused", action="store_true", help="use the reference's composition (separate pools, autograd adds)")
-    ap.add_argument("--graph", action="store_true",
-                    help="also capture the step in one HIP graph (llsa_amd.GraphedStep) and time its replay; "
-                         "reported as ms_per_step_graph next to the eager figure, which stays `value`")
     ap.add_argument("--calibrate", action="store_true",
                     help="after the timed region also launch a plain elementwise copy of 256 MiB (fp32, read 256 MiB + "
                          "write 256 MiB) five times, so that a counter profile of this command holds a kernel of known "
@@ -357,14 +406,24 @@ def main():
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) * 1e3 / args.steps
 
-    # `value` is the step as a user's training loop issues it: ~25 launches from Python.  With --graph
-    # the same step is also replayed from one captured HIP graph (one call per step; the host time of
-    # the separate launches is about what the kernels take at these sizes).
+    # `value` is the step as a user's training loop issues it: ~25 launches from Python.
     ms = time_steps(eager_step)
-    ms_graph = None
-    if args.graph:
-        graphed = llsa_amd.GraphedStep(fwd, [q, k, v], do)
-        ms_graph = time_steps(graphed.replay)
+
+    def step_quantiles(step, n):
+        """Per-step times from HIP events on the launch stream (every step is fenced by two events; the lists that run
+        on the second stream are joined back before the step's last kernel): median and 20 % / 80 % quantiles, the
+        statistics the reference's harness reports (test_kernel.py:45-51)."""
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(n + 1)]
+        ev[0].record()
+        for i in range(n):
+            step()
+            ev[i + 1].record()
+        ev[n].synchronize()
+        t = torch.tensor([ev[i].elapsed_time(ev[i + 1]) for i in range(n)], dtype=torch.float64)
+        return {"n": n, "ms_median": t.median().item(), "ms_p20": t.quantile(0.2).item(), "ms_p80": t.quantile(0.8).item(),
+                "ms_mean": t.mean().item()}
+
+    quant = step_quantiles(eager_step, max(50, args.steps))
 
     if args.calibrate:
         src = torch.ones(64 * 1024 * 1024, device=dev, dtype=torch.float32)
@@ -387,7 +446,7 @@ def main():
                                + (" (unfused composition)" if args.unfused else ""),
                    "n_kv_per_query": nkv, "algorithmic_gflop": flops / 1e9},
         "frac_of_bf16_mfma_peak": flops / (ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
-        "ms_per_step_graph": ms_graph,
+        "step_event_times": quant,
     }
 
     if not args.no_extras and op != "l3":      # (the stage profile and the CPU baseline know one and two levels)
@@ -395,15 +454,26 @@ def main():
         with torch.no_grad():
             st = stage_profile(op, q.detach(), k.detach(), v.detach(), do, t1, t2, freq, prof_iters, torch)
         alg = {"attn_fwd": 4.0 * unit_flops, "bwd_dq": 6.0 * unit_flops, "bwd_dkv": 4.0 * B * H * N * D * 16 * t1}
+        n_dense = N // 256 if op == "l2" else N // 16
         if op == "l2":
-            alg["bwd_dpkv1_sparse"] = 4.0 * B * H * N * D * 16 * t2
-            alg["bwd_dpkv_dense"] = 4.0 * B * H * N * D * (N // 256)
-        else:
-            alg["bwd_dpkv_dense"] = 4.0 * B * H * N * D * (N // 16)
+            merged = "bwd_dpkv_dense" not in st
+            alg["bwd_pooled_groups"] = 4.0 * B * H * N * D * (16 * t2 + (n_dense if merged else 0))
+        if "bwd_dpkv_dense" in st:
+            alg["bwd_dpkv_dense"] = 4.0 * B * H * N * D * n_dense
+        # algorithmic bytes of the bandwidth-bound kernels: inputs read once, results written once (bf16 = 2 B, indices 4 B)
         el = 2 * B * H * N * D
+        BH, n1, n2 = B * H, N // 16, N // 256
         hbm = {"pool_pyramid": 3 * el * (1 + 1 / 16 + (1 / 256 if op == "l2" else 0))}
         # (the pooling kernel also writes the operand tiles the attention kernels read; those bytes
         # are layout work of this implementation and are not counted as algorithmic)
+        if op == "l2":
+            hbm["topk_dense"] = BH * (2 * n2 * D * 2 + n2 * t2 * 4)
+            hbm["topk_sparse"] = BH * (2 * n1 * D * 2 + n2 * t2 * 4 + n1 * t1 * 4)
+            hbm["transpose_indices"] = BH * ((n1 * t1 * 4) * 2 + (n1 + 1) * 4 + (n2 * t2 * 4) * 3 + (n2 + 1) * 4)
+        else:
+            hbm["topk_dense"] = BH * (2 * n1 * D * 2 + n1 * t1 * 4)
+            hbm["transpose_indices"] = BH * ((n1 * t1 * 4) * 2 + (n1 + 1) * 4)
+        traffic, traffic_src = measured_traffic(args.workload)
         kernels = {}
         for name, t in st.items():
             e = {"ms": t}
@@ -411,19 +481,22 @@ def main():
                 e["tflops"] = alg[name] / (t * 1e-3) / 1e12
                 e["frac_mfma_peak"] = e["tflops"] / PEAK_BF16_TFLOPS
             if name in hbm:
+                e["algorithmic_mb"] = hbm[name] / 1e6
                 e["gbs"] = hbm[name] / (t * 1e-3) / 1e9
                 e["frac_hbm_peak"] = e["gbs"] / PEAK_HBM_GBS
+            if name in traffic:
+                e["hbm_traffic_mb"] = traffic[name] / 1e6
             kernels[name] = e
         out["kernels"] = kernels
-        out["stage_sum_ms"] = sum(st.values())
+        out["stage_sum_ms"] = sum(t for n_, t in st.items() if n_ != "bwd_kside_all_with_reductions")
         dom = max(alg, key=lambda n: st[n])
         out["roofline"] = {"kernel": dom, "bound": "mfma", "achieved": kernels[dom]["tflops"], "peak": PEAK_BF16_TFLOPS,
                            "unit": "TFLOP/s", "frac": kernels[dom]["frac_mfma_peak"],
-                           "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get(dom),
+                           "traffic": traffic.get(dom), "traffic_source": traffic_src,
                            "avg_launch_ms": st[dom], "algorithmic_gflop_per_launch": alg[dom] / 1e9}
-        out["roofline_hbm"] = {"kernel": "pool_pyramid", "bound": "hbm", "achieved": kernels["pool_pyramid"]["gbs"],
+        out["roofline_hbm"] = {"kernel": "pool_pyramid (the q, k, v launch)", "bound": "hbm", "achieved": kernels["pool_pyramid"]["gbs"],
                                "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": kernels["pool_pyramid"]["frac_hbm_peak"],
-                               "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("pool_pyramid")}
+                               "traffic": traffic.get("pool_pyramid"), "traffic_source": traffic_src}
         # dense attention on the same GPU
         try:
             import torch.nn.functional as F

@@ -44,7 +44,8 @@ extern "C" {
 #define LLSA_DTYPE_BF16 0
 #define LLSA_DTYPE_F32 1
 
-int llsa_version(void);
+#define LLSA_ABI_VERSION 200     /* changes with every change of a signature or argument structure below */
+int llsa_version(void);          /* LLSA_ABI_VERSION of the built library                                    */
 const char* llsa_last_error_string(void);
 
 /* ------------------------------------------------------------------------------------------
@@ -259,6 +260,10 @@ typedef struct llsa_attn_bwd_args {
     float w3;
 } llsa_attn_bwd_args;
 
+/* `stages` is a diagnostic for timing kernels one at a time: a mask other than 0 launches only the named kernels.
+ * Every stage but LLSA_BWD_DQ reads what that stage left in the workspace (delta, the R tiles of dout), and the
+ * reductions read partial sums the K-side stages left there: a mask is only meaningful on a workspace that a
+ * complete call (stages = 0) with the same arguments has filled before, and only its duration is of use. */
 #define LLSA_BWD_DQ 2       /* dq; also delta = rowsum(o * dout) and the R tiles of dout, which the
                                stages below read from the workspace                              */
 #define LLSA_BWD_DKV 4      /* dK/dV of the fine tokens                                          */

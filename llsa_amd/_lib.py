@@ -86,6 +86,7 @@ _SIGNATURES = {
 
 EXPORTS = tuple(_SIGNATURES)
 CHUNK_FINE = 64                                             # LLSA_CHUNK_FINE of include/llsa_hip.h
+ABI_VERSION = 200                                           # LLSA_ABI_VERSION
 STATIC_PARTIALS_MAX = 262144                                # LLSA_STATIC_PARTIALS_MAX
 
 
@@ -109,6 +110,9 @@ class Lib:
             fn.restype = res
             fn.argtypes = args
             setattr(self, name[len("llsa_"):], fn)
+        if self.version() != ABI_VERSION:      # a library built from other sources than this binding describes
+            raise ImportError(f"{path} has ABI version {self.version()}, this package needs {ABI_VERSION}: rebuild it "
+                              "(python -m llsa_amd.build)")
 
     def check(self, rc: int, what: str):
         if rc != 0:

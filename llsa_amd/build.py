@@ -29,9 +29,6 @@ FLAGS = [
 ]
 
 
-FLAGS += os.environ.get("LLSA_EXTRA_HIPCC_FLAGS", "").split()      # e.g. -DLLSA_FWD_NB=4 for tuning experiments
-
-
 def sources():
     return sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
 

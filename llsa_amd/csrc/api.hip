@@ -9,5 +9,6 @@ char* error_buffer() {
 }
 }  // namespace llsa
 
-extern "C" int llsa_version(void) { return 100; }
+// bumped whenever an argument structure or a signature of include/llsa_hip.h changes; the Python binding checks it
+extern "C" int llsa_version(void) { return LLSA_ABI_VERSION; }
 extern "C" const char* llsa_last_error_string(void) { return llsa::error_buffer(); }

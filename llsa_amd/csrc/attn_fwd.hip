@@ -19,13 +19,10 @@
 #include "llsa_host.h"
 #include "../../include/llsa_hip.h"
 
-#ifndef LLSA_FWD_NB
-#define LLSA_FWD_NB 2          // 16-key blocks per pipeline step (2 or 4)
-#endif
-
 namespace llsa {
 
 constexpr float kMaxSlack = 8.f;     // log2 units
+constexpr int NB = 2;                // 16-key blocks per pipeline step: 32 keys, one K step of the second product
 
 struct SoftmaxState {
     float m2;        // reference point of the exponentials (at most kMaxSlack below the running max), log2 units
@@ -34,22 +31,19 @@ struct SoftmaxState {
 };
 
 // Operands of one step = NB 16-key blocks, as they sit in registers between load and use.
-template <int NB>
 struct KvRegs {
     bf16x8 k[NB][2];     // K rows (R tile): block j, channel half
     bf16x4 v[NB][4];     // V (T tile): block j, channel tile dt, keys 4*(l/16)..+3
 };
 
 // Where one step's blocks live: kb[j] is the R tile of key block j, vtb[j] the T tile of its values.
-template <int NB>
 struct StepDesc {
     const bf16* kb[NB];
     const bf16* vtb[NB];
     float wratio;        // weight(previous segment) / weight(this segment) on the first step of a segment
 };
 
-template <int NB>
-__device__ __forceinline__ void load_step(KvRegs<NB>& t, const StepDesc<NB>& d, int lane) {
+__device__ __forceinline__ void load_step(KvRegs& t, const StepDesc& d, int lane) {
 #pragma unroll
     for (int j = 0; j < NB; j++) {
         t.k[j][0] = ld16(d.kb[j] + lane * 8);
@@ -61,8 +55,7 @@ __device__ __forceinline__ void load_step(KvRegs<NB>& t, const StepDesc<NB>& d, 
         for (int dt = 0; dt < 4; dt++) t.v[j][dt] = ld8(d.vtb[j] + dt * 256 + lane * 4);
 }
 
-template <int NB>
-__device__ __forceinline__ void compute_step(SoftmaxState& st, const bf16x8 bq[2], const KvRegs<NB>& t, float wratio) {
+__device__ __forceinline__ void compute_step(SoftmaxState& st, const bf16x8 bq[2], const KvRegs& t, float wratio) {
     f32x4 s[NB];
 #pragma unroll
     for (int j = 0; j < NB; j++) {
@@ -108,8 +101,7 @@ __device__ __forceinline__ void compute_step(SoftmaxState& st, const bf16x8 bq[2
 
 // Operands of one step out of the workgroup's LDS copy of shared blocks (4 KB per block: R tile
 // of the keys, then T tile of the values).
-template <int NB>
-__device__ __forceinline__ void load_step_lds(KvRegs<NB>& t, const bf16* blocks, int lane) {
+__device__ __forceinline__ void load_step_lds(KvRegs& t, const bf16* blocks, int lane) {
 #pragma unroll
     for (int j = 0; j < NB; j++) {
         t.k[j][0] = lds_ld16(blocks + j * 2 * kTile + lane * 8);
@@ -133,9 +125,8 @@ __device__ __forceinline__ void load_step_lds(KvRegs<NB>& t, const bf16* blocks,
 // the whole vector-memory queue at every wait while a copy into LDS is outstanding, which would
 // undo the register ping-pong.  This is what bounds the kernel: without the sharing every wave
 // pulls all of its 4 KB per block through the L2, and the L2's bandwidth, not the MFMA, sets the time.
-template <int NB>
 __global__ __launch_bounds__(256, 4) void attn_fwd_kernel(llsa_attn_fwd_args a) {
-    static_assert(NB == 2, "the shared phase reads an LDS buffer as two steps of two blocks");
+    static_assert(NB == 2 && kGroup == 4, "the shared phase reads an LDS buffer of four blocks as two steps of two");
     __shared__ __align__(16) bf16 sh[2][kGroup][2 * kTile];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -207,7 +198,7 @@ __global__ __launch_bounds__(256, 4) void attn_fwd_kernel(llsa_attn_fwd_args a) 
 #pragma unroll
     for (int dt = 0; dt < 4; dt++) st.acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    KvRegs<NB> ra, rb;
+    KvRegs ra, rb;
 
     // ---- shared blocks, out of LDS.  The barrier at the top of round grp says two things: every
     // wave's part of group grp has landed, and every wave is done reading the other buffer
@@ -240,7 +231,7 @@ __global__ __launch_bounds__(256, 4) void attn_fwd_kernel(llsa_attn_fwd_args a) 
         const int cn = min(kWave, a.T - c0);                  // a multiple of 4: an even number of steps
         if (c0 > 0) mine = (lane < cn) ? ip[c0 + lane] : 0;
         const int n_fine = cn / NB;
-        auto describe = [=](int t, StepDesc<NB>& d) __attribute__((always_inline)) {
+        auto describe = [=](int t, StepDesc& d) __attribute__((always_inline)) {
 #pragma unroll
             for (int j = 0; j < NB; j++) {
                 const int blk = clampi(__builtin_amdgcn_readlane(mine, NB * t + j), 0, N1 - 1);
@@ -251,7 +242,7 @@ __global__ __launch_bounds__(256, 4) void attn_fwd_kernel(llsa_attn_fwd_args a) 
         // The prefetch is unconditional (past the end it re-reads the last step) so that the loop
         // body is straight-line code: with the loads inside a branch the compiler has to drain the
         // memory queue (s_waitcnt vmcnt(0)) before every step and the overlap is lost.
-        StepDesc<NB> d;
+        StepDesc d;
         describe(0, d);
         load_step(ra, d, lane);
         for (int t = 0; t < n_fine; t += 2) {
@@ -304,7 +295,7 @@ extern "C" int llsa_attn_fwd(const llsa_attn_fwd_args* a, void* stream) {
                  "attn_fwd: tensors must be 16-byte aligned");
     LLSA_REQUIRE((a->sob % 4 == 0) && (a->soh % 4 == 0) && (a->son % 4 == 0), "attn_fwd: rows of o must be 8-byte aligned");
     const int N1 = a->N / 16;
-    hipLaunchKernelGGL(HIP_KERNEL_NAME(attn_fwd_kernel<LLSA_FWD_NB>), dim3((N1 + 3) / 4, a->B * a->H), dim3(256), 0,
+    hipLaunchKernelGGL(attn_fwd_kernel, dim3((N1 + 3) / 4, a->B * a->H), dim3(256), 0,
                        (hipStream_t)stream, *a);
     return launch_status("attn_fwd");
 }

@@ -251,8 +251,6 @@ class LlsaFused(Function):
             ctx.meta = (lib, lay, B, H, N, T, T2, levels, q.shape, q.stride(), k.stride(), v.stride(), T3)
             ctx.eps = float(eps)
             ctx.gamma_dtypes = (None if gamma_q is None else gamma_q.dtype, None if gamma_k is None else gamma_k.dtype)
-        global _last
-        _last = (I, lay, B, H, T, T2, T3, levels)
         return o
 
     @staticmethod
@@ -318,18 +316,6 @@ class LlsaFused(Function):
                 else:
                     dgk = dg
         return dq, dk, dv, None, None, None, None, None, dgq, dgk, None, None
-
-
-_last = None        # int32 arena and layout of the most recent forward (for last_selection)
-
-
-def last_selection():
-    """(indices, p_indices or None, pp_indices or None) of the most recent forward in this process, also
-    one that recorded no backward."""
-    I, lay, B, H, T, T2, T3, levels = _last
-    view = lambda off, rows, t: I[off:off + B * H * rows * t].view(B, H, rows, t)
-    return (view(lay.idx, lay.n1, T), view(lay.pidx, lay.n2, T2) if levels >= 2 else None,
-            view(lay.ppidx, lay.n3, T3) if levels == 3 else None)
 
 
 def selection(out):

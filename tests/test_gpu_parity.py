@@ -219,7 +219,7 @@ def test_selection_limits_are_errors(dev):
 
 @pytest.mark.skip(reason="capturing this case (B=1, H=2, N=16384, topk 8/4) ended in a segmentation fault of the host "
                          "process inside torch.cuda.graph's capture_end (hipStreamEndCapture), twice; the cause is not "
-                         "known, so the case stays off the GPU.  The same capture and replay at the bench shapes "
+                         "known, so the case stays off the GPU and GraphedStep's constructor raises.  The same capture and replay at the bench shapes "
                          "(B=2,H=6,N=16384,16/16 and B=4,H=6,N=4096,16) completed and matched the eager step bit for bit.")
 def test_graphed_step_matches_eager(dev):
     """A forward + backward captured in one HIP graph gives, on every replay, bit for bit what the
@@ -242,7 +242,8 @@ def test_graphed_step_matches_eager(dev):
         return [t.clone() for t in (o, q.grad, k.grad, v.grad)]
 
     ref = eager()
-    g = llsa_amd.GraphedStep(fn, [q, k, v], do)
+    from llsa_amd.utils.graphed import GraphedStep
+    g = GraphedStep(fn, [q, k, v], do)
     for rep in range(3):
         if rep == 2:                                  # new inputs, written into the graph's static buffers
             with torch.no_grad():
