@@ -123,8 +123,8 @@ def stage_profile(op, q, k, v, do, t1, t2, freq, iters, torch):
 
     def pyramid():
         return pool_pyramid([PoolSpec(q, y1=True, y2=l2, xr=True, rope=rope),
-                             PoolSpec(k, y1=True, y2=l2, xr=True, y1r=True, rope=rope),
-                             PoolSpec(v, y1=True, y2=l2, xr=True, xt=True, y1r=True, y1t=True)], freq)
+                             PoolSpec(k, y1=True, y2=l2, xr=True, y1r=True, rope=rope, y2r=l2),
+                             PoolSpec(v, y1=True, y2=l2, xr=True, xt=True, y1r=True, y1t=True, y2r=l2, y2t=l2)], freq)
 
     oq, ok, ov = pyramid()
     res["pool_pyramid"] = timed(pyramid, iters, torch)
@@ -132,10 +132,7 @@ def stage_profile(op, q, k, v, do, t1, t2, freq, iters, torch):
     tiles = dict(qr=oq["xr"], kr=ok["xr"], vr=ov["xr"], vt=ov["xt"], pkr=ok["y1r"], pvr=ov["y1r"], pvt=ov["y1t"])
     if l2:
         pq2, pk2, pv2 = oq["y2"], ok["y2"], ov["y2"]
-        lvl2 = lambda: pool_pyramid([PoolSpec(pk2, xr=True), PoolSpec(pv2, xr=True, xt=True)])
-        o2k, o2v = lvl2()
-        res["pool_level2_tiles"] = timed(lvl2, iters, torch)
-        tiles.update(pk2r=o2k["xr"], pv2r=o2v["xr"], pv2t=o2v["xt"])
+        tiles.update(pk2r=ok["y2r"], pv2r=ov["y2r"], pv2t=ov["y2t"])
         pidx = gen_sparse_indices(pq2, pk2, t2)
         res["topk_dense"] = timed(lambda: gen_sparse_indices(pq2, pk2, t2), iters, torch)
         idx = compute_topk_indices_sparse(pq, pk, pidx, t1, t2)

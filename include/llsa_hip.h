@@ -76,6 +76,8 @@ typedef struct llsa_pool_item {
     const float* gamma;     /* (64) fp32 or NULL: RMS-normalise every row first (see below)     */
     float eps;
     int32_t reserved;       /* 0                                                                */
+    void* y2r;              /* (B,H,n/4096,1024) R tiles of y2, or NULL (n % 4096 == 0)         */
+    void* y2t;              /* (B,H,n/4096,1024) T tiles of y2, or NULL (n % 4096 == 0)         */
 } llsa_pool_item;
 
 int llsa_pool_pyramid_fwd(const llsa_pool_item* items, int n_items, const void* freq /* (n,64) bf16 or NULL */,

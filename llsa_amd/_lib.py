@@ -21,7 +21,7 @@ class PoolItem(C.Structure):
                 ("n", c_int32), ("rope", c_int32),
                 ("y1", c_void_p), ("y2", c_void_p), ("xr", c_void_p), ("xt", c_void_p), ("y1r", c_void_p),
                 ("y1t", c_void_p), ("xrot", c_void_p),
-                ("gamma", c_void_p), ("eps", c_float), ("reserved", c_int32)]
+                ("gamma", c_void_p), ("eps", c_float), ("reserved", c_int32), ("y2r", c_void_p), ("y2t", c_void_p)]
 
 
 class AttnFwdArgs(C.Structure):

@@ -163,14 +163,14 @@ __global__ __launch_bounds__(128) void pool_pyramid_kernel(PoolParams p) {
         }
         stage_out(stage, (bf16*)it.xt + ((int64_t)bh * n1 + blockIdx.x * 16) * kTile, t, n_valid, false);
     }
-    if (it.y2 == nullptr && it.y1r == nullptr && it.y1t == nullptr) return;      // uniform over the workgroup
+    if (it.y2 == nullptr && it.y1r == nullptr && it.y1t == nullptr && it.y2r == nullptr && it.y2t == nullptr) return;   // uniform over the workgroup
 
     // the 16 pooled rows of this workgroup are one block of the next level
     bf16 (*sm)[kD] = reinterpret_cast<bf16 (*)[kD]>(stage);
     st16(&sm[r][c * 8], y);
     __syncthreads();
     const int n2 = it.n / (kBlk * kBlk);
-    if (it.y2 != nullptr && t < 8) {
+    if ((it.y2 != nullptr || it.y2r != nullptr || it.y2t != nullptr) && t < 8) {
         float acc[8];
 #pragma unroll
         for (int e = 0; e < 8; e++) acc[e] = 0.f;
@@ -182,7 +182,16 @@ __global__ __launch_bounds__(128) void pool_pyramid_kernel(PoolParams p) {
         bf16x8 y2;
 #pragma unroll
         for (int e = 0; e < 8; e++) y2[e] = (bf16)(acc[e] * 0.0625f);
-        st16((bf16*)it.y2 + ((int64_t)bh * n2 + blockIdx.x) * kD + t * 8, y2);
+        if (it.y2 != nullptr) st16((bf16*)it.y2 + ((int64_t)bh * n2 + blockIdx.x) * kD + t * 8, y2);
+        // this workgroup's level-2 row is row blockIdx.x % 16 of level-2 block blockIdx.x / 16: its 8-channel chunk
+        // t goes straight into that block's tiles (the other 15 rows come from the neighbouring workgroups)
+        const int64_t tile2 = ((int64_t)bh * (n2 / kBlk) + blockIdx.x / kBlk) * kTile;
+        const int r2 = blockIdx.x % kBlk;
+        if (it.y2r != nullptr) st16((bf16*)it.y2r + tile2 + (t * 16 + r2) * 8, y2);
+        if (it.y2t != nullptr) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) ((bf16*)it.y2t)[tile2 + t_tile_off(r2, t * 8 + e)] = y2[e];
+        }
     }
     if (it.y1r != nullptr)               // thread (r, c) holds chunk c of pooled row r
         st16((bf16*)it.y1r + ((int64_t)bh * n2 + blockIdx.x) * kTile + (c * 16 + r) * 8, y);
@@ -364,6 +373,9 @@ extern "C" int llsa_pool_pyramid_fwd(const llsa_pool_item* items, int n_items, c
                      "pool_pyramid: item %d: rows must be 16-byte aligned", i);
         LLSA_REQUIRE((it.y2 == nullptr && it.y1t == nullptr && it.y1r == nullptr) || it.n % 256 == 0,
                      "pool_pyramid: item %d: level-2 outputs need n %% 256 == 0 (n=%d)", i, it.n);
+        LLSA_REQUIRE((it.y2r == nullptr && it.y2t == nullptr) || it.n % 4096 == 0,
+                     "pool_pyramid: item %d: level-2 tiles need n %% 4096 == 0 (n=%d)", i, it.n);
+        LLSA_REQUIRE(aligned16(it.y2r) && aligned16(it.y2t), "pool_pyramid: item %d: outputs must be 16-byte aligned", i);
         LLSA_REQUIRE(!it.rope || freq != nullptr, "pool_pyramid: item %d: rope needs freq", i);
         LLSA_REQUIRE(it.gamma == nullptr || it.eps >= 0.f, "pool_pyramid: item %d: eps must be >= 0", i);
         LLSA_REQUIRE(aligned16(it.y1) && aligned16(it.y2) && aligned16(it.xr) && aligned16(it.xt) && aligned16(it.y1r) &&

@@ -87,15 +87,16 @@ class PoolSpec:
     rotated)."""
 
     def __init__(self, x, y1=False, y2=False, xr=False, xt=False, y1r=False, y1t=False, rope=False, xrot=False,
-                 gamma=None, eps=0.0):
+                 gamma=None, eps=0.0, y2r=False, y2t=False):
         self.x, self.y1, self.y2, self.xr, self.xt, self.y1r, self.y1t = x, y1, y2, xr, xt, y1r, y1t
+        self.y2r, self.y2t = y2r, y2t              # operand tiles of y2 (n a multiple of 4096)
         self.rope, self.xrot, self.gamma, self.eps = rope, xrot, gamma, eps
 
 
 def pool_pyramid(specs: Sequence[PoolSpec], freq: Optional[torch.Tensor] = None):
     """One launch of llsa_pool_pyramid_fwd.  Returns, per spec, a dict with the requested
     outputs: y1 (B,H,n/16,64), y2 (B,H,n/256,64), xr / xt (B,H,n/16,1024), y1r / y1t
-    (B,H,n/256,1024), xrot (B,H,n,64).  The tile layouts are described in include/llsa_hip.h."""
+    (B,H,n/256,1024), y2r / y2t (B,H,n/4096,1024), xrot (B,H,n,64).  The tile layouts are described in include/llsa_hip.h."""
     assert 1 <= len(specs) <= 4
     x0 = specs[0].x
     lib = lib_for(*[s.x for s in specs], freq)
@@ -127,6 +128,12 @@ def pool_pyramid(specs: Sequence[PoolSpec], freq: Optional[torch.Tensor] = None)
             o["y1r"] = e(B, H, n // 256, 1024)
         if s.y1t:
             o["y1t"] = e(B, H, n // 256, 1024)
+        if (s.y2r or s.y2t) and n % 4096 != 0:
+            raise ValueError(f"token count {n} is not a multiple of 4096")
+        if s.y2r:
+            o["y2r"] = e(B, H, n // 4096, 1024)
+        if s.y2t:
+            o["y2t"] = e(B, H, n // 4096, 1024)
         if s.rope and freq is None:
             raise ValueError("rope requested without a table")
         if s.xrot:
@@ -140,7 +147,8 @@ def pool_pyramid(specs: Sequence[PoolSpec], freq: Optional[torch.Tensor] = None)
             keep.append(gamma)
         items.append(PoolItem(x.data_ptr(), x.stride(0), x.stride(1), x.stride(2), n, 1 if s.rope else 0,
                               *(o[k].data_ptr() if k in o else None for k in ("y1", "y2", "xr", "xt", "y1r", "y1t", "xrot")),
-                              None if gamma is None else gamma.data_ptr(), float(s.eps), 0))
+                              None if gamma is None else gamma.data_ptr(), float(s.eps), 0,
+                              o["y2r"].data_ptr() if "y2r" in o else None, o["y2t"].data_ptr() if "y2t" in o else None))
     if freq is not None:
         require_bf16(freq)
         freq = freq.contiguous()

@@ -175,15 +175,22 @@ class LlsaFused(Function):
         stream = _stream(lib, q)
         l2, l3 = levels >= 2, levels == 3
 
+        two = l2 and not l3     # two levels: the tiles of the level-2 rows come out of the same pass (with three, a second one makes them)
         items = (PoolItem * 3)(
             PoolItem(q.data_ptr(), q.stride(0), q.stride(1), q.stride(2), N, int(rope), pa(lay.pq), pa(lay.pq2), pa(lay.qr),
-                     None, None, None, None, None if gq is None else gq.data_ptr(), float(eps), 0),
+                     None, None, None, None, None if gq is None else gq.data_ptr(), float(eps), 0, None, None),
             PoolItem(k.data_ptr(), k.stride(0), k.stride(1), k.stride(2), N, int(rope), pa(lay.pk), pa(lay.pk2), pa(lay.kr),
-                     None, pa(lay.pkr), None, None, None if gk is None else gk.data_ptr(), float(eps), 0),
+                     None, pa(lay.pkr), None, None, None if gk is None else gk.data_ptr(), float(eps), 0,
+                     pa(lay.pk2r) if two else None, None),
             PoolItem(v.data_ptr(), v.stride(0), v.stride(1), v.stride(2), N, 0, pa(lay.pv), pa(lay.pv2), pa(lay.vr),
-                     pa(lay.vt), pa(lay.pvr), pa(lay.pvt), None))
+                     pa(lay.vt), pa(lay.pvr), pa(lay.pvt), None, None, 0.0, 0,
+                     pa(lay.pv2r) if two else None, pa(lay.pv2t) if two else None))
         _check(lib, lib.pool_pyramid_fwd(items, 3, freq.data_ptr() if rope else None, B, H, stream), "pool_pyramid")
-        if l2:
+        if two:
+            _check(lib, lib.topk_dense(pa(lay.pq2), pa(lay.pk2), pi(lay.pidx), B, H, n2, T2, 1, stream), "gen_sparse_indices")
+            _check(lib, lib.topk_sparse(pa(lay.pq), pa(lay.pk), pi(lay.pidx), pi(lay.idx), B, H, n1, T, T2, stream),
+                   "compute_topk_indices_sparse")
+        elif l2:
             s2 = (H * n2 * 64, n2 * 64, 64)
             # the level-2 rows again: their tiles and (three levels) the level-3 rows with theirs
             items2 = (PoolItem * 3)(

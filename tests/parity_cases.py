@@ -72,7 +72,9 @@ def check_pool_pyramid(dev, B=1, H=2, N=512, strided=True, rope=True):
     x, *_ = randn_inputs(B, H, N, 64, dev, seed=5, strided=strided)
     x = x * 2
     freq = torch.randn(N, 64, generator=torch.Generator().manual_seed(6)).bfloat16().to(dev) if rope else None
-    out, = pool_pyramid([PoolSpec(x, y1=True, y2=True, xr=True, xt=True, y1r=True, y1t=True, rope=rope, xrot=rope)], freq)
+    lvl2 = N % 4096 == 0
+    out, = pool_pyramid([PoolSpec(x, y1=True, y2=True, xr=True, xt=True, y1r=True, y1t=True, rope=rope, xrot=rope,
+                                  y2r=lvl2, y2t=lvl2)], freq)
     xc = x.cpu()
     xr = O.rope_apply(xc, freq.cpu()) if rope else xc
     p1 = O.mean_pool(xr)
@@ -85,6 +87,9 @@ def check_pool_pyramid(dev, B=1, H=2, N=512, strided=True, rope=True):
     assert torch.equal(out["xt"].cpu(), _t_tiles(xr)), "T tiles differ"
     assert torch.equal(out["y1r"].cpu(), _r_tiles(p1)), "R tiles of the pooled level differ"
     assert torch.equal(out["y1t"].cpu(), _t_tiles(p1)), "T tiles of the pooled level differ"
+    if lvl2:
+        assert torch.equal(out["y2r"].cpu(), _r_tiles(p2)), "R tiles of the level-2 rows differ"
+        assert torch.equal(out["y2t"].cpu(), _t_tiles(p2)), "T tiles of the level-2 rows differ"
 
 
 def check_mean_pool1d(dev, dtype=torch.bfloat16, K=16, C=64, S=128, fmt='bhsc'):

@@ -21,6 +21,7 @@ def _emu():
 def test_pool_pyramid():
     P.check_pool_pyramid(DEV, N=512, strided=True, rope=True)
     P.check_pool_pyramid(DEV, N=256, strided=False, rope=False)
+    P.check_pool_pyramid(DEV, B=1, H=1, N=4096, strided=True, rope=False)       # with the tiles of the level-2 rows
 
 
 def test_mean_pool1d():
