@@ -156,6 +156,28 @@ int llsa_topk_sparse(const void* pq, const void* pk, const int32_t* parent_idx, 
                      int B, int H, int N1, int T, int T2, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * The hierarchy.  Pooled level l = 1 .. levels: its tokens are means of 16^l input tokens and weigh
+ * 16^l in the soft-max (token_weight, token_weight_2 of the reference for l = 1, 2).  A block of a
+ * level is 16 of its tokens.  A query reads: the T fine blocks its query block selected (idx); at
+ * every level l < levels the lvl[l-1].T blocks of that level which its group of 16^(l+1) queries
+ * selected (lvl[l-1].sel -- the reference's p_indices is level 1 of llsa_l2); and every block of the
+ * coarsest level.  levels = 1 is llsa_l1 (sparse_attention_res_1.py), levels = 2 llsa_l2
+ * (sparse_attention_res_2.py); deeper hierarchies have no counterpart in the reference and continue
+ * the scheme by induction on sparse_attention_res_2.py:94-149.  The coarsest level is walked in
+ * groups of four blocks: N must be a multiple of 64 * 16^levels.
+ * ---------------------------------------------------------------------------------------- */
+#define LLSA_MAX_LEVELS 4
+
+typedef struct llsa_fwd_level {
+    const void* kr;                            /* (B,H,N/16^(l+1),1024) R tiles of the level's pooled k    */
+    const void* vt;                            /* (B,H,N/16^(l+1),1024) T tiles of the level's pooled v    */
+    const int32_t* sel;                        /* (B,H,N/16^(l+1),T) blocks of this level selected by every group
+                                                  of 16^(l+1) queries; NULL at the coarsest level          */
+    int32_t T;                                 /* multiple of 4; ignored at the coarsest level             */
+    float w;                                   /* weight of one token of this level (> 0)                  */
+} llsa_fwd_level;
+
+/* ------------------------------------------------------------------------------------------
  * Forward.  Replaces sparse_indices_attn_res_fwd (sparse_attention_res_1.py:123-150) when
  * levels == 1 and sparse_indices_attn_res_2_2_fwd (sparse_attention_res_2.py:166-199) when
  * levels == 2.
@@ -164,23 +186,11 @@ typedef struct llsa_attn_fwd_args {
     const void* qr;                            /* (B,H,N/16,1024)   R tiles of q                  */
     const void* kr;                            /* (B,H,N/16,1024)   R tiles of k                  */
     const void* vt;                            /* (B,H,N/16,1024)   T tiles of v                  */
-    const void* pkr;                           /* (B,H,N/256,1024)  R tiles of level-1 pooled k   */
-    const void* pvt;                           /* (B,H,N/256,1024)  T tiles of level-1 pooled v   */
-    const void* pk2r;                          /* (B,H,N/4096,1024) R tiles of level-2 pooled k   */
-    const void* pv2t;                          /* (B,H,N/4096,1024) T tiles of level-2 pooled v   */
     const int32_t* idx;                        /* (B,H,N/16,T)   selected fine blocks             */
-    const int32_t* pidx;                       /* (B,H,N/256,T2) selected coarse blocks (l2)      */
     void* o;        int64_t sob, soh, son;     /* (B,H,N,64) out                                  */
     float* lse;                                /* (B,H,N) out, m + log(l)                          */
-    int32_t B, H, N, T, T2, levels;
-    float w1, w2;                              /* token_weight, token_weight_2                    */
-    /* levels == 3 (no counterpart in the reference): one more pooled level.  pkr/pvt then hold
-     * N/256 tiles, pk2r/pv2t N/4096 tiles, pidx is (B,H,N/256,T2) as before. */
-    const void* pk3r;                          /* (B,H,N/65536,1024) R tiles of level-3 pooled k  */
-    const void* pv3t;                          /* (B,H,N/65536,1024) T tiles of level-3 pooled v  */
-    const int32_t* ppidx;                      /* (B,H,N/4096,T3) selected level-2 blocks         */
-    int32_t T3;
-    float w3;                                  /* token_weight_3                                  */
+    int32_t B, H, N, T, levels, reserved;
+    llsa_fwd_level lvl[LLSA_MAX_LEVELS];       /* lvl[l - 1] = pooled level l                     */
 } llsa_attn_fwd_args;
 
 int llsa_attn_fwd(const llsa_attn_fwd_args* a, void* stream);
@@ -194,7 +204,7 @@ int llsa_attn_fwd(const llsa_attn_fwd_args* a, void* stream);
  * undefined (nothing is read or written out of bounds).
  * With `inv` (B,H,Mb,T) the inverse is written too: inv[q][t] = position in flat of the entry
  * that (query block q, slot t) became.  llsa_attn_bwd needs it for the selections of the pooled
- * levels (pidx, ppidx): the partial sums of a key block are stored at the positions of its list.
+ * levels (lvl[].sel): the partial sums of a key block are stored at the positions of its list.
  * ---------------------------------------------------------------------------------------- */
 int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, int32_t* work /* or NULL */,
                            int32_t* inv /* or NULL */, int B, int H, int Mb, int Kb, int T, int chunk, void* stream);
@@ -217,49 +227,46 @@ int64_t llsa_work_list_len(int Mb, int Kb, int T, int chunk);
 /* ------------------------------------------------------------------------------------------
  * Backward.  Replaces sparse_indices_attn_res_scatter_bwd_v2 (sparse_attention_res_1.py:403-471)
  * and sparse_indices_attn_res_scatter_2_2_bwd_v2 (sparse_attention_res_2.py:578-681): the
- * delta pre-pass, dQ, dK/dV over the transposed index, the sparse level-1 pooled gradients
- * and the dense coarsest pooled gradients.  The k*scale temporaries of the reference
- * (:420-422) do not exist here.  cgw1 is the factor used on the dpk/dpv path of the level-1
- * pooled tokens: the reference uses 1 for l1 (sparse_attention_res_1.py:388-389) and w1 for
- * l2 (sparse_attention_res_2.py:564).  With levels == 3 (no counterpart in the reference) the
- * level-2 pooled gradients come from a second list-driven pass over the transposed ppidx, the
- * dense pass runs on level 3, and fold_pooled chains three pool backwards.
+ * delta pre-pass, dQ, dK/dV over the transposed index, the gradients of the pooled levels under
+ * an ancestor's selection and of the dense coarsest level.  The k*scale temporaries of the
+ * reference (:420-422) do not exist here.  Levels as in the forward; lvl[l-1].gw is the factor used
+ * on the path to the level's own gradient: the reference uses 1 for the one level of llsa_l1
+ * (sparse_attention_res_1.py:388-389) where its forward and its dq use token_weight, and the
+ * weight itself everywhere in llsa_l2 (sparse_attention_res_2.py:478, :564).
  * ---------------------------------------------------------------------------------------- */
+typedef struct llsa_bwd_level {
+    const void* kr; const void* vr;              /* (B,H,N/16^(l+1),1024) R tiles of the level's pooled k, v      */
+    const int32_t* sel;                          /* as in the forward; NULL at the coarsest level                  */
+    const int32_t* off; const int32_t* inv;      /* transposed sel (Kb = N/16^(l+1)): offsets and inverse positions */
+    void* dk; void* dv;                          /* (B,H,N/16^l,64) contiguous out: gradients of the pooled k, v    */
+    int32_t T;
+    float w, gw;
+    int32_t reserved;
+} llsa_bwd_level;
+
 typedef struct llsa_attn_bwd_args {
     const void* dout; int64_t sdob, sdoh, sdon;  /* (B,H,N,64) upstream gradient                 */
     const void* o;    int64_t sob, soh, son;     /* (B,H,N,64) forward output                     */
     const float* lse;                            /* (B,H,N)                                       */
     const void* qr;  const void* kr;  const void* vr;   /* R tiles of q, k, v  (B,H,N/16,1024)    */
-    const void* pkr; const void* pvr;            /* R tiles of pk, pv   (B,H,N/256,1024)          */
-    const void* pk2r; const void* pv2r;          /* R tiles of pk2, pv2 (B,H,N/4096,1024)         */
-    const int32_t* idx;  const int32_t* pidx;
+    const int32_t* idx;                          /* (B,H,N/16,T) selected fine blocks             */
     const int32_t* off;  const int32_t* flat;  const int32_t* work;    /* transposed idx  (Kb = N/16)     */
-    const int32_t* poff; const int32_t* pinv;    /* transposed pidx (Kb = N/256): offsets and inverse positions */
     void* dq; int64_t sdqb, sdqh, sdqn;
     void* dk; int64_t sdkb, sdkh, sdkn;
     void* dv; int64_t sdvb, sdvh, sdvn;
-    void* dpk;  void* dpv;                       /* (B,H,N/16,64) contiguous out                  */
-    void* dpk2; void* dpv2;                      /* (B,H,N/256,64) contiguous out (levels == 2)   */
     void* workspace; int64_t workspace_bytes;    /* see llsa_attn_bwd_workspace_bytes             */
     const void* freq_dq;                         /* (N,64) or NULL: rotate dq back (fused rope)   */
     const void* freq_dk;                         /* (N,64) or NULL: rotate dk back; needs fold_pooled */
-    int32_t B, H, N, T, T2, levels;
-    float w1, w2, cgw1;
-    int32_t stages;                              /* 0 = everything; else a mask of LLSA_BWD_* to
-                                                    launch only those kernels (profiling)        */
+    int32_t B, H, N, T, levels;
+    int32_t stages;                              /* 0 = everything; else a mask of LLSA_BWD_* (see below) */
     int32_t fold_pooled;                         /* 0: dk, dv are the fine-token gradients only, as the
                                                     reference's kernels return them (mean_pool1d's backward
-                                                    and autograd add dpk.. afterwards).  1: dk, dv also
-                                                    receive the pooled gradients of their blocks, with the
-                                                    same bf16 roundings (= llsa_pool_bwd_accum), and dk is
-                                                    rotated back with freq_dk                          */
-    /* levels == 3 (no counterpart in the reference): one more pooled level */
-    const void* pk3r; const void* pv3r;          /* R tiles of pk3, pv3 (B,H,N/65536,1024)        */
-    const int32_t* ppidx;                        /* (B,H,N/4096,T3) selected level-2 blocks        */
-    const int32_t* ppoff; const int32_t* ppinv;  /* transposed ppidx (Kb = N/4096): offsets, inverse positions */
-    void* dpk3; void* dpv3;                      /* (B,H,N/4096,64) contiguous out                 */
-    int32_t T3;
-    float w3;
+                                                    and autograd add the pooled gradients afterwards).  1: dk, dv
+                                                    also receive the pooled gradients of their blocks, with the
+                                                    same bf16 roundings (= llsa_pool_bwd_accum, level by level),
+                                                    and dk is rotated back with freq_dk                */
+    int32_t reserved;
+    llsa_bwd_level lvl[LLSA_MAX_LEVELS];         /* lvl[l - 1] = pooled level l                     */
 } llsa_attn_bwd_args;
 
 /* `stages` is a diagnostic for timing kernels one at a time: a mask other than 0 launches only the named kernels.
@@ -269,12 +276,13 @@ typedef struct llsa_attn_bwd_args {
 #define LLSA_BWD_DQ 2       /* dq; also delta = rowsum(o * dout) and the R tiles of dout, which the
                                stages below read from the workspace                              */
 #define LLSA_BWD_DKV 4      /* dK/dV of the fine tokens                                          */
-#define LLSA_BWD_DPKV1 8    /* sparse pooled gradients: level 1 (levels >= 2), level 2 (levels == 3) */
+#define LLSA_BWD_DPKV1 8    /* gradients of the pooled levels below the coarsest (levels >= 2)   */
 #define LLSA_BWD_DENSE 16   /* dense coarsest pooled gradients (partials + reduction)            */
 #define LLSA_BWD_NO_REDUCE 32 /* with an explicit mask: leave out the reductions of partial sums (results
                                  are then incomplete; for timing the K-side kernels alone)          */
 
-int64_t llsa_attn_bwd_workspace_bytes(int B, int H, int N, int T, int T2, int T3, int levels);
+/* topk: `levels` entries, topk[0] = T of the fine blocks, topk[l] = lvl[l-1].T for l < levels */
+int64_t llsa_attn_bwd_workspace_bytes(int B, int H, int N, const int32_t* topk, int levels);
 int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream);
 
 #ifdef __cplusplus

@@ -10,8 +10,8 @@ from .kernel.hip.rope import my_rope_fn
 from .kernel.torch_op.flash_sparse_attention_res_1 import (flash_sparse_residual_attention_l1_op, llsa_l1,
                                                            llsa_l1_unfused)
 from .kernel.torch_op.flash_sparse_attention_res_2 import (flash_sparse_residual_attention_l2_op, llsa_l2,
-                                                           llsa_l2_unfused, llsa_l3)
+                                                           llsa_l2_unfused, llsa_l3, llsa_lk)
 
-__all__ = ["llsa_l1", "llsa_l2", "llsa_l3", "llsa_l1_unfused", "llsa_l2_unfused", "flash_sparse_residual_attention_l1_op",
+__all__ = ["llsa_l1", "llsa_l2", "llsa_l3", "llsa_lk", "llsa_l1_unfused", "llsa_l2_unfused", "flash_sparse_residual_attention_l1_op",
            "flash_sparse_residual_attention_l2_op", "mean_pool1d", "my_rope_fn", "my_rms_norm_fn", "permute_tokens",
            "gather_tokens"]

@@ -24,19 +24,28 @@ class PoolItem(C.Structure):
                 ("gamma", c_void_p), ("eps", c_float), ("reserved", c_int32), ("y2r", c_void_p), ("y2t", c_void_p)]
 
 
+MAX_LEVELS = 4                                              # LLSA_MAX_LEVELS
+
+
+class FwdLevel(C.Structure):
+    _fields_ = [("kr", c_void_p), ("vt", c_void_p), ("sel", c_void_p), ("T", c_int32), ("w", c_float)]
+
+
 class AttnFwdArgs(C.Structure):
-    _fields_ = [("qr", c_void_p), ("kr", c_void_p), ("vt", c_void_p), ("pkr", c_void_p), ("pvt", c_void_p),
-                ("pk2r", c_void_p), ("pv2t", c_void_p),
-                ("idx", c_void_p), ("pidx", c_void_p),
+    _fields_ = [("qr", c_void_p), ("kr", c_void_p), ("vt", c_void_p), ("idx", c_void_p),
                 ("o", c_void_p), ("sob", c_int64), ("soh", c_int64), ("son", c_int64),
                 ("lse", c_void_p),
-                ("B", c_int32), ("H", c_int32), ("N", c_int32), ("T", c_int32), ("T2", c_int32), ("levels", c_int32),
-                ("w1", c_float), ("w2", c_float),
-                ("pk3r", c_void_p), ("pv3t", c_void_p), ("ppidx", c_void_p), ("T3", c_int32), ("w3", c_float)]
+                ("B", c_int32), ("H", c_int32), ("N", c_int32), ("T", c_int32), ("levels", c_int32), ("reserved", c_int32),
+                ("lvl", FwdLevel * MAX_LEVELS)]
 
 
 def _t3(name):
     return [(name, c_void_p), ("s" + name + "b", c_int64), ("s" + name + "h", c_int64), ("s" + name + "n", c_int64)]
+
+
+class BwdLevel(C.Structure):
+    _fields_ = [("kr", c_void_p), ("vr", c_void_p), ("sel", c_void_p), ("off", c_void_p), ("inv", c_void_p),
+                ("dk", c_void_p), ("dv", c_void_p), ("T", c_int32), ("w", c_float), ("gw", c_float), ("reserved", c_int32)]
 
 
 class AttnBwdArgs(C.Structure):
@@ -44,18 +53,14 @@ class AttnBwdArgs(C.Structure):
         [("dout", c_void_p), ("sdob", c_int64), ("sdoh", c_int64), ("sdon", c_int64)]
         + _t3("o")
         + [("lse", c_void_p), ("qr", c_void_p), ("kr", c_void_p), ("vr", c_void_p),
-           ("pkr", c_void_p), ("pvr", c_void_p), ("pk2r", c_void_p), ("pv2r", c_void_p),
-           ("idx", c_void_p), ("pidx", c_void_p), ("off", c_void_p), ("flat", c_void_p), ("work", c_void_p),
-           ("poff", c_void_p), ("pinv", c_void_p)]
+           ("idx", c_void_p), ("off", c_void_p), ("flat", c_void_p), ("work", c_void_p)]
         + [("dq", c_void_p), ("sdqb", c_int64), ("sdqh", c_int64), ("sdqn", c_int64),
            ("dk", c_void_p), ("sdkb", c_int64), ("sdkh", c_int64), ("sdkn", c_int64),
            ("dv", c_void_p), ("sdvb", c_int64), ("sdvh", c_int64), ("sdvn", c_int64)]
-        + [("dpk", c_void_p), ("dpv", c_void_p), ("dpk2", c_void_p), ("dpv2", c_void_p),
-           ("workspace", c_void_p), ("workspace_bytes", c_int64), ("freq_dq", c_void_p), ("freq_dk", c_void_p),
-           ("B", c_int32), ("H", c_int32), ("N", c_int32), ("T", c_int32), ("T2", c_int32), ("levels", c_int32),
-           ("w1", c_float), ("w2", c_float), ("cgw1", c_float), ("stages", c_int32), ("fold_pooled", c_int32),
-           ("pk3r", c_void_p), ("pv3r", c_void_p), ("ppidx", c_void_p), ("ppoff", c_void_p), ("ppinv", c_void_p),
-           ("dpk3", c_void_p), ("dpv3", c_void_p), ("T3", c_int32), ("w3", c_float)])
+        + [("workspace", c_void_p), ("workspace_bytes", c_int64), ("freq_dq", c_void_p), ("freq_dk", c_void_p),
+           ("B", c_int32), ("H", c_int32), ("N", c_int32), ("T", c_int32), ("levels", c_int32),
+           ("stages", c_int32), ("fold_pooled", c_int32), ("reserved", c_int32),
+           ("lvl", BwdLevel * MAX_LEVELS)])
 
 
 P64 = C.POINTER(c_int64)
@@ -80,7 +85,7 @@ _SIGNATURES = {
     "llsa_attn_fwd": (c_int, [C.POINTER(AttnFwdArgs), c_void_p]),
     "llsa_transpose_indices": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llsa_work_list_len": (c_int64, [c_int, c_int, c_int, c_int]),
-    "llsa_attn_bwd_workspace_bytes": (c_int64, [c_int, c_int, c_int, c_int, c_int, c_int, c_int]),
+    "llsa_attn_bwd_workspace_bytes": (c_int64, [c_int, c_int, c_int, C.POINTER(c_int32), c_int]),
     "llsa_attn_bwd": (c_int, [C.POINTER(AttnBwdArgs), c_void_p]),
 }
 

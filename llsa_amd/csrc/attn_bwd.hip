@@ -86,7 +86,7 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, floa
     __shared__ __align__(16) bf16 sh[2][kGroup][2 * kTile];   // per block: R tile of K, R tile of V
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int N1 = a.N / kBlk, N2 = N1 / kBlk, N3 = N2 / kBlk;
+    const int N1 = a.N / kBlk;
     const int lid = xcd_logical_id();
     const int g = (lid % (int)gridDim.x) * 4 + wave;          // < N1: the host checks N1 % 4 == 0
     const int bh = lid / (int)gridDim.x, b = bh / a.H, h = bh % a.H;
@@ -95,43 +95,16 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, floa
 
     const bf16* kr = (const bf16*)a.kr + (int64_t)bh * N1 * kTile;
     const bf16* vr = (const bf16*)a.vr + (int64_t)bh * N1 * kTile;
-    const bf16* pk = (const bf16*)a.pkr + (int64_t)bh * N2 * kTile;
-    const bf16* pv = (const bf16*)a.pvr + (int64_t)bh * N2 * kTile;
-    const bf16* pk2 = (a.levels >= 2) ? (const bf16*)a.pk2r + (int64_t)bh * N3 * kTile : nullptr;
-    const bf16* pv2 = (a.levels >= 2) ? (const bf16*)a.pv2r + (int64_t)bh * N3 * kTile : nullptr;
     const int* ip = a.idx + ((int64_t)bh * N1 + g) * a.T;
-    const int* pip = (a.levels >= 2) ? a.pidx + ((int64_t)bh * N2 + g / kBlk) * a.T2 : nullptr;
-    const int* ppip = (a.levels == 3) ? a.ppidx + ((int64_t)bh * N3 + g / (kBlk * kBlk)) * a.T3 : nullptr;
 
-    // shared list: (l2, l3) T2 blocks of level-1 pooled tokens, (l3) T3 blocks of level-2 pooled tokens, then
-    // every block of the coarsest level
-    const int n_mid = (a.levels >= 2) ? a.T2 : 0;
-    const int n_mid2 = (a.levels == 3) ? a.T3 : 0;
-    const int n_dense = (a.levels == 3) ? N3 / kBlk : (a.levels == 2) ? N2 / kBlk : N1 / kBlk;
-    const int n_groups = (n_mid + n_mid2 + n_dense) / kGroup;
-    const int pmine = (a.levels >= 2 && lane < a.T2) ? pip[lane] : 0;   // first 64 parent entries, entry i in lane i
-    const int ppmine = (a.levels == 3 && lane < a.T3) ? ppip[lane] : 0;
-    const bf16* dense_k = (a.levels == 3) ? (const bf16*)a.pk3r + (int64_t)bh * (N3 / kBlk) * kTile : (a.levels == 2) ? pk2 : pk;
-    const bf16* dense_v = (a.levels == 3) ? (const bf16*)a.pv3r + (int64_t)bh * (N3 / kBlk) * kTile : (a.levels == 2) ? pv2 : pv;
-    const float w_dense = (a.levels == 3) ? a.w3 : (a.levels == 2) ? a.w2 : a.w1;
+    // shared list: the selected blocks of every pooled level below the coarsest, then every block of the coarsest
+    SharedList sl = shared_list(a.lvl, a.levels, a.N, bh, g, lane);
+    const int n_groups = sl.n_blocks / kGroup;
     bf16* const sh0 = &sh[0][0][0];
-    auto issue_group = [=](int grp) __attribute__((always_inline)) {   // this wave brings in block kGroup*grp + wave
-        const int sblk = kGroup * grp + wave;
-        const bf16 *kb, *vb;
-        if (sblk < n_mid) {
-            const int blk = clampi(sblk < kWave ? __builtin_amdgcn_readlane(pmine, sblk) : pip[sblk], 0, N2 - 1);
-            kb = pk + (int64_t)blk * kTile;
-            vb = pv + (int64_t)blk * kTile;
-        } else if (sblk < n_mid + n_mid2) {
-            const int j = sblk - n_mid;
-            const int blk = clampi(j < kWave ? __builtin_amdgcn_readlane(ppmine, j) : ppip[j], 0, N3 - 1);
-            kb = pk2 + (int64_t)blk * kTile;
-            vb = pv2 + (int64_t)blk * kTile;
-        } else {
-            const int u = sblk - n_mid - n_mid2;
-            kb = dense_k + (int64_t)u * kTile;
-            vb = dense_v + (int64_t)u * kTile;
-        }
+    auto issue_group = [&](int grp) __attribute__((always_inline)) {   // this wave brings in block kGroup*grp + wave
+        const SharedBlock sb = shared_block(sl, a.lvl, a.levels, a.N, bh, kGroup * grp + wave);
+        const bf16* kb = (const bf16*)a.lvl[sb.level].kr + sb.tile;
+        const bf16* vb = (const bf16*)a.lvl[sb.level].vr + sb.tile;
         bf16* dst = sh0 + ((grp & 1) * kGroup + wave) * (2 * kTile);
         copy16_global_to_lds(kb + lane * 8, dst);
         copy16_global_to_lds(kb + 512 + lane * 8, dst + 512);
@@ -179,7 +152,7 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, floa
     for (int grp = 0; grp < n_groups; grp++) {
         wait_vm0();
         __syncthreads();
-        const float w = (kGroup * grp < n_mid) ? a.w1 : (kGroup * grp < n_mid + n_mid2) ? a.w2 : w_dense;
+        const float w = a.lvl[shared_level(a.lvl, a.levels, kGroup * grp)].w;
         const bf16* blk = sh0 + (grp & 1) * kGroup * (2 * kTile);
         PairR r0;
         PairT t0;
@@ -256,43 +229,39 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, floa
 // (what the backward of the two mean pools and autograd's accumulation do in the reference:
 // every sum and every division by 16 rounded to bf16) and rotate dK back through the RoPE.
 struct PoolFold {
-    const bf16* g1k; const bf16* g1v;             // level-1 pooled gradients (BH, N/16, 64); nullptr: no folding
-    const bf16* g2k; const bf16* g2v;             // level-2 pooled gradients (BH, N/256, 64) or nullptr
+    const bf16* gk[LLSA_MAX_LEVELS];              // gradients of the pooled k per level, (BH, N/16^l, 64); depth == 0: no folding
+    const bf16* gv[LLSA_MAX_LEVELS];
     const bf16* freq;                             // (N, 64) or nullptr
-    const bf16* g3k; const bf16* g3v;             // level-3 pooled gradients (BH, N/4096, 64) or nullptr
+    int depth;                                    // pooled levels to fold in
 };
-// x: four channels of one token; g / gg: the same channels of its block's level-1 / level-2 pooled
-// gradient; f: their [sin, cos] entries.  Mirrors pool_bwd_accum_kernel.
-__device__ __forceinline__ bf16x4 fold_math(bf16x4 x, bf16x4 g, bool has_gg, bf16x4 gg, bool has_f, bf16x4 f,
-                                            bool has_g3 = false, bf16x4 g3 = bf16x4{}) {
+// What a token receives from its pooled ancestors, level by level, coarsest first (pool_bwd_accum_kernel applied down the
+// chain): below = the running sum of the level above, g = the gradient of this level's own pooled token.
+__device__ __forceinline__ bf16x4 fold_step(bf16x4 g, bf16x4 below) {
 #pragma clang fp contract(off)
-    if (has_g3) {
 #pragma unroll
-        for (int e = 0; e < 4; e++) gg[e] = (bf16)((float)gg[e] + rn_bf16((float)g3[e] * 0.0625f));
-    }
-    if (has_gg) {
-#pragma unroll
-        for (int e = 0; e < 4; e++) g[e] = (bf16)((float)g[e] + rn_bf16((float)gg[e] * 0.0625f));
-    }
-#pragma unroll
-    for (int e = 0; e < 4; e++) x[e] = (bf16)((float)x[e] + rn_bf16((float)g[e] * 0.0625f));
+    for (int e = 0; e < 4; e++) g[e] = (bf16)((float)g[e] + rn_bf16((float)below[e] * 0.0625f));
+    return g;
+}
+// x: four channels of one token; c: the same channels of the chain's sum at its level-1 ancestor; f: their [sin, cos] entries
+__device__ __forceinline__ bf16x4 fold_math(bf16x4 x, bf16x4 c, bool has_f, bf16x4 f) {
+    x = fold_step(x, c);
     return has_f ? rope_bwd4(x, f) : x;
 }
 // x: channels c0..c0+3 of token `tok` of (b,h) `bh`; which = 0 for dK, 1 for dV
 __device__ __forceinline__ bf16x4 fold_pooled(bf16x4 x, const PoolFold& f, int which, int64_t bh, int N, int tok, int c0) {
-    const bf16* g1 = which ? f.g1v : f.g1k;
-    const bf16* g2 = which ? f.g2v : f.g2k;
-    const bf16* g3 = which ? f.g3v : f.g3k;
-    const int N1 = N / kBlk;
-    const bf16x4 g = ld8(g1 + (bh * N1 + tok / kBlk) * kD + c0);
-    bf16x4 gg = g, fr = g, g3v = g;
-    if (g2 != nullptr) gg = ld8(g2 + (bh * (N1 / kBlk) + tok / (kBlk * kBlk)) * kD + c0);
-    if (g3 != nullptr) g3v = ld8(g3 + (bh * (N1 / (kBlk * kBlk)) + tok / (kBlk * kBlk * kBlk)) * kD + c0);
+    bf16x4 acc = x;
+#pragma nounroll
+    for (int l = f.depth - 1; l >= 0; l--) {
+        const int sh = 4 * (l + 1);
+        const bf16x4 g = ld8((which ? f.gv[l] : f.gk[l]) + (bh * (N >> sh) + (tok >> sh)) * kD + c0);
+        acc = (l == f.depth - 1) ? g : fold_step(g, acc);
+    }
     const bool rot = which == 0 && f.freq != nullptr;
+    bf16x4 fr = x;
     if (rot) fr = ld8(f.freq + (int64_t)tok * kD + c0);
-    return fold_math(x, g, g2 != nullptr, gg, rot, fr, g3 != nullptr, g3v);
+    return fold_math(x, acc, rot, fr);
 }
-constexpr int kFoldRows = 6 * kD;                 // LDS copy of a unit's fold operands: 6 pooled rows, then 16 freq rows
+constexpr int kFoldRows = 2 * LLSA_MAX_LEVELS * kD;   // LDS copy of a unit's fold operands: per level its dk and dv row, then 16 freq rows
 constexpr int kFoldElems = kFoldRows + kBlk * kD;
 
 struct KSideParams {
@@ -409,16 +378,17 @@ __global__ __launch_bounds__(64) void attn_kside_kernel(KSideParams p) {
     }
     // What the fold on the way out needs (the unit's pooled-gradient rows, its tokens' RoPE entries)
     // is copied into LDS now, without registers, so that no load waits at the end of the wave.
-    const bool folding = p.fold.g1k != nullptr && slot < 0;
+    const bool folding = p.fold.depth > 0 && slot < 0;
     if (folding) {
-        const int row = lane >> 3, piece = lane & 7;          // rows: dpk, dpv, dpk2, dpv2, dpk3, dpv3 of the unit; 8 x 16 bytes each
-        const int deep = p.fold.g3k != nullptr ? 3 : p.fold.g2k != nullptr ? 2 : 1;
-        if (lane < 16 * deep) {
-            const int lvl = row >> 1;                         // pooled level 1, 2, 3 -> 0, 1, 2
-            const bf16* src = (row & 1) ? (lvl == 2 ? p.fold.g3v : lvl == 1 ? p.fold.g2v : p.fold.g1v)
-                                        : (lvl == 2 ? p.fold.g3k : lvl == 1 ? p.fold.g2k : p.fold.g1k);
-            const int div = lvl == 2 ? kBlk * kBlk : lvl == 1 ? kBlk : 1;
-            src += ((int64_t)bh * (N1 / div) + unit / div) * kD;
+        const int row = lane >> 3, piece = lane & 7;          // rows: dk, dv of level 1, of level 2, ...; 8 x 16 bytes each
+        if (row < 2 * p.fold.depth) {
+            const int lvl = row >> 1;
+            int n = N1, u = unit;
+            for (int l = 0; l < lvl; l++) {
+                n /= kBlk;
+                u /= kBlk;
+            }
+            const bf16* src = ((row & 1) ? p.fold.gv[lvl] : p.fold.gk[lvl]) + ((int64_t)bh * n + u) * kD;
             copy16_global_to_lds(src + piece * 8, fold_buf);
         }
         if (p.fold.freq != nullptr) {
@@ -468,17 +438,28 @@ __global__ __launch_bounds__(64) void attn_kside_kernel(KSideParams p) {
     }
     bf16* kp = p.dk + b * p.sdkb + h * p.sdkh + (int64_t)(unit * kBlk + r) * p.sdkn + quad * 4;
     bf16* vp = p.dv + b * p.sdvb + h * p.sdvh + (int64_t)(unit * kBlk + r) * p.sdvn + quad * 4;
-    if (folding) wait_vm0();                                  // the copies into fold_buf (long since done)
+    if (folding) {
+        wait_vm0();                                           // the copies into fold_buf (long since done)
+        // the chain of pooled levels collapses into one row for dk and one for dv, left where level 1's rows were:
+        // lane (which, four channels) reads its channels of every level and is the only one to write them
+        if (lane < 32) {
+            const int which = lane >> 4, c0 = (lane & 15) * 4;
+            bf16x4 acc = lds_ld8(fold_buf + (2 * (p.fold.depth - 1) + which) * kD + c0);
+#pragma nounroll
+            for (int l = p.fold.depth - 2; l >= 0; l--) acc = fold_step(lds_ld8(fold_buf + (2 * l + which) * kD + c0), acc);
+            lds_st8(fold_buf + which * kD + c0, acc);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
 #pragma unroll
     for (int dt = 0; dt < 4; dt++) {
         bf16x4 ok = cvt4(dk[dt] * kScale), ov = cvt4(dv[dt]);
         if (folding) {
             const int c0 = dt * 16 + quad * 4;
-            const bool two = p.fold.g2k != nullptr, three = p.fold.g3k != nullptr, rot = p.fold.freq != nullptr;
-            ok = fold_math(ok, lds_ld8(fold_buf + c0), two, lds_ld8(fold_buf + 2 * kD + c0), rot,
-                           lds_ld8(fold_buf + kFoldRows + r * kD + c0), three, lds_ld8(fold_buf + 4 * kD + c0));
-            ov = fold_math(ov, lds_ld8(fold_buf + kD + c0), two, lds_ld8(fold_buf + 3 * kD + c0), false, ov, three,
-                           lds_ld8(fold_buf + 5 * kD + c0));
+            ok = fold_math(ok, lds_ld8(fold_buf + c0), p.fold.freq != nullptr, lds_ld8(fold_buf + kFoldRows + r * kD + c0));
+            ov = fold_math(ov, lds_ld8(fold_buf + kD + c0), false, ov);
         }
         st8(kp + dt * 16, ok);
         st8(vp + dt * 16, ov);
@@ -655,7 +636,7 @@ __global__ __launch_bounds__(64 * kDenseWaves) void attn_kside_dense_kernel(KSid
 // meets all of them), which saves that level a pass of its own over Q and dO.
 // ---------------------------------------------------------------------------------------
 constexpr int kGroupWaves = 4;
-constexpr int kGroupSegs = 3;
+constexpr int kGroupSegs = LLSA_MAX_LEVELS;
 constexpr int kGroupMaxBlocks = 64;               // key blocks per group over all its lists (their ids live in one lane each)
 constexpr int kGroupDenseMax = 8;                 // dense blocks are appended up to this many
 
@@ -861,7 +842,7 @@ struct ReduceJob {
     PoolFold fold;           // fine job only
 };
 struct ReduceParams {
-    ReduceJob job[4];
+    ReduceJob job[LLSA_MAX_LEVELS + 1];
     int n_jobs, H, N;
 };
 
@@ -944,7 +925,7 @@ __global__ __launch_bounds__(256) void kside_reduce_kernel(ReduceParams rp) {
                 if (c0 + k < n) acc += v[k];                   // chunk order: the sum does not depend on scheduling
         }
         bf16x4 out = cvt4(which ? acc : acc * kScale);
-        if (jb.fold.g1k != nullptr)
+        if (jb.fold.depth > 0)
             out = fold_pooled(out, jb.fold, which, bh, rp.N, unit * kBlk + r, dt * 16 + quad * 4);
         bf16* dst = which ? jb.dv + b * jb.sdvb + h * jb.sdvh + (int64_t)(unit * kBlk + r) * jb.sdvn
                           : jb.dk + b * jb.sdkb + h * jb.sdkh + (int64_t)(unit * kBlk + r) * jb.sdkn;
@@ -963,7 +944,8 @@ struct DensePlan {
 static DensePlan dense_plan(int B, int H, int N, int levels) {
     const int N1 = N / 16;
     DensePlan d;
-    d.n_tok = (levels == 3) ? N1 / 256 : (levels == 2) ? N1 / 16 : N1;
+    d.n_tok = N1;                                             // tokens of pooled level `levels`
+    for (int l = 1; l < levels; l++) d.n_tok /= 16;
     const int n_units = d.n_tok / 16;
     // Q and dO are streamed n_units / (4 * upw) times (mostly out of an L2: see the kernel); four units per wave would
     // halve that again but leave one wave per SIMD, which measured slower (1.07 ms against 0.93 ms at N = 262144)
@@ -992,26 +974,29 @@ static int64_t align256(int64_t x) { return (x + 255) & ~(int64_t)255; }
 constexpr int64_t kSlotBytes = 8 * kWave * sizeof(f32x4);     // one partial: 16 rows x 64 ch x (dK, dV) fp32
 
 struct BwdWorkspace {
-    int64_t delta, dor, part_fine, part_coarse, part_coarse2, part_dense, total;
-    int64_t slots_fine, slots_coarse, slots_coarse2;            // per (b,h)
+    int64_t delta, dor, part_fine, part_dense, total;
+    int64_t part_level[LLSA_MAX_LEVELS];                        // partial sums of pooled level l (below the coarsest) at [l - 1]
+    int64_t slots_fine, slots_level[LLSA_MAX_LEVELS];           // per (b,h)
 };
 
-static BwdWorkspace bwd_workspace(int B, int H, int N, int T, int T2, int T3, int levels) {
+// topk[0] = T of the fine blocks, topk[l] = T of pooled level l (l < levels)
+static BwdWorkspace bwd_workspace(int B, int H, int N, const int32_t* topk, int levels) {
     const int64_t BH = (int64_t)B * H, N1 = N / 16, N2 = N1 / 16;
     const DensePlan d = dense_plan(B, H, N, levels);
     BwdWorkspace w;
     // a key block has several chunks only if it has more than `chunk` entries, so at most
     // E/chunk such blocks with at most E/chunk + E/chunk chunks in total
-    w.slots_fine = 2 * (N1 * T / LLSA_CHUNK_FINE) + 2;
-    // group-major pooled passes: one partial sum per (group of 16 query blocks, entry of its ancestor's list)
-    w.slots_coarse = (levels >= 2) ? N2 * T2 : 0;
-    w.slots_coarse2 = (levels == 3) ? N2 * T3 : 0;
+    w.slots_fine = 2 * (N1 * topk[0] / LLSA_CHUNK_FINE) + 2;
     int64_t o = 0;
     w.delta = o;        o += align256(BH * N * 4);
     w.dor = o;          o += align256(BH * N * 64 * 2);
     w.part_fine = o;    o += align256(BH * w.slots_fine * kSlotBytes);
-    w.part_coarse = o;  o += align256(BH * w.slots_coarse * kSlotBytes);
-    w.part_coarse2 = o; o += align256(BH * w.slots_coarse2 * kSlotBytes);
+    // group-major pooled passes: one partial sum per (group of 16 query blocks, entry of its ancestor's list)
+    for (int l = 1; l <= LLSA_MAX_LEVELS; l++) {
+        w.slots_level[l - 1] = (l < levels) ? N2 * topk[l] : 0;
+        w.part_level[l - 1] = o;
+        o += align256(BH * w.slots_level[l - 1] * kSlotBytes);
+    }
     w.part_dense = o;   o += align256((int64_t)d.chunks * BH * (d.n_tok / 16) * kSlotBytes);
     w.total = o;
     return w;
@@ -1021,51 +1006,55 @@ static BwdWorkspace bwd_workspace(int B, int H, int N, int T, int T2, int T3, in
 
 using namespace llsa;
 
-extern "C" int64_t llsa_attn_bwd_workspace_bytes(int B, int H, int N, int T, int T2, int T3, int levels) {
-    if (B <= 0 || H <= 0 || N <= 0 || N % 16 != 0 || T <= 0 || levels < 1 || levels > 3) return -1;
-    return bwd_workspace(B, H, N, T, T2, T3, levels).total;
+extern "C" int64_t llsa_attn_bwd_workspace_bytes(int B, int H, int N, const int32_t* topk, int levels) {
+    if (B <= 0 || H <= 0 || N <= 0 || N % 16 != 0 || topk == nullptr || levels < 1 || levels > LLSA_MAX_LEVELS) return -1;
+    for (int l = 0; l < levels; l++)
+        if (topk[l] <= 0) return -1;
+    return bwd_workspace(B, H, N, topk, levels).total;
 }
 
 extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     LLSA_REQUIRE(a != nullptr, "attn_bwd: null args");
-    LLSA_REQUIRE(a->levels >= 1 && a->levels <= 3, "attn_bwd: levels must be 1, 2 or 3");
+    LLSA_REQUIRE(a->levels >= 1 && a->levels <= LLSA_MAX_LEVELS, "attn_bwd: levels must be 1..%d", LLSA_MAX_LEVELS);
     LLSA_REQUIRE(a->B > 0 && a->H > 0 && a->N > 0, "attn_bwd: bad B/H/N");
-    LLSA_REQUIRE(a->dout && a->o && a->lse && a->qr && a->kr && a->vr && a->pkr && a->pvr && a->idx &&
-                     a->off && a->flat && a->dq && a->dk && a->dv && a->dpk && a->dpv && a->workspace,
+    LLSA_REQUIRE(a->dout && a->o && a->lse && a->qr && a->kr && a->vr && a->idx && a->off && a->flat && a->dq && a->dk && a->dv &&
+                     a->workspace,
                  "attn_bwd: null tensor");
     LLSA_REQUIRE(a->T >= 4 && a->T % 4 == 0 && a->T <= a->N / 16, "attn_bwd: topk=%d must be a multiple of 4 and <= N/16", a->T);
-    LLSA_REQUIRE(a->w1 > 0.f && a->cgw1 > 0.f, "attn_bwd: weights must be > 0");
-    if (a->levels == 1) {
-        LLSA_REQUIRE(a->N % 1024 == 0, "attn_bwd: llsa_l1 needs N %% 1024 == 0 (N=%d)", a->N);
-    } else {
-        LLSA_REQUIRE(a->N % (a->levels == 3 ? 262144 : 16384) == 0, "attn_bwd: %d levels need N %% %d == 0 (N=%d)", a->levels,
-                     a->levels == 3 ? 262144 : 16384, a->N);
-        LLSA_REQUIRE(a->pk2r && a->pv2r && a->pidx && a->poff && a->pinv && a->dpk2 && a->dpv2, "attn_bwd: level-2 tensors missing");
-        LLSA_REQUIRE(a->T2 >= 4 && a->T2 % 4 == 0 && a->T2 <= a->N / 256, "attn_bwd: topk2=%d must be a multiple of 4 and <= N/256", a->T2);
-        LLSA_REQUIRE(a->w2 > 0.f, "attn_bwd: token_weight_2 must be > 0");
+    const int64_t mult = coarsest_multiple(a->levels);
+    LLSA_REQUIRE(a->N % mult == 0, "attn_bwd: %d level(s) need N %% %lld == 0 (N=%d)", a->levels, (long long)mult, a->N);
+    int32_t topk[LLSA_MAX_LEVELS] = {a->T, 0, 0, 0};
+    int listed = 0;
+    int64_t span = 256;
+    for (int l = 1; l <= a->levels; l++, span *= 16) {
+        const llsa_bwd_level& lv = a->lvl[l - 1];
+        LLSA_REQUIRE(lv.kr && lv.vr && lv.dk && lv.dv, "attn_bwd: tensors of level %d missing", l);
+        LLSA_REQUIRE(aligned16(lv.kr) && aligned16(lv.vr) && aligned16(lv.dk) && aligned16(lv.dv), "attn_bwd: tensors must be 16-byte aligned");
+        LLSA_REQUIRE(lv.w > 0.f && lv.gw > 0.f, "attn_bwd: the weights of level %d must be > 0", l);
+        if (l < a->levels) {
+            LLSA_REQUIRE(lv.sel && lv.off && lv.inv, "attn_bwd: selection of level %d or its transpose missing", l);
+            LLSA_REQUIRE(lv.T >= 4 && lv.T % 4 == 0 && lv.T <= a->N / span, "attn_bwd: topk of level %d (%d) must be a multiple of 4 and <= N/%lld",
+                         l, lv.T, (long long)span);
+            topk[l] = lv.T;
+            listed += lv.T;
+        }
     }
-    if (a->levels == 3) {
-        LLSA_REQUIRE(a->pk3r && a->pv3r && a->ppidx && a->ppoff && a->ppinv && a->dpk3 && a->dpv3, "attn_bwd: level-3 tensors missing");
-        LLSA_REQUIRE(a->T3 >= 4 && a->T3 % 4 == 0 && a->T3 <= a->N / 4096, "attn_bwd: topk3=%d must be a multiple of 4 and <= N/4096", a->T3);
-        LLSA_REQUIRE(a->w3 > 0.f, "attn_bwd: token_weight_3 must be > 0");
-    }
-    const void* al[] = {a->dout, a->o, a->qr, a->kr, a->vr, a->pkr, a->pvr, a->pk2r, a->pv2r, a->pk3r, a->pv3r,
-                        a->dq, a->dk, a->dv, a->dpk, a->dpv, a->dpk2, a->dpv2, a->dpk3, a->dpv3, a->workspace, a->freq_dq, a->lse};
+    LLSA_REQUIRE(listed + kGroupDenseMax <= kGroupMaxBlocks, "attn_bwd: the topk of the pooled levels together (%d) must not exceed %d", listed,
+                 kGroupMaxBlocks - kGroupDenseMax);
+    const void* al[] = {a->dout, a->o, a->qr, a->kr, a->vr, a->dq, a->dk, a->dv, a->workspace, a->freq_dq, a->lse};
     for (const void* p : al) LLSA_REQUIRE(aligned16(p), "attn_bwd: tensors must be 16-byte aligned");
     const int64_t st[] = {a->sdob, a->sdoh, a->sdon, a->sob, a->soh, a->son};
     for (int64_t s : st) LLSA_REQUIRE(stride_ok(s), "attn_bwd: input row strides must keep rows 16-byte aligned");
     const int64_t so[] = {a->sdqb, a->sdqh, a->sdqn, a->sdkb, a->sdkh, a->sdkn, a->sdvb, a->sdvh, a->sdvn};
     for (int64_t s : so) LLSA_REQUIRE(s % 4 == 0, "attn_bwd: output row strides must keep rows 8-byte aligned");
-    const BwdWorkspace wsp = bwd_workspace(a->B, a->H, a->N, a->T, a->T2, a->T3, a->levels);
+    const BwdWorkspace wsp = bwd_workspace(a->B, a->H, a->N, topk, a->levels);
     LLSA_REQUIRE(a->workspace_bytes >= wsp.total, "attn_bwd: workspace too small (%lld < %lld)", (long long)a->workspace_bytes,
                  (long long)wsp.total);
     LLSA_REQUIRE(a->work != nullptr, "attn_bwd: work list missing");
-    LLSA_REQUIRE(a->levels == 1 || a->T2 + (a->levels == 3 ? a->T3 : 0) + kGroupDenseMax <= kGroupMaxBlocks,
-                 "attn_bwd: topk2 + topk3 must not exceed %d", kGroupMaxBlocks - kGroupDenseMax);
 
     hipStream_t s = (hipStream_t)stream;
-    const int B = a->B, H = a->H, N = a->N, N1 = N / 16, N2 = N1 / 16, N3 = N2 / 16, BH = B * H;
-    const DensePlan d = dense_plan(B, H, N, a->levels);
+    const int B = a->B, H = a->H, N = a->N, N1 = N / 16, N2 = N1 / 16, BH = B * H, L = a->levels;
+    const DensePlan d = dense_plan(B, H, N, L);
     char* ws = (char*)a->workspace;
     float* delta = (float*)(ws + wsp.delta);
     bf16* dor = (bf16*)(ws + wsp.dor);
@@ -1080,6 +1069,10 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     rp.n_jobs = 0;
     rp.H = H;
     rp.N = N;
+    PoolFold no_fold;
+    for (int l = 0; l < LLSA_MAX_LEVELS; l++) no_fold.gk[l] = no_fold.gv[l] = nullptr;
+    no_fold.freq = nullptr;
+    no_fold.depth = 0;
     auto add_job = [&](const KSideParams& p, int chunk, int max_units, int n_chunks) {
         ReduceJob& j = rp.job[rp.n_jobs++];
         j.part = p.part; j.off = p.off; j.work = p.work; j.csr_shift = 0;
@@ -1101,10 +1094,13 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     base.qr = (const bf16*)a->qr; base.dor = dor;
     base.lse = a->lse; base.delta = delta;
     base.H = H; base.N = N; base.chunk_len = 0;
-    base.fold = PoolFold{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
-    const int64_t s1b = (int64_t)H * N1 * 64, s1h = (int64_t)N1 * 64;
-    const int64_t s2b = (int64_t)H * N2 * 64, s2h = (int64_t)N2 * 64;
-    const int64_t s3b = (int64_t)H * N3 * 64, s3h = (int64_t)N3 * 64;
+    base.fold = no_fold;
+    // pooled level l: N / 16^l tokens per (b,h), contiguous (B,H,n,64) gradients
+    auto level_tokens = [&](int l) {
+        int n = N;
+        for (int i = 0; i < l; i++) n /= 16;
+        return n;
+    };
 
     auto run_fine = [&]() {                                   // dK / dV of the fine tokens
         if (!(stages & LLSA_BWD_DKV)) return;
@@ -1116,17 +1112,21 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
         p.dk = (bf16*)a->dk; p.sdkb = a->sdkb; p.sdkh = a->sdkh; p.sdkn = a->sdkn;
         p.dv = (bf16*)a->dv; p.sdvb = a->sdvb; p.sdvh = a->sdvh; p.sdvn = a->sdvn;
         p.n_units = N1; p.w = 1.f;
-        if (fold)
-            p.fold = PoolFold{(const bf16*)a->dpk, (const bf16*)a->dpv, (a->levels >= 2) ? (const bf16*)a->dpk2 : nullptr,
-                              (a->levels >= 2) ? (const bf16*)a->dpv2 : nullptr, (const bf16*)a->freq_dk,
-                              (a->levels == 3) ? (const bf16*)a->dpk3 : nullptr, (a->levels == 3) ? (const bf16*)a->dpv3 : nullptr};
+        if (fold) {
+            for (int l = 0; l < L; l++) {
+                p.fold.gk[l] = (const bf16*)a->lvl[l].dk;
+                p.fold.gv[l] = (const bf16*)a->lvl[l].dv;
+            }
+            p.fold.freq = (const bf16*)a->freq_dk;
+            p.fold.depth = L;
+        }
         const int max_items = N1 * a->T / LLSA_CHUNK_FINE + N1;
         hipLaunchKernelGGL(attn_kside_kernel, dim3(max_items, BH), dim3(64), 0, s, p);
         add_job(p, LLSA_CHUNK_FINE, N1 * a->T / LLSA_CHUNK_FINE + 1, 0);
     };
     // pooled levels under an ancestor's selection, group-major (one launch for all of them, plus the dense level when it is small)
     auto run_groups = [&]() {
-        if (a->levels < 2 || !(stages & LLSA_BWD_DPKV1)) return;
+        if (L < 2 || !(stages & LLSA_BWD_DPKV1)) return;
         GroupParams g;
         g.qr = (const bf16*)a->qr; g.dor = dor; g.lse = a->lse; g.delta = delta;
         g.H = H; g.N = N; g.n_segs = 0; g.n_blocks = 0;
@@ -1137,46 +1137,35 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
             sgm.part = (f32x4*)(ws + part_off); sgm.n_units = n_units; sgm.owner_shift = shift; sgm.cnt = cnt; sgm.slots = slots; sgm.w = w;
             g.n_blocks += cnt;
         };
-        add_seg(a->pkr, a->pvr, a->pidx, a->pinv, wsp.part_coarse, N2, 0, a->T2, wsp.slots_coarse, a->cgw1);
-        if (a->levels == 3) add_seg(a->pk2r, a->pv2r, a->ppidx, a->ppinv, wsp.part_coarse2, N3, 4, a->T3, wsp.slots_coarse2, a->w2);
-        if (d.merged && (stages & LLSA_BWD_DENSE)) {
-            if (a->levels == 3) add_seg(a->pk3r, a->pv3r, nullptr, nullptr, wsp.part_dense, d.n_tok / 16, 0, d.n_tok / 16, 0, a->w3);
-            else add_seg(a->pk2r, a->pv2r, nullptr, nullptr, wsp.part_dense, d.n_tok / 16, 0, d.n_tok / 16, 0, a->w2);
+        for (int l = 1; l < L; l++) {                         // level l: blocks N / 16^(l+1), one list per 16^(l-1) groups
+            const llsa_bwd_level& lv = a->lvl[l - 1];
+            add_seg(lv.kr, lv.vr, lv.sel, lv.inv, wsp.part_level[l - 1], level_tokens(l + 1), 4 * (l - 1), lv.T, wsp.slots_level[l - 1], lv.gw);
         }
+        if (d.merged && (stages & LLSA_BWD_DENSE))
+            add_seg(a->lvl[L - 1].kr, a->lvl[L - 1].vr, nullptr, nullptr, wsp.part_dense, d.n_tok / 16, 0, d.n_tok / 16, 0, a->lvl[L - 1].gw);
         hipLaunchKernelGGL(attn_kside_group_kernel, dim3(N2, BH), dim3(64 * kGroupWaves), 0, s, g);
-        auto add_csr_job = [&](const GroupSeg& sgm, const int* off, void* dk, void* dv, int64_t sb, int64_t sh) {
+        for (int l = 1; l < L; l++) {
+            const GroupSeg& sgm = g.seg[l - 1];
+            const int64_t n = level_tokens(l);
             ReduceJob& j = rp.job[rp.n_jobs++];
-            j.part = sgm.part; j.off = off; j.work = nullptr; j.csr_shift = sgm.owner_shift;
-            j.dk = (bf16*)dk; j.sdkb = sb; j.sdkh = sh; j.sdkn = 64;
-            j.dv = (bf16*)dv; j.sdvb = sb; j.sdvh = sh; j.sdvn = 64;
+            j.part = sgm.part; j.off = a->lvl[l - 1].off; j.work = nullptr; j.csr_shift = sgm.owner_shift;
+            j.dk = (bf16*)a->lvl[l - 1].dk; j.sdkb = (int64_t)H * n * 64; j.sdkh = n * 64; j.sdkn = 64;
+            j.dv = (bf16*)a->lvl[l - 1].dv; j.sdvb = (int64_t)H * n * 64; j.sdvh = n * 64; j.sdvn = 64;
             j.n_units = sgm.n_units; j.chunk = 1; j.max_units = sgm.n_units;
             j.work_stride = 0; j.slot_stride = sgm.slots; j.n_chunks = 0;
-            j.fold = PoolFold{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr};
-        };
-        add_csr_job(g.seg[0], a->poff, a->dpk, a->dpv, s1b, s1h);
-        if (a->levels == 3) add_csr_job(g.seg[1], a->ppoff, a->dpk2, a->dpv2, s2b, s2h);
+            j.fold = no_fold;
+        }
     };
     // dense coarsest level: every unit (16 pooled tokens) meets every query block; the query
     // range is cut into d.chunks pieces whose partial sums are added afterwards
     auto run_dense = [&]() {
         if (!(stages & LLSA_BWD_DENSE)) return;
         KSideParams p = base;
-        if (a->levels == 3) {
-            p.kk = (const bf16*)a->pk3r; p.vv = (const bf16*)a->pv3r;
-            p.dk = (bf16*)a->dpk3; p.dv = (bf16*)a->dpv3;
-            p.sdkb = p.sdvb = s3b; p.sdkh = p.sdvh = s3h;
-            p.w = a->w3;
-        } else if (a->levels == 2) {
-            p.kk = (const bf16*)a->pk2r; p.vv = (const bf16*)a->pv2r;
-            p.dk = (bf16*)a->dpk2; p.dv = (bf16*)a->dpv2;
-            p.sdkb = p.sdvb = s2b; p.sdkh = p.sdvh = s2h;
-            p.w = a->w2;
-        } else {
-            p.kk = (const bf16*)a->pkr; p.vv = (const bf16*)a->pvr;
-            p.dk = (bf16*)a->dpk; p.dv = (bf16*)a->dpv;
-            p.sdkb = p.sdvb = s1b; p.sdkh = p.sdvh = s1h;
-            p.w = a->cgw1;
-        }
+        const llsa_bwd_level& lv = a->lvl[L - 1];
+        p.kk = (const bf16*)lv.kr; p.vv = (const bf16*)lv.vr;
+        p.dk = (bf16*)lv.dk; p.dv = (bf16*)lv.dv;
+        p.sdkb = p.sdvb = (int64_t)H * d.n_tok * 64; p.sdkh = p.sdvh = (int64_t)d.n_tok * 64;
+        p.w = lv.gw;
         p.sdkn = p.sdvn = 64;
         p.off = nullptr; p.flat = nullptr; p.flat_stride = 0; p.work = nullptr; p.work_stride = 0; p.slot_stride = 0;
         p.part = (f32x4*)(ws + wsp.part_dense);

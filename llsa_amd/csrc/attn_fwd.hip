@@ -130,7 +130,7 @@ __global__ __launch_bounds__(256, 4) void attn_fwd_kernel(llsa_attn_fwd_args a) 
     __shared__ __align__(16) bf16 sh[2][kGroup][2 * kTile];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int N1 = a.N / kBlk, N2 = N1 / kBlk, N3 = N2 / kBlk;
+    const int N1 = a.N / kBlk;
     const int lid = xcd_logical_id();
     const int g = (lid % (int)gridDim.x) * 4 + wave;          // < N1: the host checks N1 % 4 == 0
     const int bh = lid / (int)gridDim.x, b = bh / a.H, h = bh % a.H;
@@ -138,51 +138,24 @@ __global__ __launch_bounds__(256, 4) void attn_fwd_kernel(llsa_attn_fwd_args a) 
 
     const bf16* kr = (const bf16*)a.kr + (int64_t)bh * N1 * kTile;
     const bf16* vt = (const bf16*)a.vt + (int64_t)bh * N1 * kTile;
-    const bf16* pk = (const bf16*)a.pkr + (int64_t)bh * N2 * kTile;
-    const bf16* pvt = (const bf16*)a.pvt + (int64_t)bh * N2 * kTile;
-    const bf16* pk2 = (a.levels >= 2) ? (const bf16*)a.pk2r + (int64_t)bh * N3 * kTile : nullptr;
-    const bf16* pv2t = (a.levels >= 2) ? (const bf16*)a.pv2t + (int64_t)bh * N3 * kTile : nullptr;
-    const bf16* pk3 = (a.levels == 3) ? (const bf16*)a.pk3r + (int64_t)bh * (N3 / kBlk) * kTile : nullptr;
-    const bf16* pv3t = (a.levels == 3) ? (const bf16*)a.pv3t + (int64_t)bh * (N3 / kBlk) * kTile : nullptr;
     const int* ip = a.idx + ((int64_t)bh * N1 + g) * a.T;
-    const int* pip = (a.levels >= 2) ? a.pidx + ((int64_t)bh * N2 + g / kBlk) * a.T2 : nullptr;
-    const int* ppip = (a.levels == 3) ? a.ppidx + ((int64_t)bh * N3 + g / (kBlk * kBlk)) * a.T3 : nullptr;
 
-    // shared list: (l2, l3) T2 blocks of level-1 pooled tokens out of the parent's list, (l3) T3 blocks of
-    // level-2 pooled tokens out of the grand-parent's list, then every block of the coarsest level
-    const int n_mid = (a.levels >= 2) ? a.T2 : 0;
-    const int n_mid2 = (a.levels == 3) ? a.T3 : 0;
-    const int n_dense = (a.levels == 3) ? N3 / kBlk : (a.levels == 2) ? N2 / kBlk : N1 / kBlk;
-    const int n_groups = (n_mid + n_mid2 + n_dense) / kGroup; // all three are multiples of kGroup (host checks)
-    const int pmine = (a.levels >= 2 && lane < a.T2) ? pip[lane] : 0;   // first 64 parent entries, entry i in lane i
-    const int ppmine = (a.levels == 3 && lane < a.T3) ? ppip[lane] : 0;
-    const bf16* dense_k = (a.levels == 3) ? pk3 : (a.levels == 2) ? pk2 : pk;
-    const bf16* dense_vt = (a.levels == 3) ? pv3t : (a.levels == 2) ? pv2t : pvt;
-    const float w_dense = (a.levels == 3) ? a.w3 : (a.levels == 2) ? a.w2 : a.w1;
+    // Shared list: for every pooled level below the coarsest the blocks its ancestor group selected (level 1 first),
+    // then every block of the coarsest level.  The selected entries of all levels together (at most 64: the host
+    // checks) live one per lane, entry i in lane i.
+    SharedList sl = shared_list(a.lvl, a.levels, a.N, bh, g, lane);
     bf16* const sh0 = &sh[0][0][0];
-    auto issue_group = [=](int grp) __attribute__((always_inline)) {   // this wave brings in block kGroup*grp + wave
-        const int sblk = kGroup * grp + wave;
-        const bf16 *kb, *vb;
-        if (sblk < n_mid) {
-            const int blk = clampi(sblk < kWave ? __builtin_amdgcn_readlane(pmine, sblk) : pip[sblk], 0, N2 - 1);
-            kb = pk + (int64_t)blk * kTile;
-            vb = pvt + (int64_t)blk * kTile;
-        } else if (sblk < n_mid + n_mid2) {
-            const int j = sblk - n_mid;
-            const int blk = clampi(j < kWave ? __builtin_amdgcn_readlane(ppmine, j) : ppip[j], 0, N3 - 1);
-            kb = pk2 + (int64_t)blk * kTile;
-            vb = pv2t + (int64_t)blk * kTile;
-        } else {
-            const int u = sblk - n_mid - n_mid2;
-            kb = dense_k + (int64_t)u * kTile;
-            vb = dense_vt + (int64_t)u * kTile;
-        }
+    auto issue_group = [&](int grp) __attribute__((always_inline)) {   // this wave brings in block kGroup*grp + wave
+        const SharedBlock sb = shared_block(sl, a.lvl, a.levels, a.N, bh, kGroup * grp + wave);
+        const bf16* kb = (const bf16*)a.lvl[sb.level].kr + sb.tile;
+        const bf16* vb = (const bf16*)a.lvl[sb.level].vt + sb.tile;
         bf16* dst = sh0 + ((grp & 1) * kGroup + wave) * (2 * kTile);
         copy16_global_to_lds(kb + lane * 8, dst);
         copy16_global_to_lds(kb + 512 + lane * 8, dst + 512);
         copy16_global_to_lds(vb + lane * 8, dst + kTile);
         copy16_global_to_lds(vb + 512 + lane * 8, dst + kTile + 512);
     };
+    const int n_groups = sl.n_blocks / kGroup;                // every level's count is a multiple of kGroup (host checks)
     issue_group(0);
     int mine = (lane < min(kWave, a.T)) ? ip[lane] : 0;       // first 64 fine indices, entry i in lane i
 
@@ -203,14 +176,12 @@ __global__ __launch_bounds__(256, 4) void attn_fwd_kernel(llsa_attn_fwd_args a) 
     // ---- shared blocks, out of LDS.  The barrier at the top of round grp says two things: every
     // wave's part of group grp has landed, and every wave is done reading the other buffer
     // (group grp - 1), which the next fetch overwrites.
-    const float w_shared_last = w_dense;
     float w_prev = 1.f;
     for (int grp = 0; grp < n_groups; grp++) {
         wait_vm0();
         __syncthreads();
         // weight(previous segment) / weight(this one); nothing is accumulated before group 0
-        const int sb = kGroup * grp;
-        const float w_here = (sb < n_mid) ? a.w1 : (sb < n_mid + n_mid2) ? a.w2 : w_dense;
+        const float w_here = a.lvl[shared_level(a.lvl, a.levels, kGroup * grp)].w;
         const float wr = (grp == 0) ? 1.f : w_prev / w_here;
         w_prev = w_here;
         // (LDS reads first: the compiler makes every LDS read wait for all copies into LDS that
@@ -221,6 +192,7 @@ __global__ __launch_bounds__(256, 4) void attn_fwd_kernel(llsa_attn_fwd_args a) 
         compute_step(st, bq, ra, wr);
         compute_step(st, bq, rb, 1.f);
     }
+    const float w_shared_last = w_prev;                       // (the coarsest level's weight)
 
     wait_all_mem();     // nothing is in flight here: said for the compiler (see wait_all_mem)
     // ---- fine blocks, private to the wave.  Their indices are fetched 64 at a time, entry i into
@@ -270,32 +242,31 @@ using namespace llsa;
 
 extern "C" int llsa_attn_fwd(const llsa_attn_fwd_args* a, void* stream) {
     LLSA_REQUIRE(a != nullptr, "attn_fwd: null args");
-    LLSA_REQUIRE(a->levels >= 1 && a->levels <= 3, "attn_fwd: levels must be 1, 2 or 3");
+    LLSA_REQUIRE(a->levels >= 1 && a->levels <= LLSA_MAX_LEVELS, "attn_fwd: levels must be 1..%d", LLSA_MAX_LEVELS);
     LLSA_REQUIRE(a->B > 0 && a->H > 0 && a->N > 0, "attn_fwd: bad B/H/N");
-    LLSA_REQUIRE(a->qr && a->kr && a->vt && a->pkr && a->pvt && a->idx && a->o && a->lse, "attn_fwd: null tensor");
+    LLSA_REQUIRE(a->qr && a->kr && a->vt && a->idx && a->o && a->lse, "attn_fwd: null tensor");
     LLSA_REQUIRE(a->T >= 4 && a->T % 4 == 0 && a->T <= a->N / 16, "attn_fwd: topk=%d must be a multiple of 4 and <= N/16", a->T);
-    LLSA_REQUIRE(a->w1 > 0.f, "attn_fwd: token_weight must be > 0");
-    if (a->levels == 1) {
-        LLSA_REQUIRE(a->N % 1024 == 0, "attn_fwd: llsa_l1 needs N %% 1024 == 0 (N=%d): the coarse loop runs over 64-token tiles of N/16 pooled tokens", a->N);
-    } else {
-        if (a->levels == 2)
-            LLSA_REQUIRE(a->N % 16384 == 0, "attn_fwd: llsa_l2 needs N %% 16384 == 0 (N=%d): the level-2 loop runs over 64-token tiles of N/256 pooled tokens", a->N);
-        LLSA_REQUIRE(a->pk2r && a->pv2t && a->pidx, "attn_fwd: level-2 tensors missing");
-        LLSA_REQUIRE(a->T2 >= 4 && a->T2 % 4 == 0 && a->T2 <= a->N / 256, "attn_fwd: topk2=%d must be a multiple of 4 and <= N/256", a->T2);
-        LLSA_REQUIRE(a->w2 > 0.f, "attn_fwd: token_weight_2 must be > 0");
+    const int64_t mult = coarsest_multiple(a->levels);
+    LLSA_REQUIRE(a->N % mult == 0,
+                 "attn_fwd: %d level(s) need N %% %lld == 0 (N=%d): the coarsest level is walked in 64-token tiles of its N/16^levels pooled tokens",
+                 a->levels, (long long)mult, a->N);
+    int listed = 0;
+    int64_t span = 256;                                       // tokens under one block of level l
+    for (int l = 1; l <= a->levels; l++, span *= 16) {
+        const llsa_fwd_level& lv = a->lvl[l - 1];
+        LLSA_REQUIRE(lv.kr && lv.vt && aligned16(lv.kr) && aligned16(lv.vt), "attn_fwd: tiles of level %d missing or not 16-byte aligned", l);
+        LLSA_REQUIRE(lv.w > 0.f, "attn_fwd: the weight of level %d must be > 0", l);
+        if (l < a->levels) {
+            LLSA_REQUIRE(lv.sel != nullptr, "attn_fwd: selection of level %d missing", l);
+            LLSA_REQUIRE(lv.T >= 4 && lv.T % 4 == 0 && lv.T <= a->N / span, "attn_fwd: topk of level %d (%d) must be a multiple of 4 and <= N/%lld",
+                         l, lv.T, (long long)span);
+            listed += lv.T;
+        }
     }
-    if (a->levels == 3) {
-        LLSA_REQUIRE(a->N % 262144 == 0, "attn_fwd: three levels need N %% 262144 == 0 (N=%d): the level-3 loop runs over 64-token tiles of N/4096 pooled tokens", a->N);
-        LLSA_REQUIRE(a->pk3r && a->pv3t && a->ppidx, "attn_fwd: level-3 tensors missing");
-        LLSA_REQUIRE(a->T3 >= 4 && a->T3 % 4 == 0 && a->T3 <= a->N / 4096, "attn_fwd: topk3=%d must be a multiple of 4 and <= N/4096", a->T3);
-        LLSA_REQUIRE(a->w3 > 0.f && aligned16(a->pk3r) && aligned16(a->pv3t), "attn_fwd: token_weight_3 must be > 0, level-3 tiles 16-byte aligned");
-    }
-    LLSA_REQUIRE(aligned16(a->qr) && aligned16(a->kr) && aligned16(a->vt) && aligned16(a->pkr) && aligned16(a->pvt) &&
-                     aligned16(a->pk2r) && aligned16(a->pv2t) && aligned16(a->o),
-                 "attn_fwd: tensors must be 16-byte aligned");
+    LLSA_REQUIRE(listed <= 64, "attn_fwd: the topk of the pooled levels together (%d) must not exceed 64", listed);
+    LLSA_REQUIRE(aligned16(a->qr) && aligned16(a->kr) && aligned16(a->vt) && aligned16(a->o), "attn_fwd: tensors must be 16-byte aligned");
     LLSA_REQUIRE((a->sob % 4 == 0) && (a->soh % 4 == 0) && (a->son % 4 == 0), "attn_fwd: rows of o must be 8-byte aligned");
     const int N1 = a->N / 16;
-    hipLaunchKernelGGL(attn_fwd_kernel, dim3((N1 + 3) / 4, a->B * a->H), dim3(256), 0,
-                       (hipStream_t)stream, *a);
+    hipLaunchKernelGGL(attn_fwd_kernel, dim3((N1 + 3) / 4, a->B * a->H), dim3(256), 0, (hipStream_t)stream, *a);
     return launch_status("attn_fwd");
 }

@@ -147,12 +147,78 @@ __host__ __device__ inline int work_tail_len(int Kb) { return (Kb + 3) & ~3; }
 
 constexpr int kGroup = 4;      // pooled blocks per LDS buffer in the query-side attention kernels (one per wave)
 
+__device__ __forceinline__ int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+// The blocks of the pooled levels a group of query blocks reads, as the forward and the dQ kernel walk them:
+// level 1's selected blocks, level 2's, ..., then every block of the coarsest level.  `Level` is llsa_fwd_level
+// or llsa_bwd_level (fields sel, T).  Blocks of level l per (b,h): N / 16^(l+1).
+struct SharedList {
+    int mine;          // lane i: the i-th selected entry over all levels below the coarsest
+    int n_listed;      // how many of those there are
+    int n_blocks;      // n_listed + blocks of the coarsest level
+};
+struct SharedBlock {
+    int level;         // index into lvl[] (pooled level - 1)
+    int64_t tile;      // element offset of the block's tile inside the level's tile array
+};
+__host__ __device__ inline int64_t coarsest_multiple(int levels) {       // N must be a multiple of 64 * 16^levels
+    int64_t m = 64;
+    for (int l = 0; l < levels; l++) m *= 16;
+    return m;
+}
+template <typename Level>
+__device__ __forceinline__ SharedList shared_list(const Level* lvl, int levels, int N, int bh, int g, int lane) {
+    SharedList sl;
+    sl.mine = 0;
+    int base = 0, nb = N / (kBlk * kBlk);                     // blocks of level 1 per (b,h) = owners of its selection
+    int owner = g / kBlk;
+    for (int l = 1; l < levels; l++) {
+        const int T = lvl[l - 1].T;
+        if (lane >= base && lane < base + T) sl.mine = lvl[l - 1].sel[((int64_t)bh * nb + owner) * T + (lane - base)];
+        base += T;
+        nb /= kBlk;
+        owner /= kBlk;
+    }
+    sl.n_listed = base;
+    sl.n_blocks = base + nb;                                  // nb is now the block count of the coarsest level
+    return sl;
+}
+// which entry of lvl[] the i-th block of the walk belongs to (i is wave-uniform)
+template <typename Level>
+__device__ __forceinline__ int shared_level(const Level* lvl, int levels, int i) {
+    int base = 0, l = 1;
+    while (l < levels && i >= base + lvl[l - 1].T) {
+        base += lvl[l - 1].T;
+        l++;
+    }
+    return l - 1;
+}
+template <typename Level>
+__device__ __forceinline__ SharedBlock shared_block(const SharedList& sl, const Level* lvl, int levels, int N, int bh, int i) {
+    SharedBlock sb;
+    int base = 0, nb = N / (kBlk * kBlk), l = 1;
+    while (l < levels && i >= base + lvl[l - 1].T) {
+        base += lvl[l - 1].T;
+        nb /= kBlk;
+        l++;
+    }
+    int blk;
+    if (l < levels) blk = clampi(__builtin_amdgcn_readlane(sl.mine, i), 0, nb - 1);      // (i < 64 there)
+    else blk = i - sl.n_listed;
+    sb.level = l - 1;
+    sb.tile = ((int64_t)bh * nb + blk) * kTile;
+    return sb;
+}
+
 // 16- and 8-byte reads that are LDS reads by construction (ds_read_b128 / ds_read_b64)
 __device__ __forceinline__ bf16x8 lds_ld16(const bf16* p) {
     return *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>((const __attribute__((address_space(3))) bf16*)p);
 }
 __device__ __forceinline__ bf16x4 lds_ld8(const bf16* p) {
     return *reinterpret_cast<const __attribute__((address_space(3))) bf16x4*>((const __attribute__((address_space(3))) bf16*)p);
+}
+__device__ __forceinline__ void lds_st8(bf16* p, bf16x4 v) {
+    *reinterpret_cast<__attribute__((address_space(3))) bf16x4*>((__attribute__((address_space(3))) bf16*)p) = v;
 }
 
 // XCD-aware workgroup order.  The 8 XCDs of the chip each have a private L2 and receive
@@ -168,7 +234,5 @@ __device__ __forceinline__ int xcd_logical_id() {
     const int q = total / kXcds, rem = total % kXcds;
     return xcd * q + (xcd < rem ? xcd : rem) + slot;
 }
-
-__device__ __forceinline__ int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
 
 }  // namespace llsa

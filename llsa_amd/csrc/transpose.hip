@@ -218,21 +218,34 @@ __global__ __launch_bounds__(kTrThreads) void tr_scatter_kernel(const int* __res
 }
 
 // Puts every segment of `flat` in ascending order: one wave per key block sets one bit per
-// entry in a private LDS bitmap over the query blocks and reads the bits back in order.
+// entry in a private LDS bitmap over the query blocks and reads the bits back in order.  Only the
+// words between the smallest and the largest query block of the segment are cleared and read.
 __global__ __launch_bounds__(256) void sort_segments_kernel(const int* __restrict__ offsets, int* __restrict__ flat, int Mb,
                                                             int Kb, int T) {
     __builtin_amdgcn_s_setprio(3);
-    HIP_DYNAMIC_SHARED(unsigned, bitmaps)                     // 4 waves x words
+    HIP_DYNAMIC_SHARED(unsigned, bitmaps)                     // waves x words
     const int words = (Mb + 31) / 32;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int bh = blockIdx.y, n = blockIdx.x * 4 + wave;
+    const int bh = blockIdx.y, n = blockIdx.x * (int)(blockDim.x >> 6) + wave;
     if (n >= Kb) return;                                      // no workgroup barrier below
     flat += (int64_t)bh * Mb * T;
     const int* o = offsets + (int64_t)bh * (Kb + 1) + n;
     const int s = o[0], e = o[1];
     if (e - s <= 1) return;
+    int qlo = Mb - 1, qhi = 0;
+    for (int i = s + lane; i < e; i += kWave) {
+        const int q = clampi(flat[i], 0, Mb - 1);
+        qlo = q < qlo ? q : qlo;
+        qhi = q > qhi ? q : qhi;
+    }
+    for (int d = 1; d < kWave; d <<= 1) {
+        const int a = __shfl_xor(qlo, d), b = __shfl_xor(qhi, d);
+        qlo = a < qlo ? a : qlo;
+        qhi = b > qhi ? b : qhi;
+    }
+    const int w_lo = qlo >> 5, w_hi = (qhi >> 5) + 1;         // the same in every lane
     unsigned* bm = bitmaps + wave * words;
-    for (int w = lane; w < words; w += kWave) bm[w] = 0u;
+    for (int w = w_lo + lane; w < w_hi; w += kWave) bm[w] = 0u;
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     for (int i = s + lane; i < e; i += kWave) {
@@ -242,8 +255,8 @@ __global__ __launch_bounds__(256) void sort_segments_kernel(const int* __restric
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
     int out = s;
-    for (int wb = 0; wb < words; wb += kWave) {
-        unsigned wd = (wb + lane < words) ? bm[wb + lane] : 0u;
+    for (int wb = w_lo; wb < w_hi; wb += kWave) {
+        unsigned wd = (wb + lane < w_hi) ? bm[wb + lane] : 0u;
         const int cnt = __popc(wd);
         const int incl2 = wave_incl_scan(cnt, lane);
         int oo = out + incl2 - cnt;
@@ -298,8 +311,11 @@ extern "C" int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int3
     static_assert(5 * kTrWaves <= 128, "wave totals must fit their LDS slot");
     LLSA_REQUIRE(lds <= 160 * 1024 || (work != nullptr && (int64_t)Mb * T >= 4 * kTrPart),
                  "transpose_indices: Kb=%d needs %zu bytes of LDS (limit 163840)", Kb, lds);
-    const size_t lds_sort = sizeof(unsigned) * 4 * ((size_t)(Mb + 31) / 32);
-    LLSA_REQUIRE(lds_sort <= 64 * 1024, "transpose_indices: Mb=%d needs %zu bytes of LDS for the segment sort", Mb, lds_sort);
+    // the segment sort keeps one bitmap over the query blocks per wave: four waves a workgroup while they fit, then two, then one
+    const size_t bitmap = sizeof(unsigned) * ((size_t)(Mb + 31) / 32);
+    const int sort_waves = 4 * bitmap <= 160 * 1024 ? 4 : 2 * bitmap <= 160 * 1024 ? 2 : 1;
+    const size_t lds_sort = bitmap * sort_waves;
+    LLSA_REQUIRE(lds_sort <= 160 * 1024, "transpose_indices: Mb=%d needs %zu bytes of LDS for the segment sort (limit 163840)", Mb, lds_sort);
     const int64_t E = (int64_t)Mb * T;
     const bool split = work != nullptr && E >= 4 * kTrPart;
     if (!split && lds > 64 * 1024) {
@@ -320,8 +336,12 @@ extern "C" int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int3
         hipLaunchKernelGGL(HIP_KERNEL_NAME(transpose_indices_kernel<false>), dim3(B * H), dim3(kTrThreads), lds, st, idx, offsets, flat,
                            work, Mb, Kb, T, chunk, wl);
     }
-    hipLaunchKernelGGL(sort_segments_kernel, dim3((Kb + 3) / 4, B * H), dim3(256), lds_sort, (hipStream_t)stream,
-                       (const int*)offsets, flat, Mb, Kb, T);
+    if (lds_sort > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void*)sort_segments_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_sort);
+        if (e != hipSuccess) return fail(-101, "transpose_indices: cannot raise dynamic LDS to %zu bytes: %s", lds_sort, hipGetErrorString(e));
+    }
+    hipLaunchKernelGGL(sort_segments_kernel, dim3((Kb + sort_waves - 1) / sort_waves, B * H), dim3(64 * sort_waves), lds_sort,
+                       (hipStream_t)stream, (const int*)offsets, flat, Mb, Kb, T);
     if (inv != nullptr)
         hipLaunchKernelGGL(inverse_positions_kernel, dim3((unsigned)((E + 255) / 256), B * H), dim3(256), 0, (hipStream_t)stream, idx,
                            (const int*)offsets, (const int*)flat, inv, Mb, Kb, T);

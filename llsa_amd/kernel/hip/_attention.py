@@ -69,14 +69,15 @@ def attn_fwd(q, k, v, pk, pv, indices, token_weight, pk2=None, pv2=None, p_indic
     o = torch.empty_like(q) if rows_ok8(q) else torch.empty(q.shape, device=q.device, dtype=q.dtype)
     lse = torch.empty(B, H, N, device=q.device, dtype=torch.float32)
     a = AttnFwdArgs()
-    a.qr, a.kr, a.vt, a.pkr, a.pvt = (tl[n].data_ptr() for n in ("qr", "kr", "vt", "pkr", "pvt"))
-    if levels == 2:
-        a.pk2r, a.pv2t, a.pidx = tl["pk2r"].data_ptr(), tl["pv2t"].data_ptr(), pidx.data_ptr()
+    a.qr, a.kr, a.vt = (tl[n].data_ptr() for n in ("qr", "kr", "vt"))
     a.idx = idx.data_ptr()
     a.o, (a.sob, a.soh, a.son) = o.data_ptr(), s3(o)
     a.lse = lse.data_ptr()
-    a.B, a.H, a.N, a.T, a.T2, a.levels = B, H, N, T, T2, levels
-    a.w1, a.w2 = float(token_weight), float(token_weight_2)
+    a.B, a.H, a.N, a.T, a.levels = B, H, N, T, levels
+    a.lvl[0].kr, a.lvl[0].vt, a.lvl[0].w = tl["pkr"].data_ptr(), tl["pvt"].data_ptr(), float(token_weight)
+    if levels == 2:
+        a.lvl[0].sel, a.lvl[0].T = pidx.data_ptr(), T2
+        a.lvl[1].kr, a.lvl[1].vt, a.lvl[1].w = tl["pk2r"].data_ptr(), tl["pv2t"].data_ptr(), float(token_weight_2)
     lib.check(lib.attn_fwd(C.byref(a), stream_of(lib, q)), "attn_fwd")
     return o, lse
 
@@ -122,36 +123,37 @@ def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_wei
     mk = lambda t: torch.empty_like(t) if rows_ok8(t) else torch.empty(t.shape, device=t.device, dtype=t.dtype)
     dq, dk, dv = mk(q), mk(k), mk(v)
     dpk, dpv = torch.empty_like(pk, memory_format=torch.contiguous_format), torch.empty_like(pv, memory_format=torch.contiguous_format)
-    ws_bytes = lib.attn_bwd_workspace_bytes(B, H, N, T, T2, 0, levels)
+    ws_bytes = lib.attn_bwd_workspace_bytes(B, H, N, (C.c_int32 * levels)(*([T, T2][:levels])), levels)
     ws = torch.empty(ws_bytes, device=q.device, dtype=torch.uint8)
     a = AttnBwdArgs()
     a.dout, (a.sdob, a.sdoh, a.sdon) = do.data_ptr(), s3(do)
     a.o, (a.sob, a.soh, a.son) = o.data_ptr(), s3(o)
     lse = lse.contiguous()
     a.lse = lse.data_ptr()
-    for n in ("qr", "kr", "vr", "pkr", "pvr"):
+    for n in ("qr", "kr", "vr"):
         setattr(a, n, tl[n].data_ptr())
     a.idx, a.off, a.flat, a.work = idx.data_ptr(), off.data_ptr(), flat.data_ptr(), work.data_ptr()
     a.dq, (a.sdqb, a.sdqh, a.sdqn) = dq.data_ptr(), s3(dq)
     a.dk, (a.sdkb, a.sdkh, a.sdkn) = dk.data_ptr(), s3(dk)
     a.dv, (a.sdvb, a.sdvh, a.sdvn) = dv.data_ptr(), s3(dv)
-    a.dpk, a.dpv = dpk.data_ptr(), dpv.data_ptr()
+    l1 = a.lvl[0]
+    l1.kr, l1.vr, l1.dk, l1.dv = tl["pkr"].data_ptr(), tl["pvr"].data_ptr(), dpk.data_ptr(), dpv.data_ptr()
+    l1.w, l1.gw = float(token_weight), float(coarse_grad_weight)
     outs = [dq, dk, dv, dpk, dpv]
     if levels == 2:
         dpk2 = torch.empty_like(pk2, memory_format=torch.contiguous_format)
         dpv2 = torch.empty_like(pv2, memory_format=torch.contiguous_format)
-        for n in ("pk2r", "pv2r"):
-            setattr(a, n, tl[n].data_ptr())
-        a.pidx, a.poff, a.pinv = pidx.data_ptr(), poff.data_ptr(), pinv.data_ptr()
-        a.dpk2, a.dpv2 = dpk2.data_ptr(), dpv2.data_ptr()
+        l1.sel, l1.off, l1.inv, l1.T = pidx.data_ptr(), poff.data_ptr(), pinv.data_ptr(), T2
+        l2 = a.lvl[1]
+        l2.kr, l2.vr, l2.dk, l2.dv = tl["pk2r"].data_ptr(), tl["pv2r"].data_ptr(), dpk2.data_ptr(), dpv2.data_ptr()
+        l2.w = l2.gw = float(token_weight_2)
         outs += [dpk2, dpv2]
     a.workspace, a.workspace_bytes = ws.data_ptr(), ws_bytes
     if freq_dq is not None:
         require_bf16(freq_dq)
         freq_dq = freq_dq.contiguous()
         a.freq_dq = freq_dq.data_ptr()
-    a.B, a.H, a.N, a.T, a.T2, a.levels = B, H, N, T, T2, levels
-    a.w1, a.w2, a.cgw1 = float(token_weight), float(token_weight_2), float(coarse_grad_weight)
+    a.B, a.H, a.N, a.T, a.levels = B, H, N, T, levels
     if freq_dk is not None:
         require_bf16(freq_dk)
         freq_dk = freq_dk.contiguous()

@@ -21,7 +21,7 @@ import ctypes as C
 import torch
 from torch.autograd import Function
 
-from ..._lib import CHUNK_FINE, AttnBwdArgs, AttnFwdArgs, PoolItem, current_lib
+from ..._lib import CHUNK_FINE, MAX_LEVELS, AttnBwdArgs, AttnFwdArgs, PoolItem, current_lib
 
 _side = {}          # device -> (second stream, two events)
 _SIDE_STREAM_MIN_TOKENS = 1 << 17
@@ -37,12 +37,14 @@ def _align(n, a):
 
 class _Layout:
     """Offsets (in elements) of everything the forward produces, inside one bf16 arena and one
-    int32 arena; every section is contiguous (B*H, ...) and starts 256-byte aligned."""
+    int32 arena; every section is contiguous (B*H, ...) and starts 256-byte aligned.  Level 0 is the
+    tokens themselves, level l = 1..L the pooled levels (n[l] = N / 16^l tokens each)."""
 
-    def __init__(self, lib, B, H, N, levels, T, T2, grad, T3=0):
+    def __init__(self, lib, B, H, N, topks, grad):
         BH = B * H
-        n1, n2 = N // 16, N // 256
-        self.n1, self.n2 = n1, n2
+        L = len(topks)
+        n = [N // 16 ** l for l in range(L + 2)]
+        self.n, self.L = n, L
         o = 0
 
         def take(rows_per_bh, width, on=True):
@@ -53,17 +55,14 @@ class _Layout:
             o = _align(o + BH * rows_per_bh * width, 128)
             return at
 
-        l2, l3 = levels >= 2, levels == 3
-        self.pq, self.pk, self.pv = take(n1, 64), take(n1, 64), take(n1, 64)
-        self.pq2, self.pk2, self.pv2 = take(n2, 64, l2), take(n2, 64, l2), take(n2, 64, l2)
-        self.qr, self.kr, self.vr, self.vt = take(n1, 1024), take(n1, 1024), take(n1, 1024, grad), take(n1, 1024)
-        self.pkr, self.pvr, self.pvt = take(n2, 1024), take(n2, 1024, grad), take(n2, 1024)
-        n3 = max(n2 // 16, 1)
-        self.pk2r, self.pv2r, self.pv2t = take(n3, 1024, l2), take(n3, 1024, l2 and grad), take(n3, 1024, l2)
-        n4 = max(n3 // 16, 1)
-        self.n3 = n3
-        self.pq3, self.pk3, self.pv3 = take(n3, 64, l3), take(n3, 64, l3), take(n3, 64, l3)
-        self.pk3r, self.pv3r, self.pv3t = take(n4, 1024, l3), take(n4, 1024, l3 and grad), take(n4, 1024, l3)
+        # pooled rows of q, k, v per level (index l - 1), then operand tiles: level 0 (the tokens) and the pooled levels
+        self.pq = [take(n[l], 64) for l in range(1, L + 1)]
+        self.pk = [take(n[l], 64) for l in range(1, L + 1)]
+        self.pv = [take(n[l], 64) for l in range(1, L + 1)]
+        self.qr, self.kr, self.vr, self.vt = take(n[1], 1024), take(n[1], 1024), take(n[1], 1024, grad), take(n[1], 1024)
+        self.pkr = [take(n[l + 1], 1024) for l in range(1, L + 1)]
+        self.pvr = [take(n[l + 1], 1024, grad) for l in range(1, L + 1)]
+        self.pvt = [take(n[l + 1], 1024) for l in range(1, L + 1)]
         self.n_bf16 = o
 
         o = 0
@@ -76,36 +75,37 @@ class _Layout:
             o = _align(o + BH * per_bh, 64)
             return at
 
-        self.wl_f = lib.work_list_len(n1, n1, T, CHUNK_FINE)
-        self.idx, self.pidx, self.ppidx = take_i(n1 * T), take_i(n2 * T2, l2), take_i(n3 * T3, l3)
-        self.off, self.flat, self.work = take_i(n1 + 1, grad), take_i(n1 * T, grad), take_i(self.wl_f, grad)
-        self.poff, self.pflat, self.pinv = (take_i(n2 + 1, grad and l2), take_i(n2 * T2, grad and l2),
-                                            take_i(n2 * T2, grad and l2))
-        self.ppoff, self.ppflat, self.ppinv = (take_i(n3 + 1, grad and l3), take_i(n3 * T3, grad and l3),
-                                               take_i(n3 * T3, grad and l3))
+        self.wl_f = lib.work_list_len(n[1], n[1], topks[0], CHUNK_FINE)
+        # sel[0] = idx (fine blocks per query block), sel[l] = blocks of level l per group of 16^(l+1) queries
+        self.sel = [take_i(n[l + 1] * topks[l]) for l in range(L)]
+        self.off = [take_i(n[l + 1] + 1, grad) for l in range(L)]
+        self.flat = [take_i(n[l + 1] * topks[l], grad) for l in range(L)]
+        self.work = take_i(self.wl_f, grad)
+        self.inv = [None] + [take_i(n[l + 1] * topks[l], grad) for l in range(1, L)]
         self.n_i32 = o
         # backward arena (bytes): pooled gradients, then the kernels' workspace
-        self.ws_bytes = lib.attn_bwd_workspace_bytes(B, H, N, T, T2, T3, levels)
-        self.dpk = 0
-        self.dpv = _align(BH * n1 * 128, 256)
-        self.dpk2 = self.dpv + _align(BH * n1 * 128, 256)
-        self.dpv2 = self.dpk2 + _align(BH * n2 * 128, 256)
-        self.dpk3 = self.dpv2 + _align(BH * n2 * 128, 256)
-        self.dpv3 = self.dpk3 + _align(BH * n3 * 128, 256)
-        self.ws = self.dpv3 + _align(BH * n3 * 128, 256)
+        self.ws_bytes = lib.attn_bwd_workspace_bytes(B, H, N, (C.c_int32 * L)(*topks), L)
+        o = 0
+        self.dpk, self.dpv = [], []
+        for l in range(1, L + 1):
+            self.dpk.append(o)
+            o += _align(BH * n[l] * 128, 256)
+            self.dpv.append(o)
+            o += _align(BH * n[l] * 128, 256)
+        self.ws = o
         self.n_bwd = self.ws + self.ws_bytes
 
 
 _layouts = {}
 
 
-def _layout(lib, B, H, N, levels, T, T2, grad, T3=0):
-    key = (lib.path, B, H, N, levels, T, T2, grad, T3)
+def _layout(lib, B, H, N, topks, grad):
+    key = (lib.path, B, H, N, topks, grad)
     lay = _layouts.get(key)
     if lay is None:
         if len(_layouts) > 64:
             _layouts.clear()
-        lay = _layouts[key] = _Layout(lib, B, H, N, levels, T, T2, grad, T3)
+        lay = _layouts[key] = _Layout(lib, B, H, N, topks, grad)
     return lay
 
 
@@ -122,13 +122,15 @@ def _check(lib, rc, what):
 
 
 class LlsaFused(Function):
-    """forward(q, k, v, levels, topk1, topk2, block_size, freq, gamma_q, gamma_k, eps) -> o
+    """forward(q, k, v, topks, block_size, freq, gamma_q, gamma_k, eps) -> o
 
+    topks: one entry per pooled level, (topk1, topk2, ...): the fine blocks a query block keeps, then the blocks of
+    pooled level 1, 2, ... its ancestor groups keep; len(topks) = 1 is llsa_l1, 2 is llsa_l2.
     gamma_q / gamma_k ((64,) fp32 or None): RMS-normalise q / k over the head dimension first (the
     qk-norm of the reference's attention processor), inside the pooling pass; they receive gradients."""
 
     @staticmethod
-    def forward(ctx, q, k, v, levels, topk1, topk2, block_size, freq, gamma_q=None, gamma_k=None, eps=1e-5, topk3=0):
+    def forward(ctx, q, k, v, topks, block_size, freq, gamma_q=None, gamma_k=None, eps=1e-5):
         lib = current_lib()
         if block_size != 16:
             raise NotImplementedError("block_size must be 16")
@@ -142,19 +144,19 @@ class LlsaFused(Function):
         if k.shape != q.shape or v.shape != q.shape:
             raise ValueError("self-attention only: q, k, v must have the same shape")
         B, H, N, _ = q.shape
-        mult = {1: 1024, 2: 16384, 3: 262144}[levels]
+        L = len(topks)
+        if not 1 <= L <= MAX_LEVELS:
+            raise ValueError(f"1 to {MAX_LEVELS} pooled levels (got {L})")
+        mult = 64 * 16 ** L
         if N % mult != 0:
-            raise ValueError(f"llsa_l{levels} needs a token count that is a multiple of {mult} (got {N})")
-        n1, n2, n3 = N // 16, N // 256, N // 4096
-        T = min(topk1, n1)
-        T2 = min(topk2, n2) if levels >= 2 else 0
-        T3 = min(topk3, n3) if levels == 3 else 0
+            raise ValueError(f"llsa_l{L} needs a token count that is a multiple of {mult} (got {N})")
+        topks = tuple(min(int(t), N // 16 ** (l + 1)) for l, t in enumerate(topks))
         rope = freq is not None
         if rope:
             if freq.dtype != torch.bfloat16 or tuple(freq.shape) != (N, 64):
                 raise ValueError("rope table must be bf16 (N, 64)")
             freq = freq.contiguous()
-        grad = any(ctx.needs_input_grad[:3]) or ctx.needs_input_grad[8] or ctx.needs_input_grad[9]
+        grad = any(ctx.needs_input_grad[:3]) or ctx.needs_input_grad[6] or ctx.needs_input_grad[7]
         q, k, v = (t if _rows_ok(t) else t.contiguous() for t in (q, k, v))
         gq = gk = None
         if gamma_q is not None:
@@ -163,7 +165,8 @@ class LlsaFused(Function):
             gk = gamma_k.detach().to(device=q.device, dtype=torch.float32).contiguous()
         if any(g is not None and g.numel() != 64 for g in (gq, gk)):
             raise ValueError("qk-norm weights must have 64 entries")
-        lay = _layout(lib, B, H, N, levels, T, T2, grad, T3)
+        lay = _layout(lib, B, H, N, topks, grad)
+        n = lay.n
         dev = q.device
         A = torch.empty(lay.n_bf16, device=dev, dtype=torch.bfloat16)
         I = torch.empty(lay.n_i32, device=dev, dtype=torch.int32)
@@ -173,41 +176,35 @@ class LlsaFused(Function):
         pa = lambda off: None if off is None else a0 + 2 * off
         pi = lambda off: None if off is None else i0 + 4 * off
         stream = _stream(lib, q)
-        l2, l3 = levels >= 2, levels == 3
+        at = lambda lst, l: pa(lst[l - 1]) if l <= L else None      # section of pooled level l (None beyond the last)
 
-        two = l2 and not l3     # two levels: the tiles of the level-2 rows come out of the same pass (with three, a second one makes them)
+        # The pyramid.  One pass over q, k, v gives the rows of levels 1 and 2 and the tiles of levels 0, 1, 2; every
+        # further pass starts from the rows of level 2p and gives rows and tiles of levels 2p + 1 and 2p + 2.
         items = (PoolItem * 3)(
-            PoolItem(q.data_ptr(), q.stride(0), q.stride(1), q.stride(2), N, int(rope), pa(lay.pq), pa(lay.pq2), pa(lay.qr),
+            PoolItem(q.data_ptr(), q.stride(0), q.stride(1), q.stride(2), N, int(rope), at(lay.pq, 1), at(lay.pq, 2), pa(lay.qr),
                      None, None, None, None, None if gq is None else gq.data_ptr(), float(eps), 0, None, None),
-            PoolItem(k.data_ptr(), k.stride(0), k.stride(1), k.stride(2), N, int(rope), pa(lay.pk), pa(lay.pk2), pa(lay.kr),
-                     None, pa(lay.pkr), None, None, None if gk is None else gk.data_ptr(), float(eps), 0,
-                     pa(lay.pk2r) if two else None, None),
-            PoolItem(v.data_ptr(), v.stride(0), v.stride(1), v.stride(2), N, 0, pa(lay.pv), pa(lay.pv2), pa(lay.vr),
-                     pa(lay.vt), pa(lay.pvr), pa(lay.pvt), None, None, 0.0, 0,
-                     pa(lay.pv2r) if two else None, pa(lay.pv2t) if two else None))
+            PoolItem(k.data_ptr(), k.stride(0), k.stride(1), k.stride(2), N, int(rope), at(lay.pk, 1), at(lay.pk, 2), pa(lay.kr),
+                     None, at(lay.pkr, 1), None, None, None if gk is None else gk.data_ptr(), float(eps), 0, at(lay.pkr, 2), None),
+            PoolItem(v.data_ptr(), v.stride(0), v.stride(1), v.stride(2), N, 0, at(lay.pv, 1), at(lay.pv, 2), pa(lay.vr),
+                     pa(lay.vt), at(lay.pvr, 1), at(lay.pvt, 1), None, None, 0.0, 0, at(lay.pvr, 2), at(lay.pvt, 2)))
         _check(lib, lib.pool_pyramid_fwd(items, 3, freq.data_ptr() if rope else None, B, H, stream), "pool_pyramid")
-        if two:
-            _check(lib, lib.topk_dense(pa(lay.pq2), pa(lay.pk2), pi(lay.pidx), B, H, n2, T2, 1, stream), "gen_sparse_indices")
-            _check(lib, lib.topk_sparse(pa(lay.pq), pa(lay.pk), pi(lay.pidx), pi(lay.idx), B, H, n1, T, T2, stream),
-                   "compute_topk_indices_sparse")
-        elif l2:
-            s2 = (H * n2 * 64, n2 * 64, 64)
-            # the level-2 rows again: their tiles and (three levels) the level-3 rows with theirs
-            items2 = (PoolItem * 3)(
-                PoolItem(pa(lay.pk2), *s2, n2, 0, pa(lay.pk3), None, pa(lay.pk2r), None, pa(lay.pk3r), None, None),
-                PoolItem(pa(lay.pv2), *s2, n2, 0, pa(lay.pv3), None, pa(lay.pv2r), pa(lay.pv2t), pa(lay.pv3r), pa(lay.pv3t), None),
-                PoolItem(pa(lay.pq2), *s2, n2, 0, pa(lay.pq3), None, None, None, None, None, None))
-            _check(lib, lib.pool_pyramid_fwd(items2, 3 if l3 else 2, None, B, H, stream), "pool_pyramid (level-2 tiles)")
-            if l3:
-                _check(lib, lib.topk_dense(pa(lay.pq3), pa(lay.pk3), pi(lay.ppidx), B, H, n3, T3, 1, stream), "gen_sparse_indices")
-                _check(lib, lib.topk_sparse(pa(lay.pq2), pa(lay.pk2), pi(lay.ppidx), pi(lay.pidx), B, H, n2, T2, T3, stream),
-                       "compute_topk_indices_sparse (level 2)")
-            else:
-                _check(lib, lib.topk_dense(pa(lay.pq2), pa(lay.pk2), pi(lay.pidx), B, H, n2, T2, 1, stream), "gen_sparse_indices")
-            _check(lib, lib.topk_sparse(pa(lay.pq), pa(lay.pk), pi(lay.pidx), pi(lay.idx), B, H, n1, T, T2, stream),
-                   "compute_topk_indices_sparse")
-        else:
-            _check(lib, lib.topk_dense(pa(lay.pq), pa(lay.pk), pi(lay.idx), B, H, n1, T, 1, stream), "gen_sparse_indices")
+        for l0 in range(2, L, 2):               # rows of level l0 -> levels l0 + 1, l0 + 2
+            s = (H * n[l0] * 64, n[l0] * 64, 64)
+            more = (PoolItem * 3)(
+                PoolItem(at(lay.pk, l0), *s, n[l0], 0, at(lay.pk, l0 + 1), at(lay.pk, l0 + 2), None, None, at(lay.pkr, l0 + 1), None,
+                         None, None, 0.0, 0, at(lay.pkr, l0 + 2), None),
+                PoolItem(at(lay.pv, l0), *s, n[l0], 0, at(lay.pv, l0 + 1), at(lay.pv, l0 + 2), None, None, at(lay.pvr, l0 + 1),
+                         at(lay.pvt, l0 + 1), None, None, 0.0, 0, at(lay.pvr, l0 + 2), at(lay.pvt, l0 + 2)),
+                PoolItem(at(lay.pq, l0), *s, n[l0], 0, at(lay.pq, l0 + 1), at(lay.pq, l0 + 2), None, None, None, None, None))
+            _check(lib, lib.pool_pyramid_fwd(more, 3, None, B, H, stream), "pool_pyramid (deeper levels)")
+
+        # Selection, coarse to fine: a dense top-k over the coarsest level's tokens (each of them is a block of the level
+        # below), then level by level among the blocks under the parent's selection.
+        _check(lib, lib.topk_dense(at(lay.pq, L), at(lay.pk, L), pi(lay.sel[L - 1]), B, H, n[L], topks[L - 1], 1, stream),
+               "gen_sparse_indices")
+        for l in range(L - 1, 0, -1):
+            _check(lib, lib.topk_sparse(at(lay.pq, l), at(lay.pk, l), pi(lay.sel[l]), pi(lay.sel[l - 1]), B, H, n[l], topks[l - 1],
+                                        topks[l], stream), "compute_topk_indices_sparse")
 
         # The lists of the backward go to a second stream, beside the attention kernel.  The attention
         # kernel is issued first (the GPU is waiting for it); an event recorded before it lets the
@@ -224,15 +221,15 @@ class LlsaFused(Function):
             ev_idx.record(cur)
 
         f = AttnFwdArgs()
-        f.qr, f.kr, f.vt, f.pkr, f.pvt = pa(lay.qr), pa(lay.kr), pa(lay.vt), pa(lay.pkr), pa(lay.pvt)
-        f.pk2r, f.pv2t, f.pidx = pa(lay.pk2r), pa(lay.pv2t), pi(lay.pidx)
-        f.idx = pi(lay.idx)
+        f.qr, f.kr, f.vt, f.idx = pa(lay.qr), pa(lay.kr), pa(lay.vt), pi(lay.sel[0])
         f.o, f.sob, f.soh, f.son = o.data_ptr(), o.stride(0), o.stride(1), o.stride(2)
         f.lse = lse.data_ptr()
-        f.B, f.H, f.N, f.T, f.T2, f.levels = B, H, N, T, T2, levels
-        f.w1, f.w2 = 16.0, 256.0
-        if l3:
-            f.pk3r, f.pv3t, f.ppidx, f.T3, f.w3 = pa(lay.pk3r), pa(lay.pv3t), pi(lay.ppidx), T3, 4096.0
+        f.B, f.H, f.N, f.T, f.levels = B, H, N, topks[0], L
+        for l in range(1, L + 1):
+            lv = f.lvl[l - 1]
+            lv.kr, lv.vt, lv.w = at(lay.pkr, l), at(lay.pvt, l), float(16 ** l)
+            if l < L:
+                lv.sel, lv.T = pi(lay.sel[l]), topks[l]
         _check(lib, lib.attn_fwd(C.byref(f), stream), "attn_fwd")
 
         if grad:
@@ -240,14 +237,11 @@ class LlsaFused(Function):
             if side is not None:
                 side.wait_event(ev_idx)         # (the arena is older than the selection, so this covers it too)
                 s_lists = C.c_void_p(side.cuda_stream)
-            _check(lib, lib.transpose_indices(pi(lay.idx), pi(lay.off), pi(lay.flat), pi(lay.work), None, B, H, n1, n1, T, CHUNK_FINE,
-                                              s_lists), "transpose_indices")
-            if l2:
-                _check(lib, lib.transpose_indices(pi(lay.pidx), pi(lay.poff), pi(lay.pflat), None, pi(lay.pinv), B, H, n2, n2, T2,
-                                                  1, s_lists), "transpose_indices (coarse)")
-            if l3:
-                _check(lib, lib.transpose_indices(pi(lay.ppidx), pi(lay.ppoff), pi(lay.ppflat), None, pi(lay.ppinv), B, H, n3, n3, T3,
-                                                  1, s_lists), "transpose_indices (level 3)")
+            _check(lib, lib.transpose_indices(pi(lay.sel[0]), pi(lay.off[0]), pi(lay.flat[0]), pi(lay.work), None, B, H, n[1], n[1],
+                                              topks[0], CHUNK_FINE, s_lists), "transpose_indices")
+            for l in range(1, L):
+                _check(lib, lib.transpose_indices(pi(lay.sel[l]), pi(lay.off[l]), pi(lay.flat[l]), None, pi(lay.inv[l]), B, H,
+                                                  n[l + 1], n[l + 1], topks[l], 1, s_lists), "transpose_indices (pooled level)")
             if side is not None:
                 ev_lists.record(side)
                 cur.wait_event(ev_lists)
@@ -255,7 +249,7 @@ class LlsaFused(Function):
         if grad:
             # (q and k themselves are needed again only by the backward of the qk-norm)
             ctx.save_for_backward(A, I, o, lse, freq, gq, gk, q if gq is not None else None, k if gk is not None else None)
-            ctx.meta = (lib, lay, B, H, N, T, T2, levels, q.shape, q.stride(), k.stride(), v.stride(), T3)
+            ctx.meta = (lib, lay, B, H, N, topks, q.shape, q.stride(), k.stride(), v.stride())
             ctx.eps = float(eps)
             ctx.gamma_dtypes = (None if gamma_q is None else gamma_q.dtype, None if gamma_k is None else gamma_k.dtype)
         return o
@@ -263,7 +257,8 @@ class LlsaFused(Function):
     @staticmethod
     def backward(ctx, do):
         A, I, o, lse, freq, gq, gk, q_in, k_in = ctx.saved_tensors
-        lib, lay, B, H, N, T, T2, levels, shape, sq, sk, sv, T3 = ctx.meta
+        lib, lay, B, H, N, topks, shape, sq, sk, sv = ctx.meta
+        L = len(topks)
         dev = o.device
         if not _rows_ok(do):
             do = do.contiguous()
@@ -282,28 +277,24 @@ class LlsaFused(Function):
         a.dout, a.sdob, a.sdoh, a.sdon = do.data_ptr(), do.stride(0), do.stride(1), do.stride(2)
         a.o, a.sob, a.soh, a.son = o.data_ptr(), o.stride(0), o.stride(1), o.stride(2)
         a.lse = lse.data_ptr()
-        a.qr, a.kr, a.vr, a.pkr, a.pvr = pa(lay.qr), pa(lay.kr), pa(lay.vr), pa(lay.pkr), pa(lay.pvr)
-        a.pk2r, a.pv2r = pa(lay.pk2r), pa(lay.pv2r)
-        a.idx, a.pidx = pi(lay.idx), pi(lay.pidx)
-        a.off, a.flat, a.work = pi(lay.off), pi(lay.flat), pi(lay.work)
-        a.poff, a.pinv = pi(lay.poff), pi(lay.pinv)
+        a.qr, a.kr, a.vr = pa(lay.qr), pa(lay.kr), pa(lay.vr)
+        a.idx, a.off, a.flat, a.work = pi(lay.sel[0]), pi(lay.off[0]), pi(lay.flat[0]), pi(lay.work)
         a.dq, a.sdqb, a.sdqh, a.sdqn = dq.data_ptr(), dq.stride(0), dq.stride(1), dq.stride(2)
         a.dk, a.sdkb, a.sdkh, a.sdkn = dk.data_ptr(), dk.stride(0), dk.stride(1), dk.stride(2)
         a.dv, a.sdvb, a.sdvh, a.sdvn = dv.data_ptr(), dv.stride(0), dv.stride(1), dv.stride(2)
-        a.dpk, a.dpv = w0 + lay.dpk, w0 + lay.dpv
-        if levels >= 2:
-            a.dpk2, a.dpv2 = w0 + lay.dpk2, w0 + lay.dpv2
-        if levels == 3:
-            a.pk3r, a.pv3r, a.ppidx = pa(lay.pk3r), pa(lay.pv3r), pi(lay.ppidx)
-            a.ppoff, a.ppinv = pi(lay.ppoff), pi(lay.ppinv)
-            a.dpk3, a.dpv3, a.T3, a.w3 = w0 + lay.dpk3, w0 + lay.dpv3, T3, 4096.0
+        for l in range(1, L + 1):
+            lv = a.lvl[l - 1]
+            lv.kr, lv.vr = pa(lay.pkr[l - 1]), pa(lay.pvr[l - 1])
+            lv.dk, lv.dv = w0 + lay.dpk[l - 1], w0 + lay.dpv[l - 1]
+            # llsa_l1 keeps the reference's quirk: its pooled path is differentiated with weight 1
+            # (sparse_attention_res_1.py:388-389) although the forward uses token_weight
+            lv.w, lv.gw = float(16 ** l), (1.0 if L == 1 else float(16 ** l))
+            if l < L:
+                lv.sel, lv.off, lv.inv, lv.T = pi(lay.sel[l]), pi(lay.off[l]), pi(lay.inv[l]), topks[l]
         a.workspace, a.workspace_bytes = w0 + lay.ws, lay.ws_bytes
         if freq is not None:
             a.freq_dq = a.freq_dk = freq.data_ptr()
-        a.B, a.H, a.N, a.T, a.T2, a.levels = B, H, N, T, T2, levels
-        # llsa_l1 keeps the reference's quirk: its pooled path is differentiated with weight 1
-        # (sparse_attention_res_1.py:388-389) although the forward uses token_weight
-        a.w1, a.w2, a.cgw1 = 16.0, 256.0, (16.0 if levels >= 2 else 1.0)
+        a.B, a.H, a.N, a.T, a.levels = B, H, N, topks[0], L
         a.stages, a.fold_pooled = 0, 1
         stream = _stream(lib, o)
         _check(lib, lib.attn_bwd(C.byref(a), stream), "attn_bwd")
@@ -322,18 +313,16 @@ class LlsaFused(Function):
                     dgq = dg
                 else:
                     dgk = dg
-        return dq, dk, dv, None, None, None, None, None, dgq, dgk, None, None
+        return dq, dk, dv, None, None, None, dgq, dgk, None
 
 
 def selection(out):
-    """The blocks the forward that produced `out` chose: (indices (B,H,N/16,T), p_indices
-    (B,H,N/256,T2) or None), int32 views of the arena its autograd node holds."""
+    """The blocks the forward that produced `out` chose, finest first: (indices (B,H,N/16,T), p_indices
+    (B,H,N/256,T2) or None for one level, then one more tensor per further level), int32 views of the arena its
+    autograd node holds."""
     node = out.grad_fn
     I = node.saved_tensors[1]
-    _, lay, B, H, N, T, T2, levels = node.meta[:8]
-    idx = I[lay.idx:lay.idx + B * H * lay.n1 * T].view(B, H, lay.n1, T)
-    pidx = I[lay.pidx:lay.pidx + B * H * lay.n2 * T2].view(B, H, lay.n2, T2) if levels >= 2 else None
-    if levels == 3:
-        T3 = node.meta[12]
-        return idx, pidx, I[lay.ppidx:lay.ppidx + B * H * lay.n3 * T3].view(B, H, lay.n3, T3)
-    return idx, pidx
+    _, lay, B, H, N, topks = node.meta[:6]
+    L = len(topks)
+    views = [I[lay.sel[l]:lay.sel[l] + B * H * lay.n[l + 1] * topks[l]].view(B, H, lay.n[l + 1], topks[l]) for l in range(L)]
+    return tuple(views) if L >= 2 else (views[0], None)

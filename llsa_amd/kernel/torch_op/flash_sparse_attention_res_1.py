@@ -51,7 +51,7 @@ flash_sparse_residual_attention_l1_op = FlashSparseResidualAttentionL1.apply
 def llsa_l1(q, k, v, topk=8, block_size=16, rope=None, qk_norm=None):
     """flash_sparse_attention_res_1.py:41-47."""
     gq, gk, eps = qk_norm if qk_norm is not None else (None, None, 0.0)
-    return LlsaFused.apply(q, k, v, 1, topk, 0, block_size, rope, gq, gk, eps)
+    return LlsaFused.apply(q, k, v, (topk,), block_size, rope, gq, gk, eps)
 
 
 def llsa_l1_unfused(q, k, v, topk=8, block_size=16):

@@ -37,6 +37,8 @@ Pinning status (what each function is checked against, see tests/test_oracle_*):
                          `delta_in_dtype=True`; the default keeps fp32.
   *_l3                   three levels, no counterpart in the reference: fp64 closed form over the four
                          weighted segments and torch.autograd on it, selection cascade property
+  *_lk                   any number of levels: equal to *_l1, *_l2, *_l3 bit for bit at k = 1, 2, 3; at k = 4 the key
+                         sets of single queries against a direct enumeration of the definition
   rms_norm / _bwd        F.rms_norm and its autograd (fp32).  The module the model
                          calls (diffusers' RMSNorm, rope_dit_transformer_2d.py:215-218)
                          is not in the reference checkout: parity unpinned for its
@@ -651,3 +653,104 @@ def llsa_l3_bwd(do, ctx, delta_in_dtype=False):
     dk = dk + mean_pool_bwd(dpk_t, bs)
     dv = dv + mean_pool_bwd(dpv_t, bs)
     return dq, dk, dv, dict(dpk=dpk, dpv=dpv, dpk2=dpk2, dpv2=dpv2, dpk3=dpk3, dpv3=dpv3)
+
+
+# --------------------------------------------------------------------------------------
+# any number of pooled levels.  The reference has one (llsa_l1) and two (llsa_l2); the functions below state the
+# scheme for k levels by induction on sparse_attention_res_2.py:94-149 and reduce to the functions above for
+# k = 1, 2, 3 (tests/test_oracle_pins.py checks that they do, bit for bit).
+#   pks, pvs : pooled k, v of level 1 .. k        sels : [indices, p_indices, pp_indices, ...], k entries --
+#   sels[l] (B,H,N/bs^(l+1),T_l) holds the blocks of level l (level 0 = the tokens) that every group of bs^(l+1)
+#   queries selected; the coarsest level k is read in full.
+# --------------------------------------------------------------------------------------
+
+
+def _segments_lk(q, k, v, pks, pvs, sels, weights, bs):
+    B, H, N, D = q.shape
+    N1 = N // bs
+    L = len(pks)
+    segs = [(_gather_blocks(k, sels[0], bs), _gather_blocks(v, sels[0], bs), 1.0)]
+    for l in range(1, L):                                     # owner of query block g at level l: g // bs^l
+        own = sels[l].long().repeat_interleave(bs ** l, dim=2)
+        segs.append((_gather_blocks(pks[l - 1], own, bs), _gather_blocks(pvs[l - 1], own, bs), float(weights[l - 1])))
+    kc, vc = pks[L - 1], pvs[L - 1]
+    segs.append((kc[:, :, None].expand(B, H, N1, kc.shape[2], D), vc[:, :, None].expand(B, H, N1, vc.shape[2], D), float(weights[L - 1])))
+    return segs
+
+
+def attn_fwd_lk(q, k, v, pks, pvs, sels, weights=None, block_size=16):
+    weights = weights or [block_size ** (l + 1) for l in range(len(pks))]
+    return _online_softmax(q, _segments_lk(q, k, v, pks, pvs, sels, weights, block_size), block_size)
+
+
+def closed_form_lk(q, k, v, pks, pvs, sels, weights=None, bs=16):
+    weights = weights or [bs ** (l + 1) for l in range(len(pks))]
+    return attn_closed_form(q, _segments_lk(q, k, v, pks, pvs, sels, weights, bs), bs)
+
+
+def attn_bwd_lk(do, q, k, v, pks, pvs, o, lse, sels, weights=None, block_size=16, coarse_grad_weight=None, delta_in_dtype=False):
+    """Returns (dq, dk, dv, [dpk_1 .. dpk_k], [dpv_1 .. dpv_k]).  coarse_grad_weight replaces the weight of the coarsest
+    level on the path to its own gradient (the llsa_l1 quirk, see attn_bwd_l1)."""
+    B, H, N, D = q.shape
+    bs, dt = block_size, q.dtype
+    L = len(pks)
+    weights = weights or [bs ** (l + 1) for l in range(L)]
+    G = N // bs
+    scale = 1.0 / math.sqrt(D)
+    qb = q.float().reshape(B, H, G, bs, D)
+    dob = do.float().reshape(B, H, G, bs, D)
+    lse_b = lse.reshape(B, H, G, bs)
+    delta = attn_delta(o, do, delta_in_dtype).reshape(B, H, G, bs)
+    segs = _segments_lk(q, k, v, pks, pvs, sels, weights, bs)
+    parts = [_bwd_segment(qb, dob, lse_b, delta, ks, vs, w, scale, dt) for ks, vs, w in segs]
+    dq = sum(p[0] for p in parts).reshape(B, H, N, D)
+    dk = _scatter_blocks(torch.zeros(B, H, N, D), parts[0][1], sels[0], bs)
+    dv = _scatter_blocks(torch.zeros(B, H, N, D), parts[0][2], sels[0], bs)
+    dpks, dpvs = [], []
+    for l in range(1, L):
+        own = sels[l].long().repeat_interleave(bs ** l, dim=2)
+        dpks.append(_scatter_blocks(torch.zeros(B, H, pks[l - 1].shape[2], D), parts[l][1], own, bs))
+        dpvs.append(_scatter_blocks(torch.zeros(B, H, pvs[l - 1].shape[2], D), parts[l][2], own, bs))
+    last = parts[L]
+    if coarse_grad_weight is not None:
+        last = _bwd_segment(qb, dob, lse_b, delta, segs[L][0], segs[L][1], float(coarse_grad_weight), scale, dt)
+    dpks.append(last[1].sum(2))
+    dpvs.append(last[2].sum(2))
+    rn = lambda x: _rn(x, dt).to(dt)
+    return rn(dq), rn(dk), rn(dv), [rn(x) for x in dpks], [rn(x) for x in dpvs]
+
+
+def llsa_lk_fwd(q, k, v, topks, block_size=16, sels=None):
+    """k = len(topks) pooled levels: dense selection on the coarsest level's tokens (topk.py:6-9), then parent-guided
+    selection level by level (topk.py:102-197) down to the fine blocks.  sels overrides the selection."""
+    bs = block_size
+    L = len(topks)
+    pqs, pks, pvs = [], [], []
+    xq, xk, xv = q, k, v
+    for _ in range(L):
+        xq, xk, xv = mean_pool(xq, bs), mean_pool(xk, bs), mean_pool(xv, bs)
+        pqs.append(xq), pks.append(xk), pvs.append(xv)
+    if sels is None:
+        sels = [None] * L
+        sels[L - 1] = gen_sparse_indices(pqs[L - 1], pks[L - 1], topks[L - 1])
+        for l in range(L - 1, 0, -1):
+            sels[l - 1] = topk_sparse(pqs[l - 1], pks[l - 1], sels[l], topks[l - 1], bs)
+    o, lse = attn_fwd_lk(q, k, v, pks, pvs, sels, None, bs)
+    return o, dict(q=q, k=k, v=v, pqs=pqs, pks=pks, pvs=pvs, o=o, lse=lse, sels=sels, block_size=bs)
+
+
+def llsa_lk_bwd(do, ctx, delta_in_dtype=False):
+    """Backward with the chain of pool backwards autograd adds around the operator (one level: the llsa_l1 quirk)."""
+    c = ctx
+    bs = c["block_size"]
+    L = len(c["pks"])
+    dq, dk, dv, dpks, dpvs = attn_bwd_lk(do, c["q"], c["k"], c["v"], c["pks"], c["pvs"], c["o"], c["lse"], c["sels"], None, bs,
+                                         coarse_grad_weight=1.0 if L == 1 else None, delta_in_dtype=delta_in_dtype)
+    gk, gv = dpks[L - 1], dpvs[L - 1]
+    for l in range(L - 2, -1, -1):
+        gk = dpks[l] + mean_pool_bwd(gk, bs)
+        gv = dpvs[l] + mean_pool_bwd(gv, bs)
+    dk = dk + mean_pool_bwd(gk, bs)
+    dv = dv + mean_pool_bwd(gv, bs)
+    return dq, dk, dv, dict(dpks=dpks, dpvs=dpvs)
+

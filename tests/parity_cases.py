@@ -198,7 +198,12 @@ def check_transpose(dev, B=2, H=2, Mb=64, T=8, Kb=None, chunk=0):
     from llsa_amd.kernel.hip.indices_transpose import transpose_indices
     g = torch.Generator().manual_seed(12)
     kb = Kb or Mb
-    idx = torch.stack([torch.randperm(kb, generator=g)[:T] for _ in range(B * H * Mb)]).reshape(B, H, Mb, T).int()
+    if Mb <= 16384:
+        idx = torch.stack([torch.randperm(kb, generator=g)[:T] for _ in range(B * H * Mb)]).reshape(B, H, Mb, T).int()
+    else:            # distinct within a row: base + t * stride with T * stride <= kb, modulo kb
+        base = torch.randint(0, kb, (B, H, Mb, 1), generator=g)
+        stride = torch.randint(1, kb // T + 1, (B, H, Mb, 1), generator=g)
+        idx = ((base + torch.arange(T) * stride) % kb).int()
     res = transpose_indices(idx.to(dev), Kb, chunk, inverse=True)
     off, flat, inv = res[0], res[1], res[-1].cpu().long()
     ro, rf = O.transpose_indices(idx.long(), Kb)
@@ -582,3 +587,56 @@ def check_op_l3(dev, B=1, H=1, N=262144, T=16, T2=16, T3=16, rope=True, qk_norm=
     _, own = O.llsa_l3_fwd(qr, kr, vc, T, T2, T3, 16)
     same = lambda a, b: (a.sort(-1).values == b.long().sort(-1).values).all(-1).float().mean().item()
     assert same(ppidx, own["pp_indices"]) > 0.9 and same(pidx, own["p_indices"]) > 0.9 and same(idx, own["indices"]) > 0.9
+
+
+def check_op_lk_samples(dev, N=4194304, topks=(16, 16, 16, 16), H=1, queries=(0, 1234567, -1), rows=16384):
+    """llsa_lk with k = len(topks) levels at a size the whole-tensor oracle cannot hold: the selection must be a legal
+    cascade at every level and equal to the oracle's at the coarsest level and (on the first `rows` groups) below it;
+    the output and dq rows of single queries are compared with the soft-max over the key set the scheme defines,
+    enumerated on the CPU in fp64 from the device's own selection (torch.autograd for dq)."""
+    import llsa_amd
+    from llsa_amd.kernel.torch_op._fused import selection
+    L = len(topks)
+    q, k, v, do = smooth_inputs(1, H, N, 64, dev)
+    captured = {}
+
+    def run(q_, k_, v_):
+        out = llsa_amd.llsa_lk(q_, k_, v_, topks, 16)
+        captured["sel"] = [t.cpu().long() for t in selection(out)]
+        return out
+
+    o, dq, dk, dv = _grads(run, q, k, v, do)
+    sels = captured["sel"]
+    assert [tuple(s.shape) for s in sels] == [(1, H, N // 16 ** (l + 1), topks[l]) for l in range(L)]
+    for l in range(L - 1):
+        par = sels[l + 1].repeat_interleave(16, dim=2)
+        assert ((sels[l][..., :, None] // 16) == par[..., None, :]).any(-1).all(), f"level {l}: a block outside its parent's selection"
+    qc, kc, vc, doc = (t.cpu() for t in (q, k, v, do))
+    pqs, pks, pvs, xq, xk, xv = [], [], [], qc, kc, vc
+    for _ in range(L):
+        xq, xk, xv = O.mean_pool(xq, 16), O.mean_pool(xk, 16), O.mean_pool(xv, 16)
+        pqs.append(xq), pks.append(xk), pvs.append(xv)
+    rep = MEASURED.setdefault(f"op_l{L}_N{N}", {})
+    rep[f"level {L} selection (same, tie-free)"] = selection_dense_vs_oracle(f"level {L}", pqs[L - 1], pks[L - 1], sels[L - 1], topks[L - 1])
+    for l in range(L - 1, 0, -1):                            # sels[l-1] chosen under the parents sels[l]
+        r = min(rows, sels[l - 1].shape[2])
+        rep[f"level {l} selection (same, tie-free)"] = selection_sparse_vs_oracle(
+            f"level {l}", pqs[l - 1][:, :, :r], pks[l - 1], sels[l][:, :, :max(r // 16, 1)], sels[l - 1][:, :, :r], topks[l - 1])
+    for h in range(H):
+        for n in queries:
+            n = n % N
+            keys, vals, wts = [], [], []
+            for l in range(L):
+                src_k, src_v = (kc, vc) if l == 0 else (pks[l - 1], pvs[l - 1])
+                for blk in sels[l][0, h, n // 16 ** (l + 1)].tolist():
+                    keys.append(src_k[0, h, blk * 16:blk * 16 + 16]), vals.append(src_v[0, h, blk * 16:blk * 16 + 16])
+                    wts += [16.0 ** l] * 16
+            keys.append(pks[L - 1][0, h]), vals.append(pvs[L - 1][0, h])
+            wts += [16.0 ** L] * pks[L - 1].shape[2]
+            kk, vv, ww = torch.cat(keys).double(), torch.cat(vals).double(), torch.tensor(wts, dtype=torch.float64)
+            qq = qc[0, h, n].double().requires_grad_(True)
+            want = torch.softmax((kk @ qq) / 8.0 + ww.log(), 0) @ vv
+            gq, = torch.autograd.grad(want, qq, doc[0, h, n].double())
+            close(f"o[{h},{n}]", o[0, h, n], want.detach())
+            close(f"dq[{h},{n}]", dq[0, h, n], gq, rel=2e-2)
+    assert all(torch.isfinite(t).all() for t in (dk, dv))

@@ -58,16 +58,23 @@ def test_entry_points_reject_bad_arguments(lib):
     assert lib.topk_dense(16, 16, 16, 1, 1, 64, 128, 1, None) != 0          # T > n
     a = AttnFwdArgs()
     a.levels, a.B, a.H, a.N, a.T = 1, 1, 1, 1000, 8
-    a.qr = a.kr = a.vt = a.pkr = a.pvt = a.idx = a.o = a.lse = 16
-    a.w1 = 16.0
+    a.qr = a.kr = a.vt = a.idx = a.o = a.lse = 16
+    a.lvl[0].kr = a.lvl[0].vt = 16
+    a.lvl[0].w = 16.0
     assert lib.attn_fwd(C.byref(a), None) != 0
     assert b"1024" in lib.last_error_string()
     a.N, a.T = 1024, 6
     assert lib.attn_fwd(C.byref(a), None) != 0
     assert b"multiple of 4" in lib.last_error_string()
-    assert lib.attn_bwd_workspace_bytes(2, 6, 16384, 16, 16, 0, 2) > 0
-    assert lib.attn_bwd_workspace_bytes(1, 1, 262144, 16, 16, 16, 3) > lib.attn_bwd_workspace_bytes(1, 1, 262144, 16, 16, 0, 2) > 0
-    assert lib.attn_bwd_workspace_bytes(2, 6, 16384, 16, 16, 0, 4) < 0
+    a.levels, a.N, a.T = 4, 262144, 8                   # four levels need N % 4194304 == 0
+    assert lib.attn_fwd(C.byref(a), None) != 0
+    assert b"4194304" in lib.last_error_string()
+    a.levels = 5
+    assert lib.attn_fwd(C.byref(a), None) != 0
+    topk = lambda *t: (C.c_int32 * len(t))(*t)
+    assert lib.attn_bwd_workspace_bytes(2, 6, 16384, topk(16, 16), 2) > 0
+    assert lib.attn_bwd_workspace_bytes(1, 1, 262144, topk(16, 16, 16), 3) > lib.attn_bwd_workspace_bytes(1, 1, 262144, topk(16, 16), 2) > 0
+    assert lib.attn_bwd_workspace_bytes(2, 6, 16384, topk(16, 16, 16, 16, 16), 5) < 0
     assert lib.work_list_len(1024, 1024, 16, 32) == 4 + 4 * (512 + 1024) + 4 * 513 + 1024
 
 

@@ -1,7 +1,7 @@
 """The benchmark configurations at their full sizes.
 
-C2 and C3 are small enough for the CPU oracle, slice by slice.  At N = 65536, 262144 and (three
-levels) 1048576 the oracle would take minutes, so the operator is checked through properties that do not depend on
+C2 and C3 are small enough for the CPU oracle, slice by slice.  At N = 65536, 262144, (three levels) 1048576 and
+(four levels) 4194304 the oracle would take minutes, so the operator is checked through properties that do not depend on
 the size (the selection depends on q and k only, so it is the same on both sides of each):
   * constant V            -> O is that constant (the weights of fine and pooled tokens sum to 1)
   * linearity in V        -> O(a V1 + b V2) = a O(V1) + b O(V2)
@@ -70,14 +70,23 @@ def _rel(a, b):
     return ((a.double() - b.double()).norm() / b.double().norm().clamp_min(1e-30)).item()
 
 
-@pytest.mark.parametrize("N,H,levels", [(65536, 2, 2), (262144, 1, 2), (1048576, 1, 3)])
+def test_four_levels_single_queries_against_enumeration(dev):
+    """llsa_lk with four pooled levels at the smallest size it admits, N = 4194304 = 64 * 16^4."""
+    P.check_op_lk_samples(dev, N=4194304, topks=(16, 16, 16, 16))
+
+
+def test_three_levels_single_queries_against_enumeration(dev):
+    P.check_op_lk_samples(dev, N=262144, topks=(8, 4, 8), H=2)
+
+
+@pytest.mark.parametrize("N,H,levels", [(65536, 2, 2), (262144, 1, 2), (1048576, 1, 3), (4194304, 1, 4)])
 def test_large_n_properties(dev, N, H, levels):
     import llsa_amd
     from llsa_amd.utils.rope_table import rope_table
     q, k, v, do = P.smooth_inputs(1, H, N, 64, dev)
     freq = rope_table(math.isqrt(N), dtype=torch.bfloat16).to(dev)
-    if levels == 3:
-        op = lambda q_, k_, v_: llsa_amd.llsa_l3(q_, k_, v_, 16, 16, 16, 16, rope=freq)
+    if levels >= 3:
+        op = lambda q_, k_, v_: llsa_amd.llsa_lk(q_, k_, v_, (16,) * levels, 16, rope=freq)
     else:
         op = lambda q_, k_, v_: llsa_amd.llsa_l2(q_, k_, v_, 16, 16, 16, rope=freq)
 

@@ -87,6 +87,8 @@ def test_transpose(dev):
 def test_transpose_largest(dev):
     P.check_transpose(dev, B=1, H=1, Mb=16384, T=16)
     P.check_transpose(dev, B=1, H=2, Mb=16384, T=16, chunk=64)       # with the work list: the split form
+    P.check_transpose(dev, B=1, H=1, Mb=262144, T=16, chunk=64)      # the fine level of four pooled levels: 128 KB of sort bitmaps
+    P.check_transpose(dev, B=1, H=1, Mb=524288, T=2, Kb=8192, chunk=64)   # two sort waves a workgroup
 
 
 @pytest.mark.parametrize("strided,smooth", [(False, False), (True, False), (False, True)])

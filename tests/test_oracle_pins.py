@@ -390,6 +390,78 @@ def test_three_levels_match_closed_form_and_its_autograd():
         assert (a.double() - b).norm() / b.norm() < 2e-5
 
 
+def test_k_levels_reduce_to_the_one_two_and_three_level_functions_bit_for_bit():
+    g = torch.Generator().manual_seed(21)
+    B, H, N, D = 1, 2, 65536, 8
+    q, k, v, do = (torch.randn(B, H, N, D, generator=g).bfloat16() for _ in range(4))
+    o1, c1 = O.llsa_l1_fwd(q[:, :, :2048], k[:, :, :2048], v[:, :, :2048], 8)
+    ok, ck = O.llsa_lk_fwd(q[:, :, :2048], k[:, :, :2048], v[:, :, :2048], (8,))
+    assert torch.equal(o1, ok) and torch.equal(c1["lse"], ck["lse"]) and torch.equal(c1["indices"], ck["sels"][0])
+    for a, b in zip(O.llsa_l1_bwd(do[:, :, :2048], c1)[:3], O.llsa_lk_bwd(do[:, :, :2048], ck)[:3]):
+        assert torch.equal(a, b)
+    o2, c2 = O.llsa_l2_fwd(q, k, v, 4, 4)
+    ok, ck = O.llsa_lk_fwd(q, k, v, (4, 4))
+    assert torch.equal(o2, ok) and torch.equal(c2["lse"], ck["lse"])
+    assert torch.equal(c2["indices"], ck["sels"][0]) and torch.equal(c2["p_indices"], ck["sels"][1])
+    for a, b in zip(O.llsa_l2_bwd(do, c2)[:3], O.llsa_lk_bwd(do, ck)[:3]):
+        assert torch.equal(a, b)
+    o3, c3 = O.llsa_l3_fwd(q, k, v, 4, 3, 2)
+    ok, ck = O.llsa_lk_fwd(q, k, v, (4, 3, 2))
+    assert torch.equal(o3, ok) and torch.equal(c3["lse"], ck["lse"])
+    for n, s in zip(("indices", "p_indices", "pp_indices"), ck["sels"]):
+        assert torch.equal(c3[n], s)
+    for a, b in zip(O.llsa_l3_bwd(do, c3)[:3], O.llsa_lk_bwd(do, ck)[:3]):
+        assert torch.equal(a, b)
+
+
+def test_four_levels_key_sets_by_direct_enumeration_and_autograd():
+    """Four pooled levels have no counterpart in the reference.  Pinned here: for single queries the soft-max of
+    the k-level closed form is the one over the key set the scheme defines, enumerated directly (fine tokens of
+    the blocks the query's 16-group selected, level-l tokens of the blocks its 16^(l+1)-group selected with weight
+    16^l, every level-4 token with weight 16^4); the explicit backward is the gradient of that closed form."""
+    g = torch.Generator().manual_seed(22)
+    B, H, N, D = 1, 1, 2 * 65536, 4
+    q, k, v, do = (torch.randn(B, H, N, D, generator=g) for _ in range(4))
+    o, ctx = O.llsa_lk_fwd(q, k, v, (3, 2, 2, 1))
+    sels, pks, pvs = ctx["sels"], ctx["pks"], ctx["pvs"]
+    assert [tuple(s.shape) for s in sels] == [(1, 1, N // 16, 3), (1, 1, N // 256, 2), (1, 1, N // 4096, 2), (1, 1, 2, 1)]
+    oc, lc = O.closed_form_lk(*[t.double() for t in (q, k, v)], [t.double() for t in pks], [t.double() for t in pvs], sels)
+    for n in (0, 77777, N - 1):
+        keys, vals, wts = [], [], []
+        for l in range(4):
+            src_k, src_v = (k, v) if l == 0 else (pks[l - 1], pvs[l - 1])
+            for blk in sels[l][0, 0, n // 16 ** (l + 1)].tolist():
+                keys.append(src_k[0, 0, blk * 16:blk * 16 + 16]), vals.append(src_v[0, 0, blk * 16:blk * 16 + 16])
+                wts += [16.0 ** l] * 16
+        keys.append(pks[3][0, 0]), vals.append(pvs[3][0, 0])
+        wts += [16.0 ** 4] * pks[3].shape[2]
+        kk, vv, ww = torch.cat(keys).double(), torch.cat(vals).double(), torch.tensor(wts, dtype=torch.float64)
+        s = (kk @ q[0, 0, n].double()) / math.sqrt(D) + ww.log()
+        want = torch.softmax(s, 0) @ vv
+        assert torch.allclose(oc[0, 0, n], want, atol=1e-10)
+        assert lc[0, 0, n].item() == pytest.approx(torch.logsumexp(s, 0).item(), abs=1e-10)
+    got = O.attn_bwd_lk(do, q, k, v, pks, pvs, oc.float(), lc.float(), sels)
+    leaves = [t.double().requires_grad_(True) for t in (q, k, v, *pks, *pvs)]
+    oo, _ = O.closed_form_lk(*leaves[:3], leaves[3:7], leaves[7:], sels)
+    want = torch.autograd.grad(oo, leaves, do.double())
+    flat = [got[0], got[1], got[2], *got[3], *got[4]]
+    for a, b in zip(flat, want):
+        assert (a.double() - b).norm() / b.norm() < 2e-5
+    # whole operator: the chain of four pool backwards
+    pool = lambda x: x.reshape(B, H, -1, 16, D).mean(3)
+    ql, kl, vl = (t.double().requires_grad_(True) for t in (q, k, v))
+    pk_, pv_, xk, xv = [], [], kl, vl
+    for _ in range(4):
+        xk, xv = pool(xk), pool(xv)
+        pk_.append(xk), pv_.append(xv)
+    oo, _ = O.closed_form_lk(ql, kl, vl, pk_, pv_, sels)
+    wq, wk, wv = torch.autograd.grad(oo, (ql, kl, vl), do.double())
+    ctx2 = dict(ctx, o=oc.float(), lse=lc.float())
+    dq, dk, dv, _ = O.llsa_lk_bwd(do, ctx2)
+    for a, b in ((dq, wq), (dk, wk), (dv, wv)):
+        assert (a.double() - b).norm() / b.norm() < 2e-5
+
+
 def test_delta_variants():
     g = torch.Generator().manual_seed(11)
     o = torch.randn(1, 1, 8, 64, generator=g).bfloat16()
