@@ -26,8 +26,8 @@ constexpr int NB = 2;                // 16-key blocks per pipeline step: 32 keys
 
 struct SoftmaxState {
     float m2;        // reference point of the exponentials (at most kMaxSlack below the running max), log2 units
-    float lsum;      // this lane's share of the running sum, in units of the current weight
-    f32x4 acc[4];    // O^T: channel 16*dt + 4*(l/16) + e of query l%16
+    f32x4 acc[4];    // O^T: channel 16*dt + 4*(l/16) + e of query l%16, in units of the current weight
+    float lsum;      // this lane's share of the running sum of the query's p
 };
 
 // Operands of one step = NB 16-key blocks, as they sit in registers between load and use.
@@ -40,7 +40,6 @@ struct KvRegs {
 struct StepDesc {
     const bf16* kb[NB];
     const bf16* vtb[NB];
-    float wratio;        // weight(previous segment) / weight(this segment) on the first step of a segment
 };
 
 __device__ __forceinline__ void load_step(KvRegs& t, const StepDesc& d, int lane) {
@@ -55,48 +54,102 @@ __device__ __forceinline__ void load_step(KvRegs& t, const StepDesc& d, int lane
         for (int dt = 0; dt < 4; dt++) t.v[j][dt] = ld8(d.vtb[j] + dt * 256 + lane * 4);
 }
 
-__device__ __forceinline__ void compute_step(SoftmaxState& st, const bf16x8 bq[2], const KvRegs& t, float wratio) {
-    f32x4 s[NB];
+__device__ __forceinline__ void init_state(SoftmaxState& st) {
+    st.m2 = 0.f;
+    st.lsum = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++) st.acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+}
+
+// Changes the unit the accumulator and the running sum are kept in (at a boundary between segments of different weight).
+__device__ __forceinline__ void rescale(SoftmaxState& st, float f) {
+    st.lsum *= f;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++) st.acc[dt] *= f;
+}
+
+// The exponentials refer to st.m2, which follows the running maximum lazily: it moves only when the maximum
+// has grown by more than kMaxSlack (then p <= 2^kMaxSlack, harmless in bf16 and in the fp32 sums), so that the
+// accumulator is rescaled a few times per query block instead of at most steps; O = acc / sum and
+// lse = m2 + log2(sum) hold for any reference point.  The common path therefore needs no maximum over the quad
+// of lanes that share a query: every lane checks its own exponents against the slack, and only when one in the
+// wave exceeds it is the reference point moved (for all four lanes of a query alike, by the quad's largest
+// exponent).  st.m2 starts at the largest score of the first block (start_reference), so it is always finite.
+__device__ __forceinline__ void start_reference(SoftmaxState& st, const bf16x8 bq[2], const KvRegs& t) {
+    f32x4 z = {0.f, 0.f, 0.f, 0.f};
+    const f32x4 s = mfma_bf16(t.k[0][1], bq[1], mfma_bf16(t.k[0][0], bq[0], z));
+    st.m2 = quad_max(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3]))) * kScaleLog2e;
+}
+
+// x: the exponents of one step (NB blocks) relative to st.m2
+__device__ __forceinline__ void exponents(float x[NB][4], const SoftmaxState& st, const bf16x8 bq[2], const KvRegs& t) {
 #pragma unroll
     for (int j = 0; j < NB; j++) {
         f32x4 z = {0.f, 0.f, 0.f, 0.f};
-        z = mfma_bf16(t.k[j][0], bq[0], z);
-        s[j] = mfma_bf16(t.k[j][1], bq[1], z);
+        const f32x4 s = mfma_bf16(t.k[j][1], bq[1], mfma_bf16(t.k[j][0], bq[0], z));
+#pragma unroll
+        for (int e = 0; e < 4; e++) x[j][e] = fmaf(s[e], kScaleLog2e, -st.m2);
     }
-    float mx = s[0][0];
+}
+__device__ __forceinline__ float largest(const float x[NB][4]) {
+    float top = x[0][0];
 #pragma unroll
     for (int j = 0; j < NB; j++)
 #pragma unroll
-        for (int e = 0; e < 4; e++) mx = fmaxf(mx, s[j][e]);
-    mx = quad_max(mx);
-    // The exponentials refer to st.m2, which follows the running maximum lazily: it moves only when the
-    // maximum has grown by more than kMaxSlack (then p <= 2^kMaxSlack, harmless in bf16 and in the fp32
-    // sums), so that the accumulator is rescaled a few times per query block instead of at most steps.
-    // O = acc / lsum and lse = m2 + log2(lsum) hold for any reference point.
-    const float cand = mx * kScaleLog2e;
-    const float m2n = (cand > st.m2 + kMaxSlack) ? cand : st.m2;
-    const float alpha = exp2_fast(st.m2 - m2n) * wratio;
-    float rs = 0.f;
+        for (int e = 0; e < 4; e++) top = fmaxf(top, x[j][e]);
+    return top;
+}
+// the rare path: moves the reference point of every query whose largest exponent exceeds the slack
+__device__ __forceinline__ void move_reference(SoftmaxState& st, float x[NB][4], float top) {
+    top = quad_max(top);
+    const float shift = (top > kMaxSlack) ? top : 0.f;
+    st.m2 += shift;
+    rescale(st, exp2_fast(-shift));
+#pragma unroll
+    for (int j = 0; j < NB; j++)
+#pragma unroll
+        for (int e = 0; e < 4; e++) x[j][e] -= shift;
+}
+__device__ __forceinline__ void accumulate(SoftmaxState& st, const float x[NB][4], const KvRegs& t) {
     bf16x8 bp[NB / 2];
+    float rs = 0.f;
 #pragma unroll
     for (int j = 0; j < NB; j++)
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            const float p = exp2_fast(fmaf(s[j][e], kScaleLog2e, -m2n));
+            const float p = exp2_fast(x[j][e]);
             rs += p;
             bp[j >> 1][(j & 1) * 4 + e] = (bf16)p;
         }
-    st.lsum = st.lsum * alpha + rs;
-    st.m2 = m2n;
-    if (__ballot(alpha != 1.f) != 0) {        // the running max moved (or a new segment starts) somewhere in the wave
-#pragma unroll
-        for (int dt = 0; dt < 4; dt++) st.acc[dt] *= alpha;
-    }
+    st.lsum += rs;
 #pragma unroll
     for (int c = 0; c < NB / 2; c++)
 #pragma unroll
         for (int dt = 0; dt < 4; dt++)
             st.acc[dt] = mfma_bf16(cat(t.v[2 * c][dt], t.v[2 * c + 1][dt]), bp[c], st.acc[dt]);
+}
+
+__device__ __forceinline__ void compute_step(SoftmaxState& st, const bf16x8 bq[2], const KvRegs& t) {
+    float x[NB][4];
+    exponents(x, st, bq, t);
+    const float top = largest(x);
+    if (__ballot(top > kMaxSlack) != 0) move_reference(st, x, top);
+    accumulate(st, x, t);
+}
+
+// The same step for two query blocks that read the same operands, written as one straight-line piece so that the
+// products of one block overlap with the exponentials of the other (one test for the rare path covers both).
+__device__ __forceinline__ void compute_step2(SoftmaxState& sa, SoftmaxState& sb, const bf16x8 qa[2], const bf16x8 qb[2], const KvRegs& t) {
+    float xa[NB][4], xb[NB][4];
+    exponents(xa, sa, qa, t);
+    exponents(xb, sb, qb, t);
+    const float ta = largest(xa), tb = largest(xb);
+    if (__ballot(fmaxf(ta, tb) > kMaxSlack) != 0) {
+        move_reference(sa, xa, ta);
+        move_reference(sb, xb, tb);
+    }
+    accumulate(sa, xa, t);
+    accumulate(sb, xb, t);
 }
 
 // Operands of one step out of the workgroup's LDS copy of shared blocks (4 KB per block: R tile
@@ -111,6 +164,16 @@ __device__ __forceinline__ void load_step_lds(KvRegs& t, const bf16* blocks, int
     for (int j = 0; j < NB; j++)
 #pragma unroll
         for (int dt = 0; dt < 4; dt++) t.v[j][dt] = lds_ld8(blocks + j * 2 * kTile + kTile + dt * 256 + lane * 4);
+}
+
+__device__ __forceinline__ void finish_query_block(const llsa_attn_fwd_args& a, const SoftmaxState& st, int bh, int b, int h, int g, int lane) {
+    const int r = lane & 15, quad = lane >> 4;
+    const float L = quad_sum(st.lsum);
+    const float inv = 1.f / L;
+    bf16* op = (bf16*)a.o + b * a.sob + h * a.soh + (int64_t)(g * kBlk + r) * a.son + quad * 4;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++) st8(op + dt * 16, cvt4(st.acc[dt] * inv));
+    if (quad == 0) a.lse[(int64_t)bh * a.N + g * kBlk + r] = (st.m2 + __builtin_amdgcn_logf(L)) * kLn2;
 }
 
 // One wave per query block, four consecutive query blocks per workgroup.
@@ -134,7 +197,6 @@ __global__ __launch_bounds__(256, 4) void attn_fwd_kernel(llsa_attn_fwd_args a) 
     const int lid = xcd_logical_id();
     const int g = (lid % (int)gridDim.x) * 4 + wave;          // < N1: the host checks N1 % 4 == 0
     const int bh = lid / (int)gridDim.x, b = bh / a.H, h = bh % a.H;
-    const int r = lane & 15, quad = lane >> 4;
 
     const bf16* kr = (const bf16*)a.kr + (int64_t)bh * N1 * kTile;
     const bf16* vt = (const bf16*)a.vt + (int64_t)bh * N1 * kTile;
@@ -166,10 +228,7 @@ __global__ __launch_bounds__(256, 4) void attn_fwd_kernel(llsa_attn_fwd_args a) 
         bq[1] = ld16(qp + 512); // reference does) equals scaling the fp32 scores, done in the exponent
     }
     SoftmaxState st;
-    st.m2 = -INFINITY;
-    st.lsum = 0.f;
-#pragma unroll
-    for (int dt = 0; dt < 4; dt++) st.acc[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    init_state(st);
 
     KvRegs ra, rb;
 
@@ -182,17 +241,18 @@ __global__ __launch_bounds__(256, 4) void attn_fwd_kernel(llsa_attn_fwd_args a) 
         __syncthreads();
         // weight(previous segment) / weight(this one); nothing is accumulated before group 0
         const float w_here = a.lvl[shared_level(a.lvl, a.levels, kGroup * grp)].w;
-        const float wr = (grp == 0) ? 1.f : w_prev / w_here;
+        if (grp > 0 && w_here != w_prev) rescale(st, w_prev / w_here);
         w_prev = w_here;
         // (LDS reads first: the compiler makes every LDS read wait for all copies into LDS that
         // were issued before it, which would serialise the next fetch with the arithmetic of this group)
         load_step_lds(ra, &sh[grp & 1][0][0], lane);
         load_step_lds(rb, &sh[grp & 1][NB][0], lane);
         if (grp + 1 < n_groups) issue_group(grp + 1);
-        compute_step(st, bq, ra, wr);
-        compute_step(st, bq, rb, 1.f);
+        if (grp == 0) start_reference(st, bq, ra);
+        compute_step(st, bq, ra);
+        compute_step(st, bq, rb);
     }
-    const float w_shared_last = w_prev;                       // (the coarsest level's weight)
+    rescale(st, w_prev);                                      // fine tokens weigh 1
 
     wait_all_mem();     // nothing is in flight here: said for the compiler (see wait_all_mem)
     // ---- fine blocks, private to the wave.  Their indices are fetched 64 at a time, entry i into
@@ -220,20 +280,153 @@ __global__ __launch_bounds__(256, 4) void attn_fwd_kernel(llsa_attn_fwd_args a) 
         for (int t = 0; t < n_fine; t += 2) {
             describe(min(t + 1, n_fine - 1), d);
             load_step(rb, d, lane);
-            compute_step(st, bq, ra, (c0 == 0 && t == 0) ? w_shared_last : 1.f);   // fine tokens weigh 1
+            compute_step(st, bq, ra);
             if (t + 1 >= n_fine) break;
             describe(min(t + 2, n_fine - 1), d);
             load_step(ra, d, lane);
-            compute_step(st, bq, rb, 1.f);
+            compute_step(st, bq, rb);
         }
     }
 
-    const float L = quad_sum(st.lsum);
-    const float inv = 1.f / L;
-    bf16* op = (bf16*)a.o + b * a.sob + h * a.soh + (int64_t)(g * kBlk + r) * a.son + quad * 4;
+    finish_query_block(a, st, bh, b, h, g, lane);
+}
+
+// ---------------------------------------------------------------------------------------
+// Two sibling query blocks per wave (topk <= 32).  Both walk the same pooled blocks, and on coherent inputs most
+// of their fine blocks coincide, so every operand tile that both need is fetched once and multiplied twice: the
+// wave first sorts the two fine lists into [blocks both selected | only the first | only the second] and walks
+// that list in steps of NB blocks, a step of the first part feeding both soft-max states.  What bounds these
+// kernels is the rate at which tiles arrive from the L2, and this removes a quarter to a half of them.
+// A row that names a block twice keeps the plain walk (nothing is shared).
+// ---------------------------------------------------------------------------------------
+constexpr int kPairMaxTopk = 32;
+
+__global__ __launch_bounds__(256, 3) void attn_fwd_pair_kernel(llsa_attn_fwd_args a) {
+    static_assert(NB == 2 && kGroup == 4, "the shared phase reads an LDS buffer of four blocks as two steps of two");
+    __shared__ __align__(16) bf16 sh[2][kGroup][2 * kTile];
+    __shared__ int order[4][kWave];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int N1 = a.N / kBlk, T = a.T;
+    const int lid = xcd_logical_id();
+    const int g = (lid % (int)gridDim.x) * 8 + 2 * wave;      // query blocks g and g + 1 (the host checks N1 % 8 == 0)
+    const int bh = lid / (int)gridDim.x, b = bh / a.H, h = bh % a.H;
+
+    const bf16* kr = (const bf16*)a.kr + (int64_t)bh * N1 * kTile;
+    const bf16* vt = (const bf16*)a.vt + (int64_t)bh * N1 * kTile;
+    const int* ip = a.idx + ((int64_t)bh * N1 + g) * T;
+
+    SharedList sl = shared_list(a.lvl, a.levels, a.N, bh, g, lane);
+    bf16* const sh0 = &sh[0][0][0];
+    auto issue_group = [&](int grp) __attribute__((always_inline)) {
+        const SharedBlock sb = shared_block(sl, a.lvl, a.levels, a.N, bh, kGroup * grp + wave);
+        const bf16* kb = (const bf16*)a.lvl[sb.level].kr + sb.tile;
+        const bf16* vb = (const bf16*)a.lvl[sb.level].vt + sb.tile;
+        bf16* dst = sh0 + ((grp & 1) * kGroup + wave) * (2 * kTile);
+        copy16_global_to_lds(kb + lane * 8, dst);
+        copy16_global_to_lds(kb + 512 + lane * 8, dst + 512);
+        copy16_global_to_lds(vb + lane * 8, dst + kTile);
+        copy16_global_to_lds(vb + 512 + lane * 8, dst + kTile + 512);
+    };
+    const int n_groups = sl.n_blocks / kGroup;
+    issue_group(0);
+
+    // ---- the two fine lists, sorted into [both | only the first | only the second]; entry i ends in lane i
+    const int first = (lane < T) ? clampi(ip[lane], 0, N1 - 1) : -1 - lane;       // (distinct negative fillers)
+    const int second = (lane < T) ? clampi(ip[T + lane], 0, N1 - 1) : -65 - lane;
+    bool in_second = false, in_first = false, twice = false;
+    for (int j = 0; j < T; j++) {
+        const int fj = __builtin_amdgcn_readlane(first, j), sj = __builtin_amdgcn_readlane(second, j);
+        in_second |= first == sj;
+        in_first |= second == fj;
+        twice |= (first == fj && lane != j) || (second == sj && lane != j);
+    }
+    if (__ballot(twice) != 0) in_second = in_first = false;
+    unsigned long long both = __ballot(in_second);
+    if (__popcll(both) & 1) {                                 // an even number is shared: steps hold NB = 2 blocks
+        const int last = 63 - __builtin_clzll(both);
+        const int dropped = __builtin_amdgcn_readlane(first, last);
+        in_second = in_second && lane != last;
+        in_first = in_first && second != dropped;
+        both &= ~(1ull << last);
+    }
+    const int n_both = __popcll(both), n_only = T - n_both;
+    {
+        const unsigned long long below = (1ull << lane) - 1ull;
+        const unsigned long long only1 = __ballot(lane < T && !in_second), only2 = __ballot(lane < T && !in_first);
+        int* mine = order[wave];
+        if (lane < T) mine[in_second ? __popcll(both & below) : n_both + __popcll(only1 & below)] = first;
+        if (lane < T && !in_first) mine[n_both + n_only + __popcll(only2 & below)] = second;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int mine = order[wave][lane];                        // entries [0, n_both + 2 * n_only) are meaningful
+    const int steps_both = n_both / NB, steps_only = n_only / NB, n_steps = steps_both + 2 * steps_only;
+
+    bf16x8 bq[2][2];
 #pragma unroll
-    for (int dt = 0; dt < 4; dt++) st8(op + dt * 16, cvt4(st.acc[dt] * inv));
-    if (quad == 0) a.lse[(int64_t)bh * a.N + g * kBlk + r] = (st.m2 + __builtin_amdgcn_logf(L)) * kLn2;
+    for (int u = 0; u < 2; u++) {
+        const bf16* qp = (const bf16*)a.qr + ((int64_t)bh * N1 + g + u) * kTile + lane * 8;
+        bq[u][0] = ld16(qp);
+        bq[u][1] = ld16(qp + 512);
+    }
+    SoftmaxState st[2];
+    init_state(st[0]);
+    init_state(st[1]);
+    KvRegs ra, rb;
+
+    float w_prev = 1.f;
+    for (int grp = 0; grp < n_groups; grp++) {
+        wait_vm0();
+        __syncthreads();
+        const float w_here = a.lvl[shared_level(a.lvl, a.levels, kGroup * grp)].w;
+        if (grp > 0 && w_here != w_prev) {
+            rescale(st[0], w_prev / w_here);
+            rescale(st[1], w_prev / w_here);
+        }
+        w_prev = w_here;
+        load_step_lds(ra, &sh[grp & 1][0][0], lane);
+        load_step_lds(rb, &sh[grp & 1][NB][0], lane);
+        if (grp + 1 < n_groups) issue_group(grp + 1);
+        if (grp == 0) {
+            start_reference(st[0], bq[0], ra);
+            start_reference(st[1], bq[1], ra);
+        }
+        compute_step2(st[0], st[1], bq[0], bq[1], ra);
+        compute_step2(st[0], st[1], bq[0], bq[1], rb);
+    }
+    rescale(st[0], w_prev);                                   // fine tokens weigh 1
+    rescale(st[1], w_prev);
+    wait_all_mem();
+
+    auto describe = [=](int t, StepDesc& d) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < NB; j++) {
+            const int blk = __builtin_amdgcn_readlane(mine, NB * t + j);
+            d.kb[j] = kr + (int64_t)blk * kTile;
+            d.vtb[j] = vt + (int64_t)blk * kTile;
+        }
+    };
+    auto work = [&](int t, const KvRegs& regs) __attribute__((always_inline)) {
+        if (t < steps_both) compute_step2(st[0], st[1], bq[0], bq[1], regs);
+        else if (t < steps_both + steps_only) compute_step(st[0], bq[0], regs);
+        else compute_step(st[1], bq[1], regs);
+    };
+    StepDesc d;
+    describe(0, d);
+    load_step(ra, d, lane);
+    for (int t = 0; t < n_steps; t += 2) {
+        describe(min(t + 1, n_steps - 1), d);
+        load_step(rb, d, lane);
+        work(t, ra);
+        if (t + 1 >= n_steps) break;
+        describe(min(t + 2, n_steps - 1), d);
+        load_step(ra, d, lane);
+        work(t + 1, rb);
+    }
+    finish_query_block(a, st[0], bh, b, h, g, lane);
+    finish_query_block(a, st[1], bh, b, h, g + 1, lane);
 }
 
 }  // namespace llsa
@@ -267,6 +460,9 @@ extern "C" int llsa_attn_fwd(const llsa_attn_fwd_args* a, void* stream) {
     LLSA_REQUIRE(aligned16(a->qr) && aligned16(a->kr) && aligned16(a->vt) && aligned16(a->o), "attn_fwd: tensors must be 16-byte aligned");
     LLSA_REQUIRE((a->sob % 4 == 0) && (a->soh % 4 == 0) && (a->son % 4 == 0), "attn_fwd: rows of o must be 8-byte aligned");
     const int N1 = a->N / 16;
-    hipLaunchKernelGGL(attn_fwd_kernel, dim3((N1 + 3) / 4, a->B * a->H), dim3(256), 0, (hipStream_t)stream, *a);
+    if (a->T <= kPairMaxTopk && N1 % 8 == 0)
+        hipLaunchKernelGGL(attn_fwd_pair_kernel, dim3(N1 / 8, a->B * a->H), dim3(256), 0, (hipStream_t)stream, *a);
+    else
+        hipLaunchKernelGGL(attn_fwd_kernel, dim3((N1 + 3) / 4, a->B * a->H), dim3(256), 0, (hipStream_t)stream, *a);
     return launch_status("attn_fwd");
 }
