@@ -45,7 +45,7 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 # HBM-side bytes per launch (L2 <-> fabric, reads + writes) come from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # summaries under profiles/ (each counter scaled by what it reads for a 256 MiB elementwise copy; the files say how):
 # the table of the workload is parsed at run time, so the figure printed is the one the committed profile holds.
-TRAFFIC_KERNELS = {"attn_fwd": "attn_fwd_kernel", "bwd_dq": "attn_dq_kernel", "bwd_dkv": "attn_kside_kernel",
+TRAFFIC_KERNELS = {"attn_fwd": "attn_fwd_pair_kernel", "bwd_dq": "attn_dq_pair_kernel", "bwd_dkv": "attn_kside_kernel",
                    "bwd_pooled_groups": "attn_kside_group_kernel", "bwd_dpkv_dense": "attn_kside_dense_kernel",
                    "pool_pyramid": "pool_pyramid_kernel", "topk_sparse": "topk_sparse_kernel", "topk_dense": "topk_dense_radix_kernel"}
 

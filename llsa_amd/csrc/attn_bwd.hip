@@ -81,6 +81,57 @@ __device__ __forceinline__ void dq_accum(f32x4 dq[4], const PairT& p, bf16x8 bds
     for (int dt = 0; dt < 4; dt++) dq[dt] = mfma_bf16(cat(p.t[0][dt], p.t[1][dt]), bds, dq[dt]);
 }
 
+// What a wave keeps per query block
+struct DqSide {
+    bf16x8 bq[2], bdo[2];          // R operands of q and dO
+    float lse2, dl;                // log-sum-exp (log2 units) and delta of query l%16
+    f32x4 dq[4];                   // dQ^T: channel 16*dt + 4*(l/16) + e of query l%16
+};
+
+// dO comes straight from the caller's tensor, already in the register layout of an R operand
+// (lane l: row l%16, channels 8*(l/16)..+7 and 32 + 8*(l/16)..+7).  The wave also does the
+// pre-pass the K-side kernels need: delta = rowsum(O * dO) in fp32 (the reference sums in the
+// tensor dtype, sparse_attention_res_1.py:153-177) and dO as an R tile.
+__device__ __forceinline__ void dq_begin(DqSide& sd, const llsa_attn_bwd_args& a, float* __restrict__ delta, bf16* __restrict__ dor,
+                                         int bh, int b, int h, int g, int lane) {
+    const int N1 = a.N / kBlk, r = lane & 15, quad = lane >> 4, tok = g * kBlk + r;
+    const bf16* qp = (const bf16*)a.qr + ((int64_t)bh * N1 + g) * kTile + lane * 8;
+    sd.bq[0] = ld16(qp);
+    sd.bq[1] = ld16(qp + 512);
+    const bf16* gp = (const bf16*)a.dout + b * a.sdob + h * a.sdoh + (int64_t)tok * a.sdon + quad * 8;
+    const bf16* op = (const bf16*)a.o + b * a.sob + h * a.soh + (int64_t)tok * a.son + quad * 8;
+    sd.bdo[0] = ld16(gp);
+    sd.bdo[1] = ld16(gp + 32);
+    const bf16x8 o0 = ld16(op), o1 = ld16(op + 32);
+    float acc = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; e++) acc += (float)o0[e] * (float)sd.bdo[0][e];
+#pragma unroll
+    for (int e = 0; e < 8; e++) acc += (float)o1[e] * (float)sd.bdo[1][e];
+    sd.dl = quad_sum(acc);
+    bf16* tile = dor + ((int64_t)bh * N1 + g) * kTile + lane * 8;
+    st16(tile, sd.bdo[0]);
+    st16(tile + 512, sd.bdo[1]);
+    if (quad == 0) delta[(int64_t)bh * a.N + tok] = sd.dl;
+    sd.lse2 = a.lse[(int64_t)bh * a.N + tok] * kLog2e;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++) sd.dq[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+}
+__device__ __forceinline__ void dq_end(const DqSide& sd, const llsa_attn_bwd_args& a, int b, int h, int g, int lane) {
+    const int r = lane & 15, quad = lane >> 4, tok = g * kBlk + r;
+    bf16* op = (bf16*)a.dq + b * a.sdqb + h * a.sdqh + (int64_t)tok * a.sdqn + quad * 4;
+    const bf16* fq = a.freq_dq ? (const bf16*)a.freq_dq + (int64_t)tok * kD + quad * 4 : nullptr;
+#pragma unroll
+    for (int dt = 0; dt < 4; dt++) {
+        bf16x4 o = cvt4(sd.dq[dt] * kScale);
+        if (fq != nullptr) o = rope_bwd4(o, ld8(fq + dt * 16));   // rotate the gradient back
+        st8(op + dt * 16, o);
+    }
+}
+__device__ __forceinline__ void dq_pair_of_blocks(DqSide& sd, const PairR& r, const PairT& t, float w) {
+    dq_accum(sd.dq, t, dq_scores(r, sd.bq, sd.bdo, sd.lse2, sd.dl, w));
+}
+
 __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, float* __restrict__ delta,
                                                       bf16* __restrict__ dor) {
     __shared__ __align__(16) bf16 sh[2][kGroup][2 * kTile];   // per block: R tile of K, R tile of V
@@ -90,8 +141,6 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, floa
     const int lid = xcd_logical_id();
     const int g = (lid % (int)gridDim.x) * 4 + wave;          // < N1: the host checks N1 % 4 == 0
     const int bh = lid / (int)gridDim.x, b = bh / a.H, h = bh % a.H;
-    const int r = lane & 15, quad = lane >> 4;
-    const int tok = g * kBlk + r;
 
     const bf16* kr = (const bf16*)a.kr + (int64_t)bh * N1 * kTile;
     const bf16* vr = (const bf16*)a.vr + (int64_t)bh * N1 * kTile;
@@ -114,36 +163,8 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, floa
     issue_group(0);
     int mine = (lane < min(kWave, a.T)) ? ip[lane] : 0;       // first 64 fine indices, entry i in lane i
 
-    // dO comes straight from the caller's tensor, already in the register layout of an R operand
-    // (lane l: row l%16, channels 8*(l/16)..+7 and 32 + 8*(l/16)..+7).  The wave also does the
-    // pre-pass the K-side kernels need: delta = rowsum(O * dO) in fp32 (the reference sums in the
-    // tensor dtype, sparse_attention_res_1.py:153-177) and dO as an R tile.
-    bf16x8 bq[2], bdo[2];
-    float dl;
-    {
-        const bf16* qp = (const bf16*)a.qr + ((int64_t)bh * N1 + g) * kTile + lane * 8;
-        bq[0] = ld16(qp);
-        bq[1] = ld16(qp + 512);
-        const bf16* gp = (const bf16*)a.dout + b * a.sdob + h * a.sdoh + (int64_t)tok * a.sdon + quad * 8;
-        const bf16* op = (const bf16*)a.o + b * a.sob + h * a.soh + (int64_t)tok * a.son + quad * 8;
-        bdo[0] = ld16(gp);
-        bdo[1] = ld16(gp + 32);
-        const bf16x8 o0 = ld16(op), o1 = ld16(op + 32);
-        float acc = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; e++) acc += (float)o0[e] * (float)bdo[0][e];
-#pragma unroll
-        for (int e = 0; e < 8; e++) acc += (float)o1[e] * (float)bdo[1][e];
-        dl = quad_sum(acc);
-        bf16* tile = dor + ((int64_t)bh * N1 + g) * kTile + lane * 8;
-        st16(tile, bdo[0]);
-        st16(tile + 512, bdo[1]);
-        if (quad == 0) delta[(int64_t)bh * a.N + tok] = dl;
-    }
-    const float lse2 = a.lse[(int64_t)bh * a.N + tok] * kLog2e;
-    f32x4 dq[4];
-#pragma unroll
-    for (int dt = 0; dt < 4; dt++) dq[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    DqSide sd;
+    dq_begin(sd, a, delta, dor, bh, b, h, g, lane);
 
     // ---- pooled blocks out of the shared copy.  The barrier at the top of round grp says: every
     // wave's part of group grp has landed, and every wave is done reading the other buffer.  All
@@ -159,12 +180,12 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, floa
         read_k_r(r0, blk, blk + 2 * kTile, lane);
         read_v_r(r0, blk + kTile, blk + 3 * kTile, lane);
         read_k_t(t0, blk, blk + 2 * kTile, lane);
-        dq_accum(dq, t0, dq_scores(r0, bq, bdo, lse2, dl, w));
+        dq_pair_of_blocks(sd, r0, t0, w);
         read_k_r(r0, blk + 4 * kTile, blk + 6 * kTile, lane);
         read_v_r(r0, blk + 5 * kTile, blk + 7 * kTile, lane);
         read_k_t(t0, blk + 4 * kTile, blk + 6 * kTile, lane);
         if (grp + 1 < n_groups) issue_group(grp + 1);
-        dq_accum(dq, t0, dq_scores(r0, bq, bdo, lse2, dl, w));
+        dq_pair_of_blocks(sd, r0, t0, w);
     }
     __syncthreads();                                          // the shared copy is dead: its LDS becomes private slots
 
@@ -197,8 +218,7 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, floa
             read_k_r(cur, slot, slot + kTile, lane);
             read_k_t(tt, slot, slot + kTile, lane);
             if (t + 1 < n_pairs) fetch(t + 1, nxt);
-            const bf16x8 ds = dq_scores(cur, bq, bdo, lse2, dl, 1.f);
-            dq_accum(dq, tt, ds);
+            dq_pair_of_blocks(sd, cur, tt, 1.f);
         };
         fetch(0, ra);
         for (int t = 0; t < n_pairs; t += 2) {                // n_pairs is even (T % 4 == 0)
@@ -206,15 +226,102 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, floa
             work(t + 1, rb, ra);
         }
     }
+    dq_end(sd, a, b, h, g, lane);
+}
 
-    bf16* op = (bf16*)a.dq + b * a.sdqb + h * a.sdqh + (int64_t)tok * a.sdqn + quad * 4;
-    const bf16* fq = a.freq_dq ? (const bf16*)a.freq_dq + (int64_t)tok * kD + quad * 4 : nullptr;
-#pragma unroll
-    for (int dt = 0; dt < 4; dt++) {
-        bf16x4 o = cvt4(dq[dt] * kScale);
-        if (fq != nullptr) o = rope_bwd4(o, ld8(fq + dt * 16));   // rotate the gradient back
-        st8(op + dt * 16, o);
+// Two sibling query blocks per wave (topk <= kPairMaxTopk): the pooled blocks and the fine blocks both rows
+// selected are read once -- from memory and, what weighs more here, from LDS, where every key block is read
+// three times (K rows, V rows, K transposed) -- and multiplied twice.  See pair_order for the walk.
+__global__ __launch_bounds__(256, 3) void attn_dq_pair_kernel(llsa_attn_bwd_args a, float* __restrict__ delta,
+                                                              bf16* __restrict__ dor) {
+    __shared__ __align__(16) bf16 sh[2][kGroup][2 * kTile];
+    __shared__ int order[4][kWave];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int N1 = a.N / kBlk, T = a.T;
+    const int lid = xcd_logical_id();
+    const int g = (lid % (int)gridDim.x) * 8 + 2 * wave;      // query blocks g and g + 1 (the host checks N1 % 8 == 0)
+    const int bh = lid / (int)gridDim.x, b = bh / a.H, h = bh % a.H;
+
+    const bf16* kr = (const bf16*)a.kr + (int64_t)bh * N1 * kTile;
+    const bf16* vr = (const bf16*)a.vr + (int64_t)bh * N1 * kTile;
+    const int* ip = a.idx + ((int64_t)bh * N1 + g) * T;
+
+    SharedList sl = shared_list(a.lvl, a.levels, a.N, bh, g, lane);
+    const int n_groups = sl.n_blocks / kGroup;
+    bf16* const sh0 = &sh[0][0][0];
+    auto issue_group = [&](int grp) __attribute__((always_inline)) {
+        const SharedBlock sb = shared_block(sl, a.lvl, a.levels, a.N, bh, kGroup * grp + wave);
+        const bf16* kb = (const bf16*)a.lvl[sb.level].kr + sb.tile;
+        const bf16* vb = (const bf16*)a.lvl[sb.level].vr + sb.tile;
+        bf16* dst = sh0 + ((grp & 1) * kGroup + wave) * (2 * kTile);
+        copy16_global_to_lds(kb + lane * 8, dst);
+        copy16_global_to_lds(kb + 512 + lane * 8, dst + 512);
+        copy16_global_to_lds(vb + lane * 8, dst + kTile);
+        copy16_global_to_lds(vb + 512 + lane * 8, dst + kTile + 512);
+    };
+    issue_group(0);
+    const PairOrder po = pair_order(ip, T, N1, lane, order[wave]);
+    const int mine = po.mine;
+    const int steps_both = po.n_both / 2, steps_only = (T - po.n_both) / 2, n_steps = steps_both + 2 * steps_only;
+
+    DqSide sd[2];
+    dq_begin(sd[0], a, delta, dor, bh, b, h, g, lane);
+    dq_begin(sd[1], a, delta, dor, bh, b, h, g + 1, lane);
+
+    for (int grp = 0; grp < n_groups; grp++) {
+        wait_vm0();
+        __syncthreads();
+        const float w = a.lvl[shared_level(a.lvl, a.levels, kGroup * grp)].w;
+        const bf16* blk = sh0 + (grp & 1) * kGroup * (2 * kTile);
+        PairR r0;
+        PairT t0;
+        read_k_r(r0, blk, blk + 2 * kTile, lane);
+        read_v_r(r0, blk + kTile, blk + 3 * kTile, lane);
+        read_k_t(t0, blk, blk + 2 * kTile, lane);
+        dq_pair_of_blocks(sd[0], r0, t0, w);
+        dq_pair_of_blocks(sd[1], r0, t0, w);
+        read_k_r(r0, blk + 4 * kTile, blk + 6 * kTile, lane);
+        read_v_r(r0, blk + 5 * kTile, blk + 7 * kTile, lane);
+        read_k_t(t0, blk + 4 * kTile, blk + 6 * kTile, lane);
+        if (grp + 1 < n_groups) issue_group(grp + 1);
+        dq_pair_of_blocks(sd[0], r0, t0, w);
+        dq_pair_of_blocks(sd[1], r0, t0, w);
     }
+    __syncthreads();
+
+    bf16* const priv = sh0 + wave * (4 * kTile);
+    PairR ra, rb;
+    auto fetch = [=](int t, PairR& dst) __attribute__((always_inline)) {
+        bf16* slot = priv + (t & 1) * (2 * kTile);
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            const int blk = __builtin_amdgcn_readlane(mine, 2 * t + j);
+            const bf16* kb = kr + (int64_t)blk * kTile;
+            const bf16* vb = vr + (int64_t)blk * kTile;
+            copy16_global_to_lds(kb + lane * 8, slot + j * kTile);
+            copy16_global_to_lds(kb + 512 + lane * 8, slot + j * kTile + 512);
+            dst.v[j][0] = ld16(vb + lane * 8);
+            dst.v[j][1] = ld16(vb + 512 + lane * 8);
+        }
+    };
+    auto work = [&](int t, PairR& cur, PairR& nxt) __attribute__((always_inline)) {
+        wait_vm0();
+        const bf16* slot = priv + (t & 1) * (2 * kTile);
+        PairT tt;
+        read_k_r(cur, slot, slot + kTile, lane);
+        read_k_t(tt, slot, slot + kTile, lane);
+        if (t + 1 < n_steps) fetch(t + 1, nxt);
+        if (t < steps_both + steps_only) dq_pair_of_blocks(sd[0], cur, tt, 1.f);
+        if (t < steps_both || t >= steps_both + steps_only) dq_pair_of_blocks(sd[1], cur, tt, 1.f);
+    };
+    fetch(0, ra);
+    for (int t = 0; t < n_steps; t += 2) {
+        work(t, ra, rb);
+        if (t + 1 < n_steps) work(t + 1, rb, ra);
+    }
+    dq_end(sd[0], a, b, h, g, lane);
+    dq_end(sd[1], a, b, h, g + 1, lane);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -1063,7 +1170,10 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
 
     const int stages = a->stages ? a->stages : (0x7fffffff & ~LLSA_BWD_NO_REDUCE);
     if (stages & LLSA_BWD_DQ)
-        hipLaunchKernelGGL(attn_dq_kernel, dim3((N1 + 3) / 4, BH), dim3(256), 0, s, *a, delta, dor);
+        if (a->T <= kPairMaxTopk && N1 % 8 == 0)
+            hipLaunchKernelGGL(attn_dq_pair_kernel, dim3(N1 / 8, BH), dim3(256), 0, s, *a, delta, dor);
+        else
+            hipLaunchKernelGGL(attn_dq_kernel, dim3((N1 + 3) / 4, BH), dim3(256), 0, s, *a, delta, dor);
 
     ReduceParams rp;
     rp.n_jobs = 0;

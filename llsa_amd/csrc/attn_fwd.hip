@@ -299,7 +299,6 @@ __global__ __launch_bounds__(256, 4) void attn_fwd_kernel(llsa_attn_fwd_args a) 
 // kernels is the rate at which tiles arrive from the L2, and this removes a quarter to a half of them.
 // A row that names a block twice keeps the plain walk (nothing is shared).
 // ---------------------------------------------------------------------------------------
-constexpr int kPairMaxTopk = 32;
 
 __global__ __launch_bounds__(256, 3) void attn_fwd_pair_kernel(llsa_attn_fwd_args a) {
     static_assert(NB == 2 && kGroup == 4, "the shared phase reads an LDS buffer of four blocks as two steps of two");
@@ -332,37 +331,9 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_pair_kernel(llsa_attn_fwd_arg
     issue_group(0);
 
     // ---- the two fine lists, sorted into [both | only the first | only the second]; entry i ends in lane i
-    const int first = (lane < T) ? clampi(ip[lane], 0, N1 - 1) : -1 - lane;       // (distinct negative fillers)
-    const int second = (lane < T) ? clampi(ip[T + lane], 0, N1 - 1) : -65 - lane;
-    bool in_second = false, in_first = false, twice = false;
-    for (int j = 0; j < T; j++) {
-        const int fj = __builtin_amdgcn_readlane(first, j), sj = __builtin_amdgcn_readlane(second, j);
-        in_second |= first == sj;
-        in_first |= second == fj;
-        twice |= (first == fj && lane != j) || (second == sj && lane != j);
-    }
-    if (__ballot(twice) != 0) in_second = in_first = false;
-    unsigned long long both = __ballot(in_second);
-    if (__popcll(both) & 1) {                                 // an even number is shared: steps hold NB = 2 blocks
-        const int last = 63 - __builtin_clzll(both);
-        const int dropped = __builtin_amdgcn_readlane(first, last);
-        in_second = in_second && lane != last;
-        in_first = in_first && second != dropped;
-        both &= ~(1ull << last);
-    }
-    const int n_both = __popcll(both), n_only = T - n_both;
-    {
-        const unsigned long long below = (1ull << lane) - 1ull;
-        const unsigned long long only1 = __ballot(lane < T && !in_second), only2 = __ballot(lane < T && !in_first);
-        int* mine = order[wave];
-        if (lane < T) mine[in_second ? __popcll(both & below) : n_both + __popcll(only1 & below)] = first;
-        if (lane < T && !in_first) mine[n_both + n_only + __popcll(only2 & below)] = second;
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const int mine = order[wave][lane];                        // entries [0, n_both + 2 * n_only) are meaningful
-    const int steps_both = n_both / NB, steps_only = n_only / NB, n_steps = steps_both + 2 * steps_only;
+    const PairOrder po = pair_order(ip, T, N1, lane, order[wave]);
+    const int mine = po.mine;
+    const int steps_both = po.n_both / NB, steps_only = (T - po.n_both) / NB, n_steps = steps_both + 2 * steps_only;
 
     bf16x8 bq[2][2];
 #pragma unroll

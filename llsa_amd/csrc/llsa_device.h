@@ -210,6 +210,48 @@ __device__ __forceinline__ SharedBlock shared_block(const SharedList& sl, const 
     return sb;
 }
 
+// The fine lists of two sibling query blocks (rows ip[0..T) and ip[T..2T), T <= kPairMaxTopk), sorted into
+// [blocks both rows name | only the first | only the second]: entry i of that order ends in lane i (2T - n_both
+// entries), indices clamped to [0, N1).  n_both is even (an odd common block out is listed once for each row).
+// A row that names a block twice shares nothing (n_both = 0).  `scratch`: kWave ints of LDS private to the wave.
+constexpr int kPairMaxTopk = 32;
+struct PairOrder {
+    int mine;
+    int n_both;
+};
+__device__ __forceinline__ PairOrder pair_order(const int* ip, int T, int N1, int lane, int* scratch) {
+    const int first = (lane < T) ? clampi(ip[lane], 0, N1 - 1) : -1 - lane;       // (distinct negative fillers)
+    const int second = (lane < T) ? clampi(ip[T + lane], 0, N1 - 1) : -65 - lane;
+    bool in_second = false, in_first = false, twice = false;
+    for (int j = 0; j < T; j++) {
+        const int fj = __builtin_amdgcn_readlane(first, j), sj = __builtin_amdgcn_readlane(second, j);
+        in_second |= first == sj;
+        in_first |= second == fj;
+        twice |= (first == fj && lane != j) || (second == sj && lane != j);
+    }
+    if (__ballot(twice) != 0) in_second = in_first = false;
+    unsigned long long both = __ballot(in_second);
+    if (__popcll(both) & 1) {
+        const int last = 63 - __builtin_clzll(both);
+        const int dropped = __builtin_amdgcn_readlane(first, last);
+        in_second = in_second && lane != last;
+        in_first = in_first && second != dropped;
+        both &= ~(1ull << last);
+    }
+    const int n_both = __popcll(both), n_only = T - n_both;
+    const unsigned long long below = (1ull << lane) - 1ull;
+    const unsigned long long only1 = __ballot(lane < T && !in_second), only2 = __ballot(lane < T && !in_first);
+    if (lane < T) scratch[in_second ? __popcll(both & below) : n_both + __popcll(only1 & below)] = first;
+    if (lane < T && !in_first) scratch[n_both + n_only + __popcll(only2 & below)] = second;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    PairOrder po;
+    po.mine = scratch[lane];
+    po.n_both = n_both;
+    return po;
+}
+
 // 16- and 8-byte reads that are LDS reads by construction (ds_read_b128 / ds_read_b64)
 __device__ __forceinline__ bf16x8 lds_ld16(const bf16* p) {
     return *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>((const __attribute__((address_space(3))) bf16*)p);
