@@ -388,63 +388,57 @@ struct KSideParams {
     PoolFold fold;                                // fine pass only
 };
 
-// Two query blocks (g0, g1; g1 < 0: only one) against the unit's 16 key rows.  Q and dO are
-// fetched once, as R tiles: they are the A operands of S = Q.K^T and dP = dO.V^T straight from
-// the registers, and they are parked in a wave-private piece of LDS (`stage`, 4096 elements)
-// from which the transposing LDS read delivers them again as T operands for dV^T += dO^T.P and
-// dK^T += Q^T.dS.
-__device__ __forceinline__ void kside_pair(f32x4 dk[4], f32x4 dv[4], const bf16x8 bk[2], const bf16x8 bv[2],
-                                           int g0, int g1, const bf16* qrb, const bf16* dorb, const float* lseb,
-                                           const float* dlb, bf16* stage, int lane) {
-    const int quad = lane >> 4;
-    const int gg[2] = {g0, (g1 < 0) ? g0 : g1};
+// Two query blocks against the unit's 16 key rows, operands out of a wave-private piece of LDS: `stage` holds the
+// R tiles of Q and dO of the two blocks (block u: Q at 2u, dO at 2u + 1), `stats` their lse and delta rows.  The tiles
+// are read twice, plainly as the A operands of S = Q.K^T and dP = dO.V^T and with the transposing read as the T
+// operands of dV^T += dO^T.P and dK^T += Q^T.dS.
+struct KsideOperands {
     bf16x8 aq[2][2], ag[2][2];
+    bf16x4 tq[2][4], tg[2][4];
     f32x4 l4[2], d4[2];
+};
+__device__ __forceinline__ void kside_read(KsideOperands& o, const bf16* stage, const float* stats, int lane) {
+    const int quad = lane >> 4;
 #pragma unroll
     for (int u = 0; u < 2; u++) {
-        const int64_t base = (int64_t)gg[u] * kTile;
-        aq[u][0] = ld16(qrb + base + lane * 8);
-        aq[u][1] = ld16(qrb + base + 512 + lane * 8);
-        ag[u][0] = ld16(dorb + base + lane * 8);
-        ag[u][1] = ld16(dorb + base + 512 + lane * 8);
-        l4[u] = *reinterpret_cast<const f32x4*>(lseb + gg[u] * kBlk + quad * 4);
-        d4[u] = *reinterpret_cast<const f32x4*>(dlb + gg[u] * kBlk + quad * 4);
-    }
+        const bf16* q = stage + (2 * u) * kTile;
+        const bf16* g = stage + (2 * u + 1) * kTile;
+        o.aq[u][0] = lds_ld16(q + lane * 8);
+        o.aq[u][1] = lds_ld16(q + 512 + lane * 8);
+        o.ag[u][0] = lds_ld16(g + lane * 8);
+        o.ag[u][1] = lds_ld16(g + 512 + lane * 8);
 #pragma unroll
-    for (int u = 0; u < 2; u++) {
-        st16(stage + (u * 2 + 0) * kTile + lane * 8, aq[u][0]);
-        st16(stage + (u * 2 + 0) * kTile + 512 + lane * 8, aq[u][1]);
-        st16(stage + (u * 2 + 1) * kTile + lane * 8, ag[u][0]);
-        st16(stage + (u * 2 + 1) * kTile + 512 + lane * 8, ag[u][1]);
+        for (int dt = 0; dt < 4; dt++) {
+            o.tq[u][dt] = lds_t_operand(q, dt, lane);
+            o.tg[u][dt] = lds_t_operand(g, dt, lane);
+        }
+        o.l4[u] = *reinterpret_cast<const f32x4*>(stats + u * 32 + quad * 4);
+        o.d4[u] = *reinterpret_cast<const f32x4*>(stats + u * 32 + 16 + quad * 4);
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
+}
+__device__ __forceinline__ void kside_pair(f32x4 dk[4], f32x4 dv[4], const bf16x8 bk[2], const bf16x8 bv[2], const KsideOperands& o,
+                                           bool second_valid) {
     bf16x8 bp, bds;
 #pragma unroll
     for (int u = 0; u < 2; u++) {
-        const bool valid = (u == 0) || (g1 >= 0);
         f32x4 s = {0.f, 0.f, 0.f, 0.f}, dp = {0.f, 0.f, 0.f, 0.f};
-        s = mfma_bf16(aq[u][0], bk[0], s);
-        s = mfma_bf16(aq[u][1], bk[1], s);
-        dp = mfma_bf16(ag[u][0], bv[0], dp);
-        dp = mfma_bf16(ag[u][1], bv[1], dp);
+        s = mfma_bf16(o.aq[u][0], bk[0], s);
+        s = mfma_bf16(o.aq[u][1], bk[1], s);
+        dp = mfma_bf16(o.ag[u][0], bv[0], dp);
+        dp = mfma_bf16(o.ag[u][1], bv[1], dp);
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            float pe = exp2_fast(fmaf(s[e], kScaleLog2e, -l4[u][e] * kLog2e));
-            if (!valid) pe = 0.f;
+            float pe = exp2_fast(fmaf(s[e], kScaleLog2e, -o.l4[u][e] * kLog2e));
+            if (u == 1 && !second_valid) pe = 0.f;
             bp[u * 4 + e] = (bf16)pe;
-            bds[u * 4 + e] = (bf16)(pe * (dp[e] - d4[u][e]));
+            bds[u * 4 + e] = (bf16)(pe * (dp[e] - o.d4[u][e]));
         }
     }
 #pragma unroll
     for (int dt = 0; dt < 4; dt++) {
-        const bf16x4 tg0 = lds_t_operand(stage + 1 * kTile, dt, lane), tg1 = lds_t_operand(stage + 3 * kTile, dt, lane);
-        const bf16x4 tq0 = lds_t_operand(stage + 0 * kTile, dt, lane), tq1 = lds_t_operand(stage + 2 * kTile, dt, lane);
-        dv[dt] = mfma_bf16(cat(tg0, tg1), bp, dv[dt]);
-        dk[dt] = mfma_bf16(cat(tq0, tq1), bds, dk[dt]);
+        dv[dt] = mfma_bf16(cat(o.tg[0][dt], o.tg[1][dt]), bp, dv[dt]);
+        dk[dt] = mfma_bf16(cat(o.tq[0][dt], o.tq[1][dt]), bds, dk[dt]);
     }
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_wave_barrier();              // the next pair overwrites `stage`
 }
 
 // A partial sum of one unit (16 key rows x 64 channels, dK and dV) is kept in the MFMA
@@ -456,6 +450,7 @@ __device__ __forceinline__ f32x4* part_slot(f32x4* part, int64_t slot) { return 
 // with a longer one would keep its registers and LDS allocated while idle).
 __global__ __launch_bounds__(64) void attn_kside_kernel(KSideParams p) {
     __shared__ __align__(16) bf16 stage[4 * kTile];           // 2 query blocks x {Q, dO} R tiles
+    __shared__ __align__(16) float stats[64];                 // their lse and delta rows
     __shared__ __align__(16) bf16 fold_buf[kFoldElems];
     const int lid = xcd_logical_id();
     const int item = lid % (int)gridDim.x;
@@ -527,10 +522,38 @@ __global__ __launch_bounds__(64) void attn_kside_kernel(KSideParams p) {
         const bf16* dorb = p.dor + (int64_t)bh * N1 * kTile;
         const float* lseb = p.lse + (int64_t)bh * p.N;
         const float* dlb = p.delta + (int64_t)bh * p.N;
-        for (int i = 0; i < cnt; i += 2) {
+        // The operands of entries i, i + 1 are copied straight into LDS (no registers) while entries i - 2, i - 1 are
+        // worked on: a round reads everything it needs out of LDS first, then starts the next copy into the same
+        // place, then does its arithmetic.
+        auto fetch = [&](int i) __attribute__((always_inline)) {
             const int g0 = entry(i);
-            const int g1 = (i + 1 < cnt) ? entry(i + 1) : -1;
-            kside_pair(dk, dv, bk, bv, g0, g1, qrb, dorb, lseb, dlb, stage, lane);
+            const int g1 = (i + 1 < cnt) ? entry(i + 1) : g0;
+            const bf16* q0 = qrb + (int64_t)g0 * kTile + lane * 8;
+            const bf16* d0 = dorb + (int64_t)g0 * kTile + lane * 8;
+            const bf16* q1 = qrb + (int64_t)g1 * kTile + lane * 8;
+            const bf16* d1 = dorb + (int64_t)g1 * kTile + lane * 8;
+            copy16_global_to_lds(q0, stage);
+            copy16_global_to_lds(q0 + 512, stage + 512);
+            copy16_global_to_lds(d0, stage + kTile);
+            copy16_global_to_lds(d0 + 512, stage + kTile + 512);
+            copy16_global_to_lds(q1, stage + 2 * kTile);
+            copy16_global_to_lds(q1 + 512, stage + 2 * kTile + 512);
+            copy16_global_to_lds(d1, stage + 3 * kTile);
+            copy16_global_to_lds(d1 + 512, stage + 3 * kTile + 512);
+            if (lane < 16) {                                  // four floats a lane: lse g0, delta g0, lse g1, delta g1
+                const float* src = ((lane & 4) ? dlb : lseb) + ((lane & 8) ? g1 : g0) * kBlk + (lane & 3) * 4;
+                copy16_global_to_lds(reinterpret_cast<const bf16*>(src), reinterpret_cast<bf16*>(stats));
+            }
+        };
+        if (cnt > 0) fetch(0);
+        for (int i = 0; i < cnt; i += 2) {
+            wait_vm0();
+            KsideOperands o;
+            kside_read(o, stage, stats, lane);
+            wait_all_mem();                                   // every lane has its operands: the next copy may land
+            __builtin_amdgcn_wave_barrier();
+            if (i + 2 < cnt) fetch(i + 2);
+            kside_pair(dk, dv, bk, bv, o, i + 1 < cnt);
         }
     }
 
