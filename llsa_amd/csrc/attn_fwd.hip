@@ -33,7 +33,7 @@ struct SoftmaxState {
 // Operands of one step = NB 16-key blocks, as they sit in registers between load and use.
 struct KvRegs {
     bf16x8 k[NB][2];     // K rows (R tile): block j, channel half
-    bf16x4 v[NB][4];     // V (T tile): block j, channel tile dt, keys 4*(l/16)..+3
+    bf16x8 v[NB / 2][4]; // V (T tiles of a pair of blocks): channel tile dt, keys 4*(l/16)..+3 of the first block, then of the second
 };
 
 // Where one step's blocks live: kb[j] is the R tile of key block j, vtb[j] the T tile of its values.
@@ -48,10 +48,12 @@ __device__ __forceinline__ void load_step(KvRegs& t, const StepDesc& d, int lane
         t.k[j][0] = ld16(d.kb[j] + lane * 8);
         t.k[j][1] = ld16(d.kb[j] + 512 + lane * 8);
     }
+    // (the two halves of an operand are loaded one after the other so that they land in adjacent registers)
 #pragma unroll
-    for (int j = 0; j < NB; j++)
+    for (int c = 0; c < NB / 2; c++)
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++) t.v[j][dt] = ld8(d.vtb[j] + dt * 256 + lane * 4);
+        for (int dt = 0; dt < 4; dt++)
+            t.v[c][dt] = cat(ld8(d.vtb[2 * c] + dt * 256 + lane * 4), ld8(d.vtb[2 * c + 1] + dt * 256 + lane * 4));
 }
 
 __device__ __forceinline__ void init_state(SoftmaxState& st) {
@@ -126,7 +128,7 @@ __device__ __forceinline__ void accumulate(SoftmaxState& st, const float x[NB][4
     for (int c = 0; c < NB / 2; c++)
 #pragma unroll
         for (int dt = 0; dt < 4; dt++)
-            st.acc[dt] = mfma_bf16(cat(t.v[2 * c][dt], t.v[2 * c + 1][dt]), bp[c], st.acc[dt]);
+            st.acc[dt] = mfma_bf16(t.v[c][dt], bp[c], st.acc[dt]);
 }
 
 __device__ __forceinline__ void compute_step(SoftmaxState& st, const bf16x8 bq[2], const KvRegs& t) {
@@ -161,9 +163,13 @@ __device__ __forceinline__ void load_step_lds(KvRegs& t, const bf16* blocks, int
         t.k[j][1] = lds_ld16(blocks + j * 2 * kTile + 512 + lane * 8);
     }
 #pragma unroll
-    for (int j = 0; j < NB; j++)
+    for (int c = 0; c < NB / 2; c++)
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++) t.v[j][dt] = lds_ld8(blocks + j * 2 * kTile + kTile + dt * 256 + lane * 4);
+        for (int dt = 0; dt < 4; dt++) {
+            t.v[c][dt] = cat(lds_ld8(blocks + (2 * c) * 2 * kTile + kTile + dt * 256 + lane * 4),
+                             lds_ld8(blocks + (2 * c + 1) * 2 * kTile + kTile + dt * 256 + lane * 4));
+            __builtin_amdgcn_sched_barrier(0);    // (keeps the two reads one paired LDS read: paired with any other read they need moves)
+        }
 }
 
 __device__ __forceinline__ void finish_query_block(const llsa_attn_fwd_args& a, const SoftmaxState& st, int bh, int b, int h, int g, int lane) {

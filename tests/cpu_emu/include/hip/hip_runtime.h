@@ -123,6 +123,7 @@ inline int __clz(int x) { return x ? __builtin_clz((unsigned)x) : 32; }
 #define __builtin_amdgcn_logf(x) log2f(x)
 #define __builtin_amdgcn_rcpf(x) (1.0f / (x))
 #define __builtin_amdgcn_s_setprio(x) ((void)0)
+#define __builtin_amdgcn_sched_barrier(x) ((void)0)
 #define __builtin_amdgcn_wave_barrier() emu::wave_sync()
 #define __builtin_amdgcn_global_load_lds(g, l, size, off, aux) \
     __builtin_memcpy((char*)(l) + (size) * emu::lane_id(), (const char*)(g), (size))
