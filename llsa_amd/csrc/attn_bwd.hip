@@ -58,8 +58,9 @@ __device__ __forceinline__ void read_k_t(PairT& o, const bf16* k0, const bf16* k
     }
 }
 // dS^T of a pair of key blocks, as the B operand of the dQ product
-__device__ __forceinline__ bf16x8 dq_scores(const PairR& p, const bf16x8 bq[2], const bf16x8 bdo[2], float lse2,
-                                            float delta, float w) {
+// (lse2w: the query's log-sum-exp minus log2 of the segment's weight, log2 units: the weight rides in the exponent)
+__device__ __forceinline__ bf16x8 dq_scores(const PairR& p, const bf16x8 bq[2], const bf16x8 bdo[2], float lse2w,
+                                            float delta) {
     bf16x8 bds;
 #pragma unroll
     for (int j = 0; j < 2; j++) {
@@ -70,7 +71,7 @@ __device__ __forceinline__ bf16x8 dq_scores(const PairR& p, const bf16x8 bq[2], 
         dp = mfma_bf16(p.v[j][1], bdo[1], dp);
 #pragma unroll
         for (int e = 0; e < 4; e++) {
-            const float pe = exp2_fast(fmaf(s[e], kScaleLog2e, -lse2)) * w;
+            const float pe = exp2_fast(fmaf(s[e], kScaleLog2e, -lse2w));
             bds[j * 4 + e] = (bf16)(pe * (dp[e] - delta));
         }
     }
@@ -128,8 +129,8 @@ __device__ __forceinline__ void dq_end(const DqSide& sd, const llsa_attn_bwd_arg
         st8(op + dt * 16, o);
     }
 }
-__device__ __forceinline__ void dq_pair_of_blocks(DqSide& sd, const PairR& r, const PairT& t, float w) {
-    dq_accum(sd.dq, t, dq_scores(r, sd.bq, sd.bdo, sd.lse2, sd.dl, w));
+__device__ __forceinline__ void dq_pair_of_blocks(DqSide& sd, const PairR& r, const PairT& t, float log2w) {
+    dq_accum(sd.dq, t, dq_scores(r, sd.bq, sd.bdo, sd.lse2 - log2w, sd.dl));
 }
 
 __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, float* __restrict__ delta,
@@ -173,7 +174,7 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, floa
     for (int grp = 0; grp < n_groups; grp++) {
         wait_vm0();
         __syncthreads();
-        const float w = a.lvl[shared_level(a.lvl, a.levels, kGroup * grp)].w;
+        const float w = __builtin_amdgcn_logf(a.lvl[shared_level(a.lvl, a.levels, kGroup * grp)].w);   // log2
         const bf16* blk = sh0 + (grp & 1) * kGroup * (2 * kTile);
         PairR r0;
         PairT t0;
@@ -218,7 +219,7 @@ __global__ __launch_bounds__(256) void attn_dq_kernel(llsa_attn_bwd_args a, floa
             read_k_r(cur, slot, slot + kTile, lane);
             read_k_t(tt, slot, slot + kTile, lane);
             if (t + 1 < n_pairs) fetch(t + 1, nxt);
-            dq_pair_of_blocks(sd, cur, tt, 1.f);
+            dq_pair_of_blocks(sd, cur, tt, 0.f);
         };
         fetch(0, ra);
         for (int t = 0; t < n_pairs; t += 2) {                // n_pairs is even (T % 4 == 0)
@@ -269,11 +270,12 @@ __global__ __launch_bounds__(256, 3) void attn_dq_pair_kernel(llsa_attn_bwd_args
     dq_begin(sd[0], a, delta, dor, bh, b, h, g, lane);
     dq_begin(sd[1], a, delta, dor, bh, b, h, g + 1, lane);
 
-    for (int grp = 0; grp < n_groups; grp++) {
+    // (two groups per trip: the buffer a group sits in is then a constant and every LDS address a lane-invariant
+    // base plus an immediate)
+    auto shared_group = [&](int grp, const bf16* blk) __attribute__((always_inline)) {
         wait_vm0();
         __syncthreads();
-        const float w = a.lvl[shared_level(a.lvl, a.levels, kGroup * grp)].w;
-        const bf16* blk = sh0 + (grp & 1) * kGroup * (2 * kTile);
+        const float w = __builtin_amdgcn_logf(a.lvl[shared_level(a.lvl, a.levels, kGroup * grp)].w);   // log2
         PairR r0;
         PairT t0;
         read_k_r(r0, blk, blk + 2 * kTile, lane);
@@ -287,6 +289,10 @@ __global__ __launch_bounds__(256, 3) void attn_dq_pair_kernel(llsa_attn_bwd_args
         if (grp + 1 < n_groups) issue_group(grp + 1);
         dq_pair_of_blocks(sd[0], r0, t0, w);
         dq_pair_of_blocks(sd[1], r0, t0, w);
+    };
+    for (int grp = 0; grp < n_groups; grp += 2) {
+        shared_group(grp, sh0);
+        if (grp + 1 < n_groups) shared_group(grp + 1, sh0 + kGroup * (2 * kTile));
     }
     __syncthreads();
 
@@ -312,8 +318,8 @@ __global__ __launch_bounds__(256, 3) void attn_dq_pair_kernel(llsa_attn_bwd_args
         read_k_r(cur, slot, slot + kTile, lane);
         read_k_t(tt, slot, slot + kTile, lane);
         if (t + 1 < n_steps) fetch(t + 1, nxt);
-        if (t < steps_both + steps_only) dq_pair_of_blocks(sd[0], cur, tt, 1.f);
-        if (t < steps_both || t >= steps_both + steps_only) dq_pair_of_blocks(sd[1], cur, tt, 1.f);
+        if (t < steps_both + steps_only) dq_pair_of_blocks(sd[0], cur, tt, 0.f);
+        if (t < steps_both || t >= steps_both + steps_only) dq_pair_of_blocks(sd[1], cur, tt, 0.f);
     };
     fetch(0, ra);
     for (int t = 0; t < n_steps; t += 2) {
