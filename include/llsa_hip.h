@@ -164,7 +164,10 @@ int llsa_topk_sparse(const void* pq, const void* pk, const int32_t* parent_idx, 
  * coarsest level.  levels = 1 is llsa_l1 (sparse_attention_res_1.py), levels = 2 llsa_l2
  * (sparse_attention_res_2.py); deeper hierarchies have no counterpart in the reference and continue
  * the scheme by induction on sparse_attention_res_2.py:94-149.  The coarsest level is walked in
- * groups of four blocks: N must be a multiple of 64 * 16^levels.
+ * groups of four blocks: N must be a multiple of 64 * 16^levels.  Indices outside their range are
+ * clamped into it; a row of idx that names a block twice counts it twice in the forward and in dq
+ * (as the reference's gather does) -- the K-side gradients need distinct entries, see
+ * llsa_transpose_indices.
  * ---------------------------------------------------------------------------------------- */
 #define LLSA_MAX_LEVELS 4
 

@@ -271,6 +271,23 @@ def check_attn_l1(dev, B=1, H=2, N=1024, T=8, strided=False, smooth=False, weigh
                                                 **kw), N)
 
 
+def check_attn_fwd_repeated_block(dev, B=1, H=2, N=1024, T=8):
+    """The forward kernel with rows that name a block twice (a caller's indices may; a top-k output does not): such
+    a row counts the block twice, like the reference's gather, and the sibling row that shares a wave with it must
+    not be affected.  Every fourth query block repeats its first entry in its last."""
+    from llsa_amd.kernel.hip._attention import attn_fwd
+    q, k, v, _ = randn_inputs(B, H, N, 64, dev, seed=31)
+    qc, kc, vc = (t.cpu() for t in (q, k, v))
+    pk, pv = O.mean_pool(kc), O.mean_pool(vc)
+    idx = _selection_l1(qc, kc, T).clone()
+    idx[:, :, ::4, T - 1] = idx[:, :, ::4, 0]
+    idx[:, :, 1::8, 1] = idx[:, :, 0::8, 0]              # and some siblings that share blocks with the repeating row
+    o, lse = attn_fwd(q, k, v, pk.to(dev), pv.to(dev), idx.int().to(dev), 16.0)
+    ro, rl = O.attn_fwd_l1(qc, kc, vc, pk, pv, idx, 16.0)
+    close("o", o, ro)
+    assert (lse.cpu() - rl).abs().max() < 2e-3, f"lse differs by {(lse.cpu() - rl).abs().max():.3e}"
+
+
 def check_attn_l2(dev, B=1, H=1, N=16384, T=8, T2=4, smooth=False, hot=None):
     from llsa_amd.kernel.hip._attention import attn_bwd, attn_fwd
     q, k, v, do = smooth_inputs(B, H, N, 64, dev) if smooth else randn_inputs(B, H, N, 64, dev, seed=15)

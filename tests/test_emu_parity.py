@@ -80,6 +80,7 @@ def test_attn_l1_hot_block():
 def test_attn_special_cases():
     P.check_attn_reduces_to_sdpa(DEV, B=1, H=1, N=1024)
     P.check_constant_v(DEV)
+    P.check_attn_fwd_repeated_block(DEV, B=1, H=1, N=1024, T=8)
 
 
 @pytest.mark.parametrize("fused,rope", [(True, False), (True, True), (False, False)])

@@ -115,6 +115,7 @@ def test_attn_hot_blocks(dev):
 def test_attn_special_cases(dev):
     P.check_attn_reduces_to_sdpa(dev, B=1, H=2, N=1024)
     P.check_constant_v(dev)
+    P.check_attn_fwd_repeated_block(dev)
 
 
 @pytest.mark.parametrize("smooth", [False, True])
