@@ -44,7 +44,7 @@ extern "C" {
 #define LLSA_DTYPE_BF16 0
 #define LLSA_DTYPE_F32 1
 
-#define LLSA_ABI_VERSION 200     /* changes with every change of a signature or argument structure below */
+#define LLSA_ABI_VERSION 201     /* changes with every change of a signature or argument structure below */
 int llsa_version(void);          /* LLSA_ABI_VERSION of the built library                                    */
 const char* llsa_last_error_string(void);
 
@@ -154,6 +154,13 @@ int llsa_topk_dense(const void* pq, const void* pk, int32_t* out_idx, int B, int
                     int round_scores, void* stream);
 int llsa_topk_sparse(const void* pq, const void* pk, const int32_t* parent_idx, int32_t* out_idx,
                      int B, int H, int N1, int T, int T2, void* stream);
+/* llsa_topk_dense on the parent level followed by llsa_topk_sparse under its result, in one launch
+ * (every workgroup of the second selection first selects its own parent row): the same two results,
+ * parent_out (B,H,N1/16,T2) and out_idx (B,H,N1,T).  pq_parent, pk_parent (B,H,N1/16,64) are the pooled
+ * rows one level above pq, pk (B,H,N1,64).  N1/16 may not exceed llsa_topk_cascade_max_parents(). */
+int llsa_topk_cascade(const void* pq_parent, const void* pk_parent, int32_t* parent_out, const void* pq, const void* pk,
+                      int32_t* out_idx, int B, int H, int N1, int T, int T2, void* stream);
+int llsa_topk_cascade_max_parents(void);
 
 /* ------------------------------------------------------------------------------------------
  * The hierarchy.  Pooled level l = 1 .. levels: its tokens are means of 16^l input tokens and weigh

@@ -82,6 +82,8 @@ _SIGNATURES = {
     "llsa_rope_bwd": (c_int, [c_void_p, P64, c_void_p, c_void_p, P64, c_int, c_int, c_int, c_void_p]),
     "llsa_topk_dense": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llsa_topk_sparse": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "llsa_topk_cascade": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "llsa_topk_cascade_max_parents": (c_int, []),
     "llsa_attn_fwd": (c_int, [C.POINTER(AttnFwdArgs), c_void_p]),
     "llsa_transpose_indices": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llsa_work_list_len": (c_int64, [c_int, c_int, c_int, c_int]),
@@ -91,7 +93,7 @@ _SIGNATURES = {
 
 EXPORTS = tuple(_SIGNATURES)
 CHUNK_FINE = 64                                             # LLSA_CHUNK_FINE of include/llsa_hip.h
-ABI_VERSION = 200                                           # LLSA_ABI_VERSION
+ABI_VERSION = 201                                           # LLSA_ABI_VERSION
 STATIC_PARTIALS_MAX = 262144                                # LLSA_STATIC_PARTIALS_MAX
 
 

@@ -265,13 +265,19 @@ __global__ __launch_bounds__(1024) void topk_dense_radix_kernel(const bf16* __re
 }
 
 constexpr int kSparseWaves = 8;       // two rows per wave: four workgroups fit a CU and the grid is one round
+// pq_par != nullptr: the parents are selected here first -- row G of the level above (N1/16 tokens, at most
+// kCascadeMaxParents) against all of its keys, scores rounded to bf16, top T2 as topk_dense_radix_kernel does it -- and
+// written to par_out; otherwise they are read from pidx.
 __global__ __launch_bounds__(64 * kSparseWaves) void topk_sparse_kernel(const bf16* __restrict__ pq, const bf16* __restrict__ pk,
                                                            const int* __restrict__ pidx, int* __restrict__ out, int N1,
-                                                           int T, int T2) {
+                                                           int T, int T2, const bf16* __restrict__ pq_par,
+                                                           const bf16* __restrict__ pk_par, int* __restrict__ par_out) {
     __shared__ unsigned su[16][kMaxCand + 1];
     __shared__ int cand[kMaxCand];
     __shared__ unsigned sel_u[16][kWave];
     __shared__ int sel_i[16][kWave];
+    __shared__ int par[kMaxCand / 16];
+    static_assert(16 * (kMaxCand + 1) >= kRadixMaxN, "the parents' scores borrow the candidates' score rows");
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int bh = blockIdx.y, G = blockIdx.x;
@@ -279,8 +285,30 @@ __global__ __launch_bounds__(64 * kSparseWaves) void topk_sparse_kernel(const bf
     const bf16* pqb = pq + ((int64_t)bh * N1 + G * kBlk) * kD;
     const bf16* pkb = pk + (int64_t)bh * N1 * kD;
 
-    for (int i = tid; i < C; i += 64 * kSparseWaves)
-        cand[i] = clampi(pidx[((int64_t)bh * N2 + G) * T2 + i / kBlk], 0, N2 - 1) * kBlk + (i % kBlk);
+    if (pq_par != nullptr) {
+        unsigned* su_par = &su[0][0];
+        const bf16* qt = pq_par + ((int64_t)bh * N2 + (G & ~15)) * kD;     // the tile of 16 rows that holds row G
+        bf16x8 bp[2];
+        bp[0] = ld16(qt + (lane & 15) * kD + (lane >> 4) * 8);
+        bp[1] = ld16(qt + (lane & 15) * kD + (lane >> 4) * 8 + 32);
+        for (int tile = wave; tile < N2 / 16; tile += kSparseWaves) {
+            f32x4 s = score_tile(pk_par + ((int64_t)bh * N2 + tile * 16) * kD, bp);
+            if ((lane & 15) == (G & 15)) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) su_par[tile * 16 + 4 * (lane >> 4) + e] = ordered_bits(rn_bf16(s[e])) & 0xFFFF0000u;
+            }
+        }
+        __syncthreads();
+        if (wave == 0)
+            wave_topk_radix_any(
+                su_par, N2, T2, [](int pos) { return pos; }, sel_u[0], sel_i[0], par, lane, 16, 32 - __builtin_clz(N2 - 1));
+        __syncthreads();
+        if (tid < T2) par_out[((int64_t)bh * N2 + G) * T2 + tid] = par[tid];
+    } else {
+        if (tid < T2) par[tid] = clampi(pidx[((int64_t)bh * N2 + G) * T2 + tid], 0, N2 - 1);
+        __syncthreads();
+    }
+    for (int i = tid; i < C; i += 64 * kSparseWaves) cand[i] = par[i / kBlk] * kBlk + (i % kBlk);
     bf16x8 bq[2];
     bq[0] = ld16(pqb + (lane & 15) * kD + (lane >> 4) * 8);
     bq[1] = ld16(pqb + (lane & 15) * kD + (lane >> 4) * 8 + 32);
@@ -330,6 +358,25 @@ extern "C" int llsa_topk_sparse(const void* pq, const void* pk, const int32_t* p
     LLSA_REQUIRE(T >= 1 && T <= kMaxT && T <= T2 * 16, "topk_sparse: need 1 <= T <= min(%d, 16*T2), got %d", kMaxT, T);
     LLSA_REQUIRE(aligned16(pq) && aligned16(pk), "topk_sparse: inputs must be 16-byte aligned");
     hipLaunchKernelGGL(topk_sparse_kernel, dim3(N1 / 16, B * H), dim3(64 * kSparseWaves), 0, (hipStream_t)stream, (const bf16*)pq,
-                       (const bf16*)pk, parent_idx, out_idx, N1, T, T2);
+                       (const bf16*)pk, parent_idx, out_idx, N1, T, T2, (const bf16*)nullptr, (const bf16*)nullptr, (int*)nullptr);
     return launch_status("topk_sparse");
+}
+
+// (a workgroup selects its parent row on one wave: beyond a few hundred parent tokens the separate dense kernel,
+// sixteen rows per workgroup side by side, is faster -- 277 vs 120 + 43 us at 1024)
+constexpr int kCascadeMaxParents = 256;
+extern "C" int llsa_topk_cascade_max_parents(void) { return kCascadeMaxParents; }
+
+extern "C" int llsa_topk_cascade(const void* pq_parent, const void* pk_parent, int32_t* parent_out, const void* pq, const void* pk,
+                                 int32_t* out_idx, int B, int H, int N1, int T, int T2, void* stream) {
+    LLSA_REQUIRE(pq_parent && pk_parent && parent_out && pq && pk && out_idx, "topk_cascade: null argument");
+    LLSA_REQUIRE(B > 0 && H > 0 && N1 > 0 && N1 % 256 == 0, "topk_cascade: N1=%d must be a positive multiple of 256", N1);
+    LLSA_REQUIRE(N1 / 16 <= kCascadeMaxParents, "topk_cascade: at most %d parent tokens (got %d): use llsa_topk_dense and llsa_topk_sparse",
+                 kCascadeMaxParents, N1 / 16);
+    LLSA_REQUIRE(T2 >= 1 && T2 * 16 <= kMaxCand && T2 <= N1 / 16, "topk_cascade: need 1 <= T2 <= min(%d, N1/16), got %d", kMaxCand / 16, T2);
+    LLSA_REQUIRE(T >= 1 && T <= kMaxT && T <= T2 * 16, "topk_cascade: need 1 <= T <= min(%d, 16*T2), got %d", kMaxT, T);
+    LLSA_REQUIRE(aligned16(pq) && aligned16(pk) && aligned16(pq_parent) && aligned16(pk_parent), "topk_cascade: inputs must be 16-byte aligned");
+    hipLaunchKernelGGL(topk_sparse_kernel, dim3(N1 / 16, B * H), dim3(64 * kSparseWaves), 0, (hipStream_t)stream, (const bf16*)pq,
+                       (const bf16*)pk, (const int*)nullptr, out_idx, N1, T, T2, (const bf16*)pq_parent, (const bf16*)pk_parent, parent_out);
+    return launch_status("topk_cascade");
 }

@@ -38,3 +38,21 @@ def compute_topk_indices_sparse(pq, pk, p_indices, topk=8, p_topk=8, block_size=
     lib.check(lib.topk_sparse(ptr(pq.contiguous()), ptr(pk.contiguous()), ptr(pi), ptr(out), B, H, M, topk, p_topk,
                               stream_of(lib, pq)), "compute_topk_indices_sparse")
     return out
+
+
+def topk_cascade(pq_parent, pk_parent, pq, pk, topk=8, p_topk=8):
+    """gen_sparse_indices on the parent level and compute_topk_indices_sparse under its result in one launch
+    (topk.py:6-9, :172-197): returns (p_indices, indices) exactly as the two calls would.  The parent level may
+    have at most llsa_topk_cascade_max_parents() tokens."""
+    lib = lib_for(pq, pk, pq_parent, pk_parent)
+    require_bf16(pq, pk, pq_parent, pk_parent)
+    require_head_dim(pq)
+    B, H, M, D = pq.shape
+    if pq_parent.shape != (B, H, M // BLOCK, D) or pk_parent.shape != pq_parent.shape or pk.shape != pq.shape:
+        raise ValueError("the parent level must be (B, H, M/16, 64) for (B, H, M, 64) rows")
+    p_topk = min(p_topk, M // BLOCK)
+    p_out = torch.empty(B, H, M // BLOCK, p_topk, device=pq.device, dtype=torch.int32)
+    out = torch.empty(B, H, M, topk, device=pq.device, dtype=torch.int32)
+    lib.check(lib.topk_cascade(ptr(pq_parent.contiguous()), ptr(pk_parent.contiguous()), ptr(p_out), ptr(pq.contiguous()),
+                               ptr(pk.contiguous()), ptr(out), B, H, M, topk, p_topk, stream_of(lib, pq)), "topk_cascade")
+    return p_out, out

@@ -200,9 +200,16 @@ class LlsaFused(Function):
 
         # Selection, coarse to fine: a dense top-k over the coarsest level's tokens (each of them is a block of the level
         # below), then level by level among the blocks under the parent's selection.
-        _check(lib, lib.topk_dense(at(lay.pq, L), at(lay.pk, L), pi(lay.sel[L - 1]), B, H, n[L], topks[L - 1], 1, stream),
-               "gen_sparse_indices")
-        for l in range(L - 1, 0, -1):
+        first = L - 1               # the first parent-guided selection still to do
+        if L >= 2 and n[L] <= lib.topk_cascade_max_parents():
+            # the dense selection rides in the workgroups of the first parent-guided one: one launch less
+            _check(lib, lib.topk_cascade(at(lay.pq, L), at(lay.pk, L), pi(lay.sel[L - 1]), at(lay.pq, L - 1), at(lay.pk, L - 1),
+                                         pi(lay.sel[L - 2]), B, H, n[L - 1], topks[L - 2], topks[L - 1], stream), "topk_cascade")
+            first = L - 2
+        else:
+            _check(lib, lib.topk_dense(at(lay.pq, L), at(lay.pk, L), pi(lay.sel[L - 1]), B, H, n[L], topks[L - 1], 1, stream),
+                   "gen_sparse_indices")
+        for l in range(first, 0, -1):
             _check(lib, lib.topk_sparse(at(lay.pq, l), at(lay.pk, l), pi(lay.sel[l]), pi(lay.sel[l - 1]), B, H, n[l], topks[l - 1],
                                         topks[l], stream), "compute_topk_indices_sparse")
 

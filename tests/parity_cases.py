@@ -192,6 +192,20 @@ def check_topk_sparse(dev, B=1, H=2, N1=256, T=8, T2=4):
     assert (idx == ref).all(-1)[o_ok].all(), "order differs on rows with well separated scores"
 
 
+def check_topk_cascade(dev, B=1, H=2, N1=1024, T=8, T2=4):
+    """The one-launch cascade gives, bit for bit, what the dense selection followed by the parent-guided one give."""
+    from llsa_amd.kernel.hip.topk import compute_topk_indices_sparse, gen_sparse_indices, topk_cascade
+    g = torch.Generator().manual_seed(17)
+    pq = torch.randn(B, H, N1, 64, generator=g).bfloat16()
+    pk = torch.randn(B, H, N1, 64, generator=g).bfloat16()
+    pq2, pk2 = O.mean_pool(pq, 16), O.mean_pool(pk, 16)
+    p_ref = gen_sparse_indices(pq2.to(dev), pk2.to(dev), T2)
+    ref = compute_topk_indices_sparse(pq.to(dev), pk.to(dev), p_ref, T, T2)
+    p_got, got = topk_cascade(pq2.to(dev), pk2.to(dev), pq.to(dev), pk.to(dev), T, T2)
+    assert torch.equal(p_got.cpu(), p_ref.cpu()), "parent selection differs from llsa_topk_dense"
+    assert torch.equal(got.cpu(), ref.cpu()), "selection differs from llsa_topk_sparse under the same parents"
+
+
 def check_transpose(dev, B=2, H=2, Mb=64, T=8, Kb=None, chunk=0):
     """chunk > 0 also asks for the work list, which with Mb*T >= 65536 entries switches the kernel to
     its split form (histogram and scatter over many workgroups)."""

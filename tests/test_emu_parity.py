@@ -46,6 +46,7 @@ def test_topk_dense_multi_chunk():
 
 def test_topk_sparse():
     P.check_topk_sparse(DEV, N1=256, T=8, T2=4)
+    P.check_topk_cascade(DEV, B=1, H=1, N1=512, T=8, T2=4)
 
 
 def test_permute():

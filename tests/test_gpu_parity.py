@@ -75,6 +75,9 @@ def test_topk_dense(dev):
 def test_topk_sparse(dev):
     P.check_topk_sparse(dev, B=2, H=3, N1=1024, T=16, T2=16)
     P.check_topk_sparse(dev, B=1, H=1, N1=256, T=8, T2=4)
+    P.check_topk_cascade(dev, B=2, H=3, N1=1024, T=16, T2=16)
+    P.check_topk_cascade(dev, B=1, H=1, N1=4096, T=16, T2=32)        # 256 parent tokens: the most the cascade takes
+    P.check_topk_cascade(dev, B=1, H=2, N1=256, T=4, T2=4)
 
 
 def test_transpose(dev):
