@@ -47,7 +47,8 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 # the table of the workload is parsed at run time, so the figure printed is the one the committed profile holds.
 TRAFFIC_KERNELS = {"attn_fwd": "attn_fwd_pair_kernel", "bwd_dq": "attn_dq_pair_kernel", "bwd_dkv": "attn_kside_kernel",
                    "bwd_pooled_groups": "attn_kside_group_kernel", "bwd_dpkv_dense": "attn_kside_dense_kernel",
-                   "pool_pyramid": "pool_pyramid_kernel", "topk_sparse": "topk_sparse_kernel", "topk_dense": "topk_dense_radix_kernel"}
+                   "pool_pyramid": "pool_pyramid_kernel", "topk_sparse": "topk_sparse_kernel", "topk_cascade": "topk_sparse_kernel",
+                   "topk_dense": "topk_dense_radix_kernel"}
 
 
 def measured_traffic(workload):
@@ -133,10 +134,16 @@ def stage_profile(op, q, k, v, do, t1, t2, freq, iters, torch):
     if l2:
         pq2, pk2, pv2 = oq["y2"], ok["y2"], ov["y2"]
         tiles.update(pk2r=ok["y2r"], pv2r=ov["y2r"], pv2t=ov["y2t"])
-        pidx = gen_sparse_indices(pq2, pk2, t2)
-        res["topk_dense"] = timed(lambda: gen_sparse_indices(pq2, pk2, t2), iters, torch)
-        idx = compute_topk_indices_sparse(pq, pk, pidx, t1, t2)
-        res["topk_sparse"] = timed(lambda: compute_topk_indices_sparse(pq, pk, pidx, t1, t2), iters, torch)
+        from llsa_amd._lib import current_lib
+        if N // 256 <= current_lib().topk_cascade_max_parents():      # what the operator launches at this size: both in one
+            from llsa_amd.kernel.hip.topk import topk_cascade
+            pidx, idx = topk_cascade(pq2, pk2, pq, pk, t1, t2)
+            res["topk_cascade"] = timed(lambda: topk_cascade(pq2, pk2, pq, pk, t1, t2), iters, torch)
+        else:
+            pidx = gen_sparse_indices(pq2, pk2, t2)
+            res["topk_dense"] = timed(lambda: gen_sparse_indices(pq2, pk2, t2), iters, torch)
+            idx = compute_topk_indices_sparse(pq, pk, pidx, t1, t2)
+            res["topk_sparse"] = timed(lambda: compute_topk_indices_sparse(pq, pk, pidx, t1, t2), iters, torch)
         kw = dict(pk2=pk2, pv2=pv2, p_indices=pidx, token_weight_2=256.0)
         cgw = 16.0
     else:
@@ -466,6 +473,7 @@ def main():
         if op == "l2":
             hbm["topk_dense"] = BH * (2 * n2 * D * 2 + n2 * t2 * 4)
             hbm["topk_sparse"] = BH * (2 * n1 * D * 2 + n2 * t2 * 4 + n1 * t1 * 4)
+            hbm["topk_cascade"] = hbm["topk_dense"] + hbm["topk_sparse"]      # (both selections in one launch)
             hbm["transpose_indices"] = BH * ((n1 * t1 * 4) * 2 + (n1 + 1) * 4 + (n2 * t2 * 4) * 3 + (n2 + 1) * 4)
         else:
             hbm["topk_dense"] = BH * (2 * n1 * D * 2 + n1 * t1 * 4)
