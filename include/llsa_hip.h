@@ -177,6 +177,7 @@ int llsa_topk_cascade_max_parents(void);
  * llsa_transpose_indices.
  * ---------------------------------------------------------------------------------------- */
 #define LLSA_MAX_LEVELS 4
+#define LLSA_POOLED_TOPK_MAX 56     /* the T of the pooled levels below the coarsest may add up to this much (forward and backward) */
 
 typedef struct llsa_fwd_level {
     const void* kr;                            /* (B,H,N/16^(l+1),1024) R tiles of the level's pooled k    */

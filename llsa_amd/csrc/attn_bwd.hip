@@ -775,6 +775,7 @@ constexpr int kGroupWaves = 4;
 constexpr int kGroupSegs = LLSA_MAX_LEVELS;
 constexpr int kGroupMaxBlocks = 64;               // key blocks per group over all its lists (their ids live in one lane each)
 constexpr int kGroupDenseMax = 8;                 // dense blocks are appended up to this many
+static_assert(LLSA_POOLED_TOPK_MAX + kGroupDenseMax <= kGroupMaxBlocks, "a group's lists must fit one lane per key block");
 
 struct GroupSeg {
     const bf16* kk; const bf16* vv;               // R tiles of this level's pooled k, v: (BH, n_units, 1024)
@@ -1086,7 +1087,7 @@ static DensePlan dense_plan(int B, int H, int N, int levels) {
     // Q and dO are streamed n_units / (4 * upw) times (mostly out of an L2: see the kernel); four units per wave would
     // halve that again but leave one wave per SIMD, which measured slower (1.07 ms against 0.93 ms at N = 262144)
     d.upw = (n_units % 8 == 0 && n_units >= 16) ? 2 : 1;
-    const int groups = (n_units / (kDenseWaves * d.upw)) * B * H;   // workgroups per piece of the query range
+    const int groups = max(1, n_units / (kDenseWaves * d.upw)) * B * H;   // workgroups per piece of the query range
     // The query range is cut so that the workgroups fill the chip's resident slots (256 CUs x the workgroups the
     // registers allow per CU) a whole number of times, three if there is that much work: a count just above a
     // multiple of the slots leaves a last round in which a few workgroups run alone.
@@ -1143,7 +1144,8 @@ static BwdWorkspace bwd_workspace(int B, int H, int N, const int32_t* topk, int 
 using namespace llsa;
 
 extern "C" int64_t llsa_attn_bwd_workspace_bytes(int B, int H, int N, const int32_t* topk, int levels) {
-    if (B <= 0 || H <= 0 || N <= 0 || N % 16 != 0 || topk == nullptr || levels < 1 || levels > LLSA_MAX_LEVELS) return -1;
+    if (B <= 0 || H <= 0 || N <= 0 || topk == nullptr || levels < 1 || levels > LLSA_MAX_LEVELS) return -1;
+    if (N % coarsest_multiple(levels) != 0) return -1;       // what llsa_attn_bwd asks of N: whole 64-token tiles of the coarsest level
     for (int l = 0; l < levels; l++)
         if (topk[l] <= 0) return -1;
     return bwd_workspace(B, H, N, topk, levels).total;
@@ -1175,8 +1177,8 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
             listed += lv.T;
         }
     }
-    LLSA_REQUIRE(listed + kGroupDenseMax <= kGroupMaxBlocks, "attn_bwd: the topk of the pooled levels together (%d) must not exceed %d", listed,
-                 kGroupMaxBlocks - kGroupDenseMax);
+    LLSA_REQUIRE(listed <= LLSA_POOLED_TOPK_MAX, "attn_bwd: the topk of the pooled levels together (%d) must not exceed %d", listed,
+                 LLSA_POOLED_TOPK_MAX);
     const void* al[] = {a->dout, a->o, a->qr, a->kr, a->vr, a->dq, a->dk, a->dv, a->workspace, a->freq_dq, a->lse};
     for (const void* p : al) LLSA_REQUIRE(aligned16(p), "attn_bwd: tensors must be 16-byte aligned");
     const int64_t st[] = {a->sdob, a->sdoh, a->sdon, a->sob, a->soh, a->son};

@@ -433,7 +433,8 @@ extern "C" int llsa_attn_fwd(const llsa_attn_fwd_args* a, void* stream) {
             listed += lv.T;
         }
     }
-    LLSA_REQUIRE(listed <= 64, "attn_fwd: the topk of the pooled levels together (%d) must not exceed 64", listed);
+    LLSA_REQUIRE(listed <= LLSA_POOLED_TOPK_MAX, "attn_fwd: the topk of the pooled levels together (%d) must not exceed %d", listed,
+                 LLSA_POOLED_TOPK_MAX);
     LLSA_REQUIRE(aligned16(a->qr) && aligned16(a->kr) && aligned16(a->vt) && aligned16(a->o), "attn_fwd: tensors must be 16-byte aligned");
     LLSA_REQUIRE((a->sob % 4 == 0) && (a->soh % 4 == 0) && (a->son % 4 == 0), "attn_fwd: rows of o must be 8-byte aligned");
     const int N1 = a->N / 16;

@@ -4,10 +4,13 @@ on the CPU through the x86 emulation build of the same sources (tests/test_emu_p
 
 Tolerances (bf16): outputs and gradients must satisfy
     rel-L2 error      <= 1e-2
-    max-abs error     <= 2e-2             for every element whose reference value is below 2 in magnitude
-                      <= 2e-2 * |ref|     for the others (one bf16 ulp is 1.6e-2 in [2, 4), 3.1e-2 in [4, 8): a flat
-                                          2e-2 is below the resolution of the output format there)
-Integer results (pool bit patterns, indices on tie-free rows, CSR) must be identical.
+    max-abs error     <= 2e-2             flat, on the benchmark configurations and in the smoke test (FLAT = True below:
+                                          every check of the whole operator on the smooth-field inputs)
+                      <= 2e-2             for every element whose reference value is below 2 in magnitude, and
+                      <= 2e-2 * |ref|     for the others, on the random stress shapes only (N(0,1) inputs scaled up, hot
+                                          blocks: one bf16 ulp is 1.6e-2 in [2, 4), 3.1e-2 in [4, 8), so a flat 2e-2 is
+                                          below the resolution of the output format there)
+Integer results (pool bit patterns, indices on rows the rounding cannot decide otherwise, CSR) must be identical.
 """
 import math
 
@@ -20,13 +23,16 @@ MAX_ABS = 2e-2
 MEASURED = {}        # name of the last check -> {tensor: (rel-L2, max-abs)}, for reports
 
 
-def close(name, got, ref, rel=REL_L2, mabs=MAX_ABS, report=None):
+def close(name, got, ref, rel=REL_L2, mabs=MAX_ABS, report=None, flat=False):
+    """flat=True: max-abs <= mabs on every element, whatever its magnitude (the bound the target states)."""
     g, r = got.detach().double().cpu(), ref.detach().double().cpu()
     assert g.shape == r.shape, f"{name}: shape {tuple(g.shape)} vs {tuple(r.shape)}"
     assert torch.isfinite(g).all(), f"{name}: non-finite values"
     err = (g - r).abs()
     e_rel = ((g - r).norm() / r.norm().clamp_min(1e-30)).item()
     e_abs = err.max().item()
+    if flat:
+        assert e_abs <= mabs, f"{name}: max-abs {e_abs:.3e} (<= {mabs}, flat)"
     bound = torch.where(r.abs() < 2.0, torch.full_like(r, mabs), mabs * r.abs())
     worst = (err - bound).max().item()
     assert e_rel <= rel, f"{name}: rel-L2 {e_rel:.3e} (<= {rel})"
@@ -136,6 +142,37 @@ def _safe_rows(score, T, eps_rel):
     return boundary_ok, ordered_ok
 
 
+def decided_rows_dense(pq, pk, T):
+    """Rows of the bf16-rounded dense selection whose top-T SET cannot depend on how the fp32 dot products were
+    summed.  Device and oracle round the same 64-term dot product to bf16 (topk.py:7), added in different orders:
+    the two fp32 values differ by a few ulps, and the rounded values differ only where the fp32 value sits that close
+    to the midpoint of two neighbouring bf16 numbers.  With delta = 2^-20 * sum_c |pq_c pk_c| (a bound on the
+    summation error with a wide margin: 64 terms, eps = 2^-24), every score has a lowest and a highest possible
+    rounded value, lo = bf16(s - delta) and hi = bf16(s + delta) (equal for an unambiguous score).  A row is decided
+    when every ambiguous member of the oracle's top-T stays strictly above whatever any outsider can reach and
+    every ambiguous outsider stays strictly below whatever any member can fall to; the unambiguous scores have the
+    same bits on both sides, and so the same ranking with the same tie rule (smaller index first).  Returns
+    (decided (.., n) bool, ordered (.., n) bool: no ambiguous score anywhere among the best T + 1, so that the order
+    of the T indices is decided too)."""
+    s = pq.float() @ pk.float().transpose(-1, -2)
+    mag = pq.float().abs() @ pk.float().abs().transpose(-1, -2)
+    delta = mag * 2.0 ** -20
+    lo, hi = (s - delta).bfloat16().float(), (s + delta).bfloat16().float()
+    amb = lo != hi
+    ref = O.topk_lowest_index(s.bfloat16(), T)
+    member = torch.zeros_like(amb).scatter_(-1, ref, True)
+    inf = torch.full_like(s, float("inf"))
+    min_in_lo = torch.where(member, lo, inf).amin(-1, keepdim=True)
+    max_out_hi = torch.where(member, -inf, hi).amax(-1, keepdim=True)
+    bad = amb & ((member & (lo <= max_out_hi)) | (~member & (hi >= min_in_lo)))
+    decided = ~bad.any(-1)
+    # order: the best T + 1 (by the rounded score) and everything that could tie with them must be unambiguous
+    n = s.shape[-1]
+    kth1 = torch.sort(s.bfloat16().float(), -1, descending=True).values[..., min(T, n - 1):min(T, n - 1) + 1]
+    ordered = decided & ~(amb & (hi >= kth1)).any(-1)
+    return decided, ordered
+
+
 def check_topk_dense(dev, B=1, H=2, n=64, T=8, round_scores=True, min_safe=0.3):
     from llsa_amd.kernel.hip.topk import gen_sparse_indices
     g = torch.Generator().manual_seed(9)
@@ -146,9 +183,12 @@ def check_topk_dense(dev, B=1, H=2, n=64, T=8, round_scores=True, min_safe=0.3):
     assert (idx.sort(-1).values.diff(dim=-1) > 0).all(), "duplicate index in a row"
     exact = O.dense_scores(pq, pk, round_to_input=False)
     ref = O.topk_lowest_index(O.dense_scores(pq, pk, round_to_input=round_scores), T)
-    # one bf16 ulp is 2^-8 relative: demand 2^-6 of separation on the unrounded scores
-    b_ok, o_ok = _safe_rows(exact, T, 2.0 ** -6 if round_scores else 1e-4)
-    assert b_ok.float().mean() >= min_safe, f"test input has too few tie-free rows ({b_ok.float().mean():.2f})"
+    if round_scores:
+        b_ok, o_ok = decided_rows_dense(pq, pk, T)
+        min_safe = max(min_safe, 0.85)
+    else:
+        b_ok, o_ok = _safe_rows(exact, T, 1e-4)
+    assert b_ok.float().mean() >= min_safe, f"test input has too few decided rows ({b_ok.float().mean():.2f})"
     same_set = (idx.sort(-1).values == ref.sort(-1).values).all(-1)
     assert same_set[b_ok].all(), "selected set differs on tie-free rows"
     assert (idx == ref).all(-1)[o_ok].all(), "order differs on rows with well separated scores"
@@ -373,15 +413,14 @@ def check_constant_v(dev, N=1024):
 # ------------------------------------------------------------------------------------------
 def selection_dense_vs_oracle(what, pq, pk, got, T, strict=True):
     """The device's coarsest selection `got` (.., n, T) against the oracle's own: torch.matmul's bf16-rounded
-    scores (topk.py:6-9) ranked with ties to the smaller index.  Index sets must be identical on every row whose
-    T-th and (T+1)-th unrounded scores are further apart than 2^-6 relative (a bf16 ulp is 2^-8), and everywhere
-    the selection must be a legal top-k of the rounded scores.  Returns (fraction of rows with identical sets,
-    fraction of rows that pass the gap criterion)."""
+    scores (topk.py:6-9) ranked with ties to the smaller index.  Index sets must be identical on every row that
+    the summation order of the dot products cannot decide otherwise (decided_rows_dense: exact ties included, they
+    go to the smaller index on both sides), and everywhere the selection must be a legal top-k of the rounded
+    scores.  Returns (fraction of rows with identical sets, fraction of rows under the strict check)."""
     got = got.long()
-    exact = O.dense_scores(pq, pk, round_to_input=False)
     rounded = O.dense_scores(pq, pk)
     ref = O.topk_lowest_index(rounded, T)
-    b_ok, _ = _safe_rows(exact, T, 2.0 ** -6)
+    b_ok, _ = decided_rows_dense(pq, pk, T)
     same = (got.sort(-1).values == ref.sort(-1).values).all(-1)
     assert (got.sort(-1).values.diff(dim=-1) > 0).all(), f"{what}: duplicate index in a row"
     if strict:
@@ -519,7 +558,7 @@ def check_op_l1(dev, B=1, H=2, N=1024, T=8, fused=True, rope=False, strided=Fals
     rq, rk = _norm_backward(rq, rk, qc, kc, norm)
     tag = f"l1 B={B} H={H} N={N} T={T}" + (" rope" if rope else "") + (" qk_norm" if qk_norm else "") + ("" if fused else " unfused")
     for name, a, b in (("o", o, ro), ("dq", dq, rq), ("dk", dk, rk), ("dv", dv, rv)):
-        close(name, a, b, report=tag)
+        close(name, a, b, report=tag, flat=smooth)
     # the selection against the oracle's own (the oracle pooled the same rows: ctx) -- identical index sets on
     # tie-free rows, a legal top-k everywhere
     MEASURED[tag]["selection (same, tie-free)"] = selection_dense_vs_oracle("indices", ctx["pq"], ctx["pk"], idx, T, strict=not qk_norm)
@@ -552,13 +591,14 @@ def check_op_l2(dev, B=1, H=1, N=16384, T=8, T2=4, fused=True, rope=False, smoot
         for b, h in slices:
             cut = lambda t: t[b:b + 1, h:h + 1]
             _compare_op_l2(f"l2 B={B} H={H} N={N} T={T}/{T2} slice ({b},{h})", *(cut(t) for t in (q, k, v, do, o, dq, dk, dv)),
-                           cut(captured["idx"]), cut(captured["pidx"]), T, T2, freq, norm)
+                           cut(captured["idx"]), cut(captured["pidx"]), T, T2, freq, norm, flat=smooth)
         return
     _compare_op_l2(f"l2 B={B} H={H} N={N} T={T}/{T2}" + (" rope" if rope else "") + (" qk_norm" if qk_norm else "")
-                   + ("" if fused else " unfused"), q, k, v, do, o, dq, dk, dv, captured["idx"], captured["pidx"], T, T2, freq, norm)
+                   + ("" if fused else " unfused"), q, k, v, do, o, dq, dk, dv, captured["idx"], captured["pidx"], T, T2, freq, norm,
+                   flat=smooth)
 
 
-def _compare_op_l2(tag, q, k, v, do, o, dq, dk, dv, dev_idx, dev_pidx, T, T2, freq, norm):
+def _compare_op_l2(tag, q, k, v, do, o, dq, dk, dv, dev_idx, dev_pidx, T, T2, freq, norm, flat=False):
     rope, qk_norm = freq is not None, norm is not None
     qc, kc, vc, doc = (t.cpu().contiguous() for t in (q, k, v, do))
     fc = freq.cpu() if rope else None
@@ -570,7 +610,7 @@ def _compare_op_l2(tag, q, k, v, do, o, dq, dk, dv, dev_idx, dev_pidx, T, T2, fr
         rq, rk = O.rope_apply_bwd(rq, fc), O.rope_apply_bwd(rk, fc)
     rq, rk = _norm_backward(rq, rk, qc, kc, norm)
     for name, a, b in (("o", o, ro), ("dq", dq, rq), ("dk", dk, rk), ("dv", dv, rv)):
-        close(name, a, b, report=tag)
+        close(name, a, b, report=tag, flat=flat)
     # both levels of the selection against the oracle's own: the coarse one on the level-2 pooled rows, the fine
     # one under the parents the device chose (wherever those equal the oracle's this is the whole cascade)
     pidx, idx = dev_pidx.cpu().long(), dev_idx.cpu().long()
@@ -611,10 +651,10 @@ def check_op_l3(dev, B=1, H=1, N=262144, T=16, T2=16, T3=16, rope=True, qk_norm=
     if rope:
         rq, rk = O.rope_apply_bwd(rq, fc), O.rope_apply_bwd(rk, fc)
     rq, rk = _norm_backward(rq, rk, qc, kc, norm)
-    close("o", o, ro)
-    close("dq", dq, rq)
-    close("dk", dk, rk)
-    close("dv", dv, rv)
+    close("o", o, ro, flat=True)
+    close("dq", dq, rq, flat=True)
+    close("dk", dk, rk, flat=True)
+    close("dv", dv, rv, flat=True)
     _, own = O.llsa_l3_fwd(qr, kr, vc, T, T2, T3, 16)
     same = lambda a, b: (a.sort(-1).values == b.long().sort(-1).values).all(-1).float().mean().item()
     assert same(ppidx, own["pp_indices"]) > 0.9 and same(pidx, own["p_indices"]) > 0.9 and same(idx, own["indices"]) > 0.9

@@ -75,6 +75,17 @@ def test_entry_points_reject_bad_arguments(lib):
     assert lib.attn_bwd_workspace_bytes(2, 6, 16384, topk(16, 16), 2) > 0
     assert lib.attn_bwd_workspace_bytes(1, 1, 262144, topk(16, 16, 16), 3) > lib.attn_bwd_workspace_bytes(1, 1, 262144, topk(16, 16), 2) > 0
     assert lib.attn_bwd_workspace_bytes(2, 6, 16384, topk(16, 16, 16, 16, 16), 5) < 0
+    # a token count the coarsest level cannot tile is an error, not a division by zero in the work split
+    assert lib.attn_bwd_workspace_bytes(1, 1, 512, topk(8), 1) < 0
+    assert lib.attn_bwd_workspace_bytes(1, 1, 4096, topk(8, 8), 2) < 0
+    assert lib.attn_bwd_workspace_bytes(1, 1, 1024, topk(8), 1) > 0
+    a.levels, a.N, a.T = 3, 262144, 8                   # forward and backward share the limit on the pooled levels' topk
+    for l in range(3):
+        a.lvl[l].kr = a.lvl[l].vt = a.lvl[l].sel = 16
+        a.lvl[l].w = 16.0
+    a.lvl[0].T = a.lvl[1].T = 32
+    assert lib.attn_fwd(C.byref(a), None) != 0
+    assert b"must not exceed 56" in lib.last_error_string()
     assert lib.work_list_len(1024, 1024, 16, 32) == 4 + 4 * (512 + 1024) + 4 * 513 + 1024
 
 

@@ -181,6 +181,40 @@ def test_full_dit_s_step_against_oracle_ops_gpu(monkeypatch):
 
 
 @pytest.mark.gpu
+def test_full_dit_s_at_batch_8_equals_its_quarters():
+    """The training-step configuration at its batch size (8 images of 3 x 128 x 128, 12 layers, 6 heads, llsa_l2 topk
+    16/16): samples do not interact (the operator has one grid axis over B x H, layer norms and the qk norm are per
+    token), so the loss of the batch is the mean of the losses of its four quarters of two run on their own, and
+    every parameter gradient the mean of theirs; everything must be finite."""
+    torch.manual_seed(5)
+    dev = torch.device("cuda:0")
+    model = D.PixelDiT(num_attention_heads=6, num_layers=12, sample_size=128, levels=2, sparse_topk=16).to(dev)
+    batch = [x.to(dev) for x in _batch(8, 128, seed=6)]
+    loss8, grads8 = _loss_and_grads(model, batch, dev)
+    assert loss8 == loss8 and all(torch.isfinite(g).all() for g in grads8.values())
+    parts = []
+    for i in range(0, 8, 2):
+        model.zero_grad(set_to_none=True)
+        parts.append(_loss_and_grads(model, [x[i:i + 2] for x in batch], dev))
+    mean_loss = sum(l for l, _ in parts) / 4
+    assert abs(loss8 - mean_loss) <= 2e-3 * abs(mean_loss), (loss8, mean_loss)
+    worst, worst_sel = ("", 0.0), ("", 0.0)
+    for n, g in grads8.items():
+        r = sum(gr[n] for _, gr in parts) / 4
+        err = ((g - r).norm() / r.norm().clamp_min(1e-12)).item()
+        # parameters that act only through the attention scores also see which near-tied blocks were selected, and a
+        # GEMM over 8 x 16384 rows may round q and k differently from one over 2 x 16384 rows
+        if any(t in n for t in ("to_q.", "to_k.", "norm_q_weight", "norm_k_weight")):
+            worst_sel = max(worst_sel, (n, err), key=lambda x: x[1])
+        else:
+            worst = max(worst, (n, err), key=lambda x: x[1])
+    print(f"batch 8 vs quarters: loss {loss8:.6f} / {mean_loss:.6f}, worst gradient {worst}, through the scores {worst_sel}")
+    # (bf16 GEMMs over 8 x 16384 rows against 4 times 2 x 16384: the weight gradients are summed in another order)
+    assert worst[1] <= 2e-2, f"gradient of {worst[0]} differs from the mean over the quarters by rel-L2 {worst[1]:.3e}"
+    assert worst_sel[1] <= 0.2, f"gradient of {worst_sel[0]} differs from the mean over the quarters by rel-L2 {worst_sel[1]:.3e}"
+
+
+@pytest.mark.gpu
 def test_training_reduces_the_loss():
     torch.manual_seed(0)
     dev = torch.device("cuda:0")
