@@ -782,7 +782,11 @@ struct GroupSeg {
     const int* sel;                               // (BH, n_groups >> owner_shift, cnt) blocks selected by the group's ancestor;
                                                   // nullptr: blocks 0..cnt-1 (dense level)
     const int* inv;                               // (BH, n_groups >> owner_shift, cnt) position of each entry in the transposed selection
-    f32x4* part;                                  // partial sums
+    bf16x4* part;                                 // partial sums, in the accumulator layout of part_slot but rounded to bf16: the
+                                                  // group-major pass writes one per (group, key block), 8 KB each in fp32, which at
+                                                  // 16384 tokens is more memory traffic than everything else the pass moves; a group's
+                                                  // sum over its 256 queries is taken in fp32 and rounded once (2^-9 relative), and the
+                                                  // reduction adds the rounded sums of a key block's groups in fp32
     int n_units, owner_shift, cnt;
     int64_t slots;                                // partial slots per (b,h) (sparse) -- positions are clamped into them
     float w;
@@ -798,7 +802,7 @@ struct GroupStats { f32x4 l[2], d[2]; };
 
 // UPW key blocks against the group's 16 query blocks, two query blocks per step, operands out of LDS.
 template <int UPW>
-__device__ __forceinline__ void group_pass(const bf16x8 (&bk)[2][2], const bf16x8 (&bv)[2][2], const float (&w)[2], f32x4* const (&dst)[2],
+__device__ __forceinline__ void group_pass(const bf16x8 (&bk)[2][2], const bf16x8 (&bv)[2][2], const float (&w)[2], bf16x4* const (&dst)[2],
                                            const bf16* shq, const bf16* shg, const float* lseb, const float* dlb, int lane) {
     const int quad = lane >> 4;
     f32x4 dk[UPW][4], dv[UPW][4];
@@ -871,12 +875,14 @@ __device__ __forceinline__ void group_pass(const bf16x8 (&bk)[2][2], const bf16x
         load_stats((t + 2) & (kBlk / 2 - 1), sa);             // (the last one re-reads step 0: no branch around loads)
         step(t + 1, sb);
     }
+    // The partial sums of this pass leave as bf16 (see GroupSeg::part): the sum over the group's 256 queries was
+    // taken in fp32, and the result the reduction makes of them is a bf16 tensor.
 #pragma unroll
     for (int j = 0; j < UPW; j++)
 #pragma unroll
         for (int dt = 0; dt < 4; dt++) {
-            dst[j][dt * kWave + lane] = dk[j][dt] * w[j];
-            dst[j][(4 + dt) * kWave + lane] = dv[j][dt] * w[j];
+            dst[j][dt * kWave + lane] = cvt4(dk[j][dt] * w[j]);
+            dst[j][(4 + dt) * kWave + lane] = cvt4(dv[j][dt] * w[j]);
         }
 }
 
@@ -932,7 +938,7 @@ __global__ __launch_bounds__(64 * kGroupWaves, 2) void attn_kside_group_kernel(G
 
     bf16x8 bk[2][2], bv[2][2];
     float w[2];
-    f32x4* dst[2];
+    bf16x4* dst[2];
     auto fetch = [&](int j, int u) __attribute__((always_inline)) {    // K, V tiles of key block j into register set u
         const int sgi = __builtin_amdgcn_readlane(my_seg, j);
         const int unit = __builtin_amdgcn_readlane(my_unit, j);
@@ -945,7 +951,7 @@ __global__ __launch_bounds__(64 * kGroupWaves, 2) void attn_kside_group_kernel(G
         bv[u][0] = ld16(vp);
         bv[u][1] = ld16(vp + 512);
         w[u] = sg.w;
-        dst[u] = part_slot(sg.part, ((int64_t)(unsigned)slo) | ((int64_t)shi << 32));
+        dst[u] = sg.part + (((int64_t)(unsigned)slo) | ((int64_t)shi << 32)) * (8 * kWave);
     };
     if (lo < hi) fetch(lo, 0);
     if (lo + 1 < hi) fetch(lo + 1, 1);
@@ -966,7 +972,8 @@ __global__ __launch_bounds__(64 * kGroupWaves, 2) void attn_kside_group_kernel(G
 // unit's partial slots, added in chunk order, so it does not depend on scheduling.  One launch
 // serves the three K-side passes.
 struct ReduceJob {
-    const f32x4* part;
+    const f32x4* part;       // fp32 partial sums, or, with half_part, the bf16 ones of the group-major pass (as bf16x4)
+    int half_part;
     const int* off;          // CSR offsets (list-driven jobs) or nullptr (dense job)
     const int* work;         // work list (fine job); nullptr with `off`: the partial sums of unit u are slots
                              // [off[u] << csr_shift, off[u + 1] << csr_shift) (group-major pooled jobs)
@@ -1052,14 +1059,27 @@ __global__ __launch_bounds__(256) void kside_reduce_kernel(ReduceParams rp) {
             stride = (int64_t)gridDim.y * jb.n_units;
         }
         f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-        const f32x4* ps = jb.part + first * (8 * kWave) + reg * kWave + lane;
-        for (int c0 = 0; c0 < n; c0 += 16) {
-            f32x4 v[16];
+        const int64_t at = first * (8 * kWave) + reg * kWave + lane;
+        if (jb.half_part) {
+            const bf16x4* ps = reinterpret_cast<const bf16x4*>(jb.part) + at;
+            for (int c0 = 0; c0 < n; c0 += 16) {
+                bf16x4 v[16];
 #pragma unroll
-            for (int k = 0; k < 16; k++) v[k] = ps[(int64_t)min(c0 + k, n - 1) * stride * (8 * kWave)];
+                for (int k = 0; k < 16; k++) v[k] = ps[(int64_t)min(c0 + k, n - 1) * stride * (8 * kWave)];
 #pragma unroll
-            for (int k = 0; k < 16; k++)
-                if (c0 + k < n) acc += v[k];                   // chunk order: the sum does not depend on scheduling
+                for (int k = 0; k < 16; k++)
+                    if (c0 + k < n) acc += f32x4{(float)v[k][0], (float)v[k][1], (float)v[k][2], (float)v[k][3]};
+            }
+        } else {
+            const f32x4* ps = jb.part + at;
+            for (int c0 = 0; c0 < n; c0 += 16) {
+                f32x4 v[16];
+#pragma unroll
+                for (int k = 0; k < 16; k++) v[k] = ps[(int64_t)min(c0 + k, n - 1) * stride * (8 * kWave)];
+#pragma unroll
+                for (int k = 0; k < 16; k++)
+                    if (c0 + k < n) acc += v[k];               // chunk order: the sum does not depend on scheduling
+            }
         }
         bf16x4 out = cvt4(which ? acc : acc * kScale);
         if (jb.fold.depth > 0)
@@ -1216,7 +1236,7 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     no_fold.depth = 0;
     auto add_job = [&](const KSideParams& p, int chunk, int max_units, int n_chunks) {
         ReduceJob& j = rp.job[rp.n_jobs++];
-        j.part = p.part; j.off = p.off; j.work = p.work; j.csr_shift = 0;
+        j.part = p.part; j.half_part = 0; j.off = p.off; j.work = p.work; j.csr_shift = 0;
         j.dk = p.dk; j.sdkb = p.sdkb; j.sdkh = p.sdkh; j.sdkn = p.sdkn;
         j.dv = p.dv; j.sdvb = p.sdvb; j.sdvh = p.sdvh; j.sdvn = p.sdvn;
         j.n_units = p.n_units; j.chunk = chunk; j.max_units = max_units;
@@ -1275,7 +1295,7 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
                            int cnt, int64_t slots, float w) {
             GroupSeg& sgm = g.seg[g.n_segs++];
             sgm.kk = (const bf16*)kk; sgm.vv = (const bf16*)vv; sgm.sel = sel; sgm.inv = inv;
-            sgm.part = (f32x4*)(ws + part_off); sgm.n_units = n_units; sgm.owner_shift = shift; sgm.cnt = cnt; sgm.slots = slots; sgm.w = w;
+            sgm.part = (bf16x4*)(ws + part_off); sgm.n_units = n_units; sgm.owner_shift = shift; sgm.cnt = cnt; sgm.slots = slots; sgm.w = w;
             g.n_blocks += cnt;
         };
         for (int l = 1; l < L; l++) {                         // level l: blocks N / 16^(l+1), one list per 16^(l-1) groups
@@ -1289,7 +1309,7 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
             const GroupSeg& sgm = g.seg[l - 1];
             const int64_t n = level_tokens(l);
             ReduceJob& j = rp.job[rp.n_jobs++];
-            j.part = sgm.part; j.off = a->lvl[l - 1].off; j.work = nullptr; j.csr_shift = sgm.owner_shift;
+            j.part = (const f32x4*)sgm.part; j.half_part = 1; j.off = a->lvl[l - 1].off; j.work = nullptr; j.csr_shift = sgm.owner_shift;
             j.dk = (bf16*)a->lvl[l - 1].dk; j.sdkb = (int64_t)H * n * 64; j.sdkh = n * 64; j.sdkn = 64;
             j.dv = (bf16*)a->lvl[l - 1].dv; j.sdvb = (int64_t)H * n * 64; j.sdvh = n * 64; j.sdvn = 64;
             j.n_units = sgm.n_units; j.chunk = 1; j.max_units = sgm.n_units;
@@ -1313,6 +1333,7 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
         p.n_units = d.n_tok / 16; p.chunk_len = d.chunk_len;
         if (d.merged) {                                       // the group-major pass has written one partial sum per group
             add_job(p, 1, p.n_units, d.chunks);
+            rp.job[rp.n_jobs - 1].half_part = 1;
             return;
         }
         const dim3 grid(p.n_units / (kDenseWaves * d.upw) * d.chunks, BH), block(64 * kDenseWaves);
