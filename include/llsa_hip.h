@@ -44,7 +44,7 @@ extern "C" {
 #define LLSA_DTYPE_BF16 0
 #define LLSA_DTYPE_F32 1
 
-#define LLSA_ABI_VERSION 201     /* changes with every change of a signature or argument structure below */
+#define LLSA_ABI_VERSION 202     /* changes with every change of a signature or argument structure below */
 int llsa_version(void);          /* LLSA_ABI_VERSION of the built library                                    */
 const char* llsa_last_error_string(void);
 
@@ -219,6 +219,17 @@ int llsa_attn_fwd(const llsa_attn_fwd_args* a, void* stream);
  * ---------------------------------------------------------------------------------------- */
 int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, int32_t* work /* or NULL */,
                            int32_t* inv /* or NULL */, int B, int H, int Mb, int Kb, int T, int chunk, void* stream);
+
+/* The same for several index tensors of one operator call (the selections of all its levels) with as few launches as
+ * possible: every job is what one llsa_transpose_indices call takes, all jobs share B and H.  Jobs small enough
+ * for one workgroup per (b,h) to hold a bitmap of (key block, query block) in LDS -- roughly Mb * Kb <= 2^20 --
+ * are done in ONE launch together, already sorted; the others go job by job.  It has no counterpart of its own in
+ * the reference, which calls transpose_indices once per index tensor (sparse_attention_res_2.py:593-594). */
+typedef struct llsa_transpose_job {
+    const int32_t* idx; int32_t* offsets; int32_t* flat; int32_t* work /* or NULL */; int32_t* inv /* or NULL */;
+    int32_t Mb, Kb, T, chunk;
+} llsa_transpose_job;
+int llsa_transpose_indices_multi(const llsa_transpose_job* jobs, int n_jobs, int B, int H, void* stream);
 
 /* Work list for the K-side backward kernels, written by llsa_transpose_indices when `work` is
  * given: every key block's segment is cut into chunks of at most `chunk` entries, one work item

@@ -65,6 +65,12 @@ class AttnBwdArgs(C.Structure):
 
 P64 = C.POINTER(c_int64)
 
+
+class TransposeJob(C.Structure):
+    _fields_ = [("idx", c_void_p), ("offsets", c_void_p), ("flat", c_void_p), ("work", c_void_p), ("inv", c_void_p),
+                ("Mb", c_int32), ("Kb", c_int32), ("T", c_int32), ("chunk", c_int32)]
+
+
 _SIGNATURES = {
     "llsa_version": (c_int, []),
     "llsa_last_error_string": (C.c_char_p, []),
@@ -86,6 +92,7 @@ _SIGNATURES = {
     "llsa_topk_cascade_max_parents": (c_int, []),
     "llsa_attn_fwd": (c_int, [C.POINTER(AttnFwdArgs), c_void_p]),
     "llsa_transpose_indices": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "llsa_transpose_indices_multi": (c_int, [C.POINTER(TransposeJob), c_int, c_int, c_int, c_void_p]),
     "llsa_work_list_len": (c_int64, [c_int, c_int, c_int, c_int]),
     "llsa_attn_bwd_workspace_bytes": (c_int64, [c_int, c_int, c_int, C.POINTER(c_int32), c_int]),
     "llsa_attn_bwd": (c_int, [C.POINTER(AttnBwdArgs), c_void_p]),
@@ -93,7 +100,7 @@ _SIGNATURES = {
 
 EXPORTS = tuple(_SIGNATURES)
 CHUNK_FINE = 64                                             # LLSA_CHUNK_FINE of include/llsa_hip.h
-ABI_VERSION = 201                                           # LLSA_ABI_VERSION
+ABI_VERSION = 202                                           # LLSA_ABI_VERSION
 STATIC_PARTIALS_MAX = 262144                                # LLSA_STATIC_PARTIALS_MAX
 
 

@@ -50,7 +50,7 @@ __device__ __forceinline__ bf16x8 rope_chunk_bwd(bf16x8 g, bf16x8 f) {
 struct PoolParams {
     llsa_pool_item it[4];
     const bf16* freq;
-    int H;
+    int H, n_items;
 };
 
 // The operand tiles of the workgroup's 16 blocks are one contiguous 32 KB piece of the tile
@@ -99,14 +99,17 @@ __device__ __forceinline__ void rms_norm_rows(bf16x8 xv[16], const float* gamma,
 template <bool NORM>
 __global__ __launch_bounds__(128) void pool_pyramid_kernel(PoolParams p) {
     __shared__ __align__(16) bf16 stage[16 * 128 * 8];
-    const llsa_pool_item& it = p.it[blockIdx.z];
+    // (items interleaved along x: q and k with their rotation are arithmetic-heavy, v with its two tiles is store-heavy,
+    // and workgroups start in x order -- a launch that runs one item after the other works in phases)
+    const int item = (int)blockIdx.x % p.n_items, bx = (int)blockIdx.x / p.n_items;
+    const llsa_pool_item& it = p.it[item];
     const int n1 = it.n / kBlk;
-    if ((int)blockIdx.x * 16 >= n1) return;       // uniform over the workgroup
+    if (bx * 16 >= n1) return;                    // uniform over the workgroup
     const int bh = blockIdx.y, b = bh / p.H, h = bh % p.H;
     const int t = threadIdx.x, c = t & 7, r = t >> 3;
-    const int blk = blockIdx.x * 16 + r;
+    const int blk = bx * 16 + r;
     const bool valid = blk < n1;
-    const int n_valid = min(16, n1 - (int)blockIdx.x * 16);
+    const int n_valid = min(16, n1 - bx * 16);
 
     bf16x8 xv[16];
     bf16x8 y = zero8();
@@ -143,7 +146,7 @@ __global__ __launch_bounds__(128) void pool_pyramid_kernel(PoolParams p) {
 #pragma unroll
             for (int i = 0; i < 16; i++) st16(stage + (r * 128 + swz_r(c * 16 + i, r)) * 8, xv[i]);
         }
-        stage_out(stage, (bf16*)it.xr + ((int64_t)bh * n1 + blockIdx.x * 16) * kTile, t, n_valid, true);
+        stage_out(stage, (bf16*)it.xr + ((int64_t)bh * n1 + bx * 16) * kTile, t, n_valid, true);
     }
     if (it.xt != nullptr) {              // T tile: channels 8c+e, 8c+e+1 of tokens 4q..4q+3 are one 16-byte unit
         if (valid) {
@@ -161,7 +164,7 @@ __global__ __launch_bounds__(128) void pool_pyramid_kernel(PoolParams p) {
                     st16(stage + (r * 128 + swz_t(u)) * 8, v);
                 }
         }
-        stage_out(stage, (bf16*)it.xt + ((int64_t)bh * n1 + blockIdx.x * 16) * kTile, t, n_valid, false);
+        stage_out(stage, (bf16*)it.xt + ((int64_t)bh * n1 + bx * 16) * kTile, t, n_valid, false);
     }
     if (it.y2 == nullptr && it.y1r == nullptr && it.y1t == nullptr && it.y2r == nullptr && it.y2t == nullptr) return;   // uniform over the workgroup
 
@@ -182,11 +185,11 @@ __global__ __launch_bounds__(128) void pool_pyramid_kernel(PoolParams p) {
         bf16x8 y2;
 #pragma unroll
         for (int e = 0; e < 8; e++) y2[e] = (bf16)(acc[e] * 0.0625f);
-        if (it.y2 != nullptr) st16((bf16*)it.y2 + ((int64_t)bh * n2 + blockIdx.x) * kD + t * 8, y2);
-        // this workgroup's level-2 row is row blockIdx.x % 16 of level-2 block blockIdx.x / 16: its 8-channel chunk
+        if (it.y2 != nullptr) st16((bf16*)it.y2 + ((int64_t)bh * n2 + bx) * kD + t * 8, y2);
+        // this workgroup's level-2 row is row bx % 16 of level-2 block bx / 16: its 8-channel chunk
         // t goes straight into that block's tiles (the other 15 rows come from the neighbouring workgroups)
-        const int64_t tile2 = ((int64_t)bh * (n2 / kBlk) + blockIdx.x / kBlk) * kTile;
-        const int r2 = blockIdx.x % kBlk;
+        const int64_t tile2 = ((int64_t)bh * (n2 / kBlk) + bx / kBlk) * kTile;
+        const int r2 = bx % kBlk;
         if (it.y2r != nullptr) st16((bf16*)it.y2r + tile2 + (t * 16 + r2) * 8, y2);
         if (it.y2t != nullptr) {
 #pragma unroll
@@ -194,7 +197,7 @@ __global__ __launch_bounds__(128) void pool_pyramid_kernel(PoolParams p) {
         }
     }
     if (it.y1r != nullptr)               // thread (r, c) holds chunk c of pooled row r
-        st16((bf16*)it.y1r + ((int64_t)bh * n2 + blockIdx.x) * kTile + (c * 16 + r) * 8, y);
+        st16((bf16*)it.y1r + ((int64_t)bh * n2 + bx) * kTile + (c * 16 + r) * 8, y);
     if (it.y1t != nullptr) {             // thread -> (channel ch, token half)
         const int ch = t & 63, half = t >> 6;
 #pragma unroll
@@ -202,7 +205,7 @@ __global__ __launch_bounds__(128) void pool_pyramid_kernel(PoolParams p) {
             bf16x4 v;
 #pragma unroll
             for (int j = 0; j < 4; j++) v[j] = sm[half * 8 + q * 4 + j][ch];
-            st8((bf16*)it.y1t + ((int64_t)bh * n2 + blockIdx.x) * kTile + t_tile_off(half * 8 + q * 4, ch), v);
+            st8((bf16*)it.y1t + ((int64_t)bh * n2 + bx) * kTile + t_tile_off(half * 8 + q * 4, ch), v);
         }
     }
 }
@@ -387,7 +390,8 @@ extern "C" int llsa_pool_pyramid_fwd(const llsa_pool_item* items, int n_items, c
     for (int i = n_items; i < 4; i++) p.it[i] = items[0];
     bool norm = false;
     for (int i = 0; i < n_items; i++) norm = norm || items[i].gamma != nullptr;
-    dim3 grid((max_n + 255) / 256, B * H, n_items);
+    p.n_items = n_items;
+    dim3 grid((max_n + 255) / 256 * n_items, B * H);
     if (norm)
         hipLaunchKernelGGL(HIP_KERNEL_NAME(pool_pyramid_kernel<true>), grid, dim3(128), 0, (hipStream_t)stream, p);
     else

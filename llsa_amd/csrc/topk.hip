@@ -205,16 +205,16 @@ __device__ __forceinline__ void wave_topk_radix(const unsigned* u, int npos, int
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();
-    if (lane < T) {
+    {   // final order by rank counting among the T winners: winner j sits in lane j and is handed round with readlane
         const unsigned mu = sel_u[lane];
         const int mi = sel_i[lane];
         int rank = 0;
         for (int j = 0; j < T; j++) {
-            const unsigned ou = sel_u[j];
-            const int oi = sel_i[j];
+            const unsigned ou = (unsigned)__builtin_amdgcn_readlane((int)mu, j);
+            const int oi = __builtin_amdgcn_readlane(mi, j);
             rank += (ou > mu || (ou == mu && (oi < mi || (oi == mi && j < lane)))) ? 1 : 0;
         }
-        out[rank] = mi;
+        if (lane < T) out[rank] = mi;
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
     __builtin_amdgcn_wave_barrier();

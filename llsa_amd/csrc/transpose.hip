@@ -7,6 +7,7 @@
 #include "llsa_device.h"
 #include "llsa_host.h"
 #include "../../include/llsa_hip.h"
+#include <algorithm>
 
 namespace llsa {
 
@@ -24,69 +25,22 @@ __device__ __forceinline__ int wave_incl_scan(int v, int lane) {
 
 constexpr int kTrPart = 16 * kTrThreads;       // entries per workgroup of the split path
 
-// Work list (optional): the K-side kernels walk each key block's segment in chunks of at most
-// `chunk` entries so that a popular key block does not serialise on one wave.  Per (b,h), all
-// records 4 ints (16-byte aligned when the list is, so that one load fetches a record):
-//   work[0] = number of items, work[1] = number of partial-sum slots, work[2] = number of key
-//   blocks with more than one chunk, work[3] unused,
-//   work[4 + 4i ..]             item i = {key block n, first entry in flat, entries, partial-sum slot
-//                               or -1 when n has one chunk}      (items of one key block are adjacent),
-//   work[4 + 4 max_items + 4j ..] j-th key block with more than one chunk = {n, first slot, chunks, 0}.
-// Every key block has at least one item (an unselected block's item has no entries and only
-// writes zeros), and max_items = Mb*T/chunk + Kb.  Items with more than chunk/2 entries come first
-// in the list: a wave walks its item serially, so the long ones have to start early or the kernel
-// ends with a few waves still working.
-// SPLIT = false: the whole job of one (b,h).  SPLIT = true (many entries): the middle step of three --
-// tr_count_kernel has left the histogram in the tail of the work list, this kernel scans it, writes
-// offsets and work list and leaves every segment's start in the same place as the cursor that
-// tr_scatter_kernel advances.
-template <bool SPLIT>
-__global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int* __restrict__ idx, int* __restrict__ offsets,
-                                                                      int* __restrict__ flat, int* __restrict__ work,
-                                                                      int Mb, int Kb, int T, int chunk, int work_stride) {
-    // These kernels run beside the forward attention kernel on a second stream and are on the
-    // critical path of nothing until the backward starts, but one slow workgroup per (b,h) is all
-    // there is of them: let their waves go first when they share a CU.
-    __builtin_amdgcn_s_setprio(3);
-    HIP_DYNAMIC_SHARED(int, smem)
-    int* pos = smem;                               // Kb
-    int* wave_tot = smem + (SPLIT ? 0 : Kb);       // 5 * kTrWaves (the split form keeps no counters in LDS)
-
+// The middle step of every form of the transpose: counts per key block -> offsets, segment starts and the work list.
+// count_of(i): entries of key block i; set_start(i, start): where the caller wants the start of segment i (its cursor);
+// wave_tot: 5 * kTrWaves ints of LDS.  Called by all kTrThreads threads of the workgroup; `work` already points at the
+// (b,h)'s list (or is nullptr).  E: the sum of all counts.
+template <typename CountFn, typename StartFn>
+__device__ __forceinline__ int offsets_and_work_list(CountFn count_of, StartFn set_start, int* wave_tot, int* __restrict__ offsets,
+                                                      int* __restrict__ work, int Kb, int E_items, int E_total, int chunk) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int bh = blockIdx.x;
-    const int E = Mb * T;
-    idx += (int64_t)bh * E;
-    flat += (int64_t)bh * E;
-    offsets += (int64_t)bh * (Kb + 1);
-
-    constexpr int kBatch = 16;
-    int* tail = SPLIT ? work + (int64_t)bh * work_stride + (work_stride - work_tail_len(Kb)) : nullptr;
-    if (!SPLIT) {
-        for (int i = tid; i < Kb; i += kTrThreads) pos[i] = 0;
-    }
-    __syncthreads();
-    // entries are taken 16 per thread at a time, all 16 loads issued before the first is used
-    for (int e0 = 0; e0 < (SPLIT ? 0 : E); e0 += kBatch * kTrThreads) {
-        int v[kBatch];
-#pragma unroll
-        for (int k = 0; k < kBatch; k++) {
-            const int e = e0 + k * kTrThreads + tid;
-            v[k] = (e < E) ? idx[e] : -1;
-        }
-#pragma unroll
-        for (int k = 0; k < kBatch; k++)
-            if (e0 + k * kTrThreads + tid < E) atomicAdd(&pos[clampi(v[k], 0, Kb - 1)], 1);
-    }
-    __syncthreads();
-
-    // exclusive scan over pos[0..Kb): each thread owns `per` consecutive counters
+    // exclusive scan over the counts: each thread owns `per` consecutive counters
     const int per = (Kb + kTrThreads - 1) / kTrThreads;
     const int c0 = min(tid * per, Kb), c1 = min(c0 + per, Kb);
     // l_items: short items, l_long: long items (more than chunk/2 entries)
     const int long_min = chunk / 2 + 1;
     int local = 0, l_items = 0, l_slots = 0, l_multi = 0, l_long = 0;
     for (int i = c0; i < c1; i++) {
-        const int c = SPLIT ? tail[i] : pos[i];
+        const int c = count_of(i);
         const int nch = max(1, (c + chunk - 1) / chunk);
         const int n_long = (nch - 1) + ((c - (nch - 1) * chunk >= long_min) ? 1 : 0);   // all chunks but the last are full
         local += c;
@@ -121,13 +75,11 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
         }
     }
     run_i += total_long;                                      // short items follow the long ones
-    if (work != nullptr) work += (int64_t)bh * work_stride;
-    const int max_items = E / chunk + Kb;
+    const int max_items = E_items / chunk + Kb;
     for (int i = c0; i < c1; i++) {
-        const int c = SPLIT ? tail[i] : pos[i];
+        const int c = count_of(i);
         offsets[i] = run;
-        if (SPLIT) tail[i] = run;
-        else pos[i] = run;
+        set_start(i, run);
         run += c;
         if (work != nullptr) {
             const int nch = max(1, (c + chunk - 1) / chunk);
@@ -149,13 +101,79 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
             run_s += (nch > 1) ? nch : 0;
         }
     }
-    if (tid == 0) offsets[Kb] = E;
+    if (tid == kTrThreads - 1) offsets[Kb] = run;             // (the last thread's running sum is the total)
     if (work != nullptr && tid == kTrThreads - 1) {
         work[0] = run_i;                                      // (the last thread's short items end the list)
         work[1] = run_s;
         work[2] = run_m;
         work[3] = 0;
     }
+    (void)E_total;
+    return run;                                               // the end of this thread's key blocks: the total for the last thread
+}
+
+// Work list (optional): the K-side kernels walk each key block's segment in chunks of at most
+// `chunk` entries so that a popular key block does not serialise on one wave.  Per (b,h), all
+// records 4 ints (16-byte aligned when the list is, so that one load fetches a record):
+//   work[0] = number of items, work[1] = number of partial-sum slots, work[2] = number of key
+//   blocks with more than one chunk, work[3] unused,
+//   work[4 + 4i ..]             item i = {key block n, first entry in flat, entries, partial-sum slot
+//                               or -1 when n has one chunk}      (items of one key block are adjacent),
+//   work[4 + 4 max_items + 4j ..] j-th key block with more than one chunk = {n, first slot, chunks, 0}.
+// Every key block has at least one item (an unselected block's item has no entries and only
+// writes zeros), and max_items = Mb*T/chunk + Kb.  Items with more than chunk/2 entries come first
+// in the list: a wave walks its item serially, so the long ones have to start early or the kernel
+// ends with a few waves still working.
+// SPLIT = false: the whole job of one (b,h).  SPLIT = true (many entries): the middle step of three --
+// tr_count_kernel has left the histogram in the tail of the work list, this kernel scans it, writes
+// offsets and work list and leaves every segment's start in the same place as the cursor that
+// tr_scatter_kernel advances.
+template <bool SPLIT>
+__global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int* __restrict__ idx, int* __restrict__ offsets,
+                                                                      int* __restrict__ flat, int* __restrict__ work,
+                                                                      int Mb, int Kb, int T, int chunk, int work_stride) {
+    // These kernels run beside the forward attention kernel on a second stream and are on the
+    // critical path of nothing until the backward starts, but one slow workgroup per (b,h) is all
+    // there is of them: let their waves go first when they share a CU.
+    __builtin_amdgcn_s_setprio(3);
+    HIP_DYNAMIC_SHARED(int, smem)
+    int* pos = smem;                               // Kb
+    int* wave_tot = smem + (SPLIT ? 0 : Kb);       // 5 * kTrWaves (the split form keeps no counters in LDS)
+
+    const int tid = threadIdx.x;
+    const int bh = blockIdx.x;
+    const int E = Mb * T;
+    idx += (int64_t)bh * E;
+    flat += (int64_t)bh * E;
+    offsets += (int64_t)bh * (Kb + 1);
+
+    constexpr int kBatch = 16;
+    int* tail = SPLIT ? work + (int64_t)bh * work_stride + (work_stride - work_tail_len(Kb)) : nullptr;
+    if (!SPLIT) {
+        for (int i = tid; i < Kb; i += kTrThreads) pos[i] = 0;
+    }
+    __syncthreads();
+    // entries are taken 16 per thread at a time, all 16 loads issued before the first is used
+    for (int e0 = 0; e0 < (SPLIT ? 0 : E); e0 += kBatch * kTrThreads) {
+        int v[kBatch];
+#pragma unroll
+        for (int k = 0; k < kBatch; k++) {
+            const int e = e0 + k * kTrThreads + tid;
+            v[k] = (e < E) ? idx[e] : -1;
+        }
+#pragma unroll
+        for (int k = 0; k < kBatch; k++)
+            if (e0 + k * kTrThreads + tid < E) atomicAdd(&pos[clampi(v[k], 0, Kb - 1)], 1);
+    }
+    __syncthreads();
+
+    if (work != nullptr) work += (int64_t)bh * work_stride;
+    offsets_and_work_list([&](int i) { return SPLIT ? tail[i] : pos[i]; },
+                          [&](int i, int start) {
+                              if (SPLIT) tail[i] = start;
+                              else pos[i] = start;
+                          },
+                          wave_tot, offsets, work, Kb, E, E, chunk);
     __syncthreads();
 
     for (int e0 = 0; e0 < (SPLIT ? 0 : E); e0 += kBatch * kTrThreads) {
@@ -172,6 +190,114 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
         }
     }
     // pos[n] is now the END of segment n; the segments are sorted by sort_segments_kernel
+}
+
+// The whole transpose of a small job in one workgroup and one pass, sorted as it is built: the workgroup keeps one
+// bitmap over the query blocks per key block in LDS (Kb rows of Mb bits; one word of padding per row keeps the rows
+// off each other's banks), every entry sets its bit, a key block's count is the population of its row, and its
+// segment is written by reading the row's bits back in order -- ascending query blocks with no scatter through
+// atomic cursors and no sorting pass afterwards; the inverse position of an entry is its segment's start plus the
+// bits below its own.  Several jobs (the selections of all levels of one operator call) share a launch:
+// blockIdx.y picks the job.  A job fits when its bitmaps do (tr_bitmap_lds_ints); bigger ones take the kernels above.
+struct TrJob {
+    const int* idx; int* offsets; int* flat; int* work; int* inv;
+    int Mb, Kb, T, chunk, work_stride;
+};
+struct TrJobs {
+    TrJob job[LLSA_MAX_LEVELS];
+};
+__host__ __device__ inline int64_t tr_bitmap_lds_ints(int Mb, int Kb) { return (int64_t)Kb * ((Mb + 31) / 32 + 1) + 5 * kTrWaves; }
+constexpr int64_t kTrBitmapMaxInts = 36 * 1024;               // 144 KB
+
+__global__ __launch_bounds__(kTrThreads) void transpose_bitmap_kernel(TrJobs jobs) {
+    HIP_DYNAMIC_SHARED(int, smem)
+    const TrJob& jb = jobs.job[blockIdx.y];
+    const int Mb = jb.Mb, Kb = jb.Kb, T = jb.T;
+    const int words = (Mb + 31) / 32, stride = words + 1;
+    unsigned* bm = reinterpret_cast<unsigned*>(smem);         // [Kb][stride]
+    int* wave_tot = smem + Kb * stride;                       // 5 * kTrWaves
+    const int tid = threadIdx.x, bh = blockIdx.x;
+    const int E = Mb * T;
+    const int* idx = jb.idx + (int64_t)bh * E;
+    int* flat = jb.flat + (int64_t)bh * E;
+    int* offsets = jb.offsets + (int64_t)bh * (Kb + 1);
+    int* work = jb.work ? jb.work + (int64_t)bh * jb.work_stride : nullptr;
+
+    for (int i = tid; i < Kb * stride; i += kTrThreads) bm[i] = 0u;
+    __syncthreads();
+    constexpr int kBatch = 16;
+    for (int e0 = 0; e0 < E; e0 += kBatch * kTrThreads) {     // 16 loads in flight per thread
+        int v[kBatch];
+#pragma unroll
+        for (int k = 0; k < kBatch; k++) {
+            const int e = e0 + k * kTrThreads + tid;
+            v[k] = (e < E) ? idx[e] : -1;
+        }
+#pragma unroll
+        for (int k = 0; k < kBatch; k++) {
+            const int e = e0 + k * kTrThreads + tid;
+            if (e < E) {
+                const int q = e / T;
+                atomicOr(&bm[clampi(v[k], 0, Kb - 1) * stride + (q >> 5)], 1u << (q & 31));
+            }
+        }
+    }
+    __syncthreads();
+    // counts -> the padding word of each row; the scan then leaves the segment's start there
+    for (int n = tid; n < Kb; n += kTrThreads) {
+        int c = 0;
+        for (int w = 0; w < words; w++) c += __popc(bm[n * stride + w]);
+        bm[n * stride + words] = (unsigned)c;
+    }
+    __syncthreads();
+    const int my_end = offsets_and_work_list([&](int i) { return (int)bm[i * stride + words]; },
+                                             [&](int i, int st) { bm[i * stride + words] = (unsigned)st; },      // the count gives way to the start
+                                             wave_tot, offsets, work, Kb, E, E, jb.chunk);
+    __syncthreads();                                          // (everybody has read the wave totals)
+    if (tid == kTrThreads - 1) wave_tot[0] = my_end;          // the end of the last segment
+    __syncthreads();
+    if (jb.inv != nullptr) {                                  // (needs the bitmaps: before the rows are re-used below)
+        int* inv = jb.inv + (int64_t)bh * E;
+        for (int e = tid; e < E; e += kTrThreads) {
+            const int q = e / T, n = clampi(idx[e], 0, Kb - 1);
+            const unsigned* row = bm + n * stride;
+            int pos = (int)row[words];
+            for (int w = 0; w < (q >> 5); w++) pos += __popc(row[w]);
+            pos += __popc(row[q >> 5] & ((1u << (q & 31)) - 1u));
+            inv[e] = pos;
+        }
+        __syncthreads();
+    }
+    // The segment of key block n, ascending: one loop over the row's set bits (a mask of its non-empty words says where the next
+    // one is), so a wave makes as many rounds as its longest segment has entries.  The phase is bound by its stores, 4 bytes per
+    // lane into a line of its own (11 of the kernel's 20 us at 1024 x 1024 blocks, topk 16); staging the segments in the rest
+    // of LDS for a linear copy was slower still (bank conflicts: the segments of a wave's rows start 16 words apart).
+    for (int n = tid; n < Kb; n += kTrThreads) {
+        const unsigned* row = bm + n * stride;
+        int out = (int)row[words];
+        for (int w0 = 0; w0 < words; w0 += 32) {
+            const int nw = min(32, words - w0);
+            unsigned full = 0u;
+            int bits = 0;
+            for (int w = 0; w < nw; w++) {
+                const unsigned wd = row[w0 + w];
+                full |= (wd != 0u ? 1u : 0u) << w;
+                bits += __popc(wd);
+            }
+            unsigned wd = 0u;
+            int base = 0;
+            for (int j = 0; j < bits; j++) {
+                if (wd == 0u) {
+                    const int w = __ffs((int)full) - 1;
+                    full &= full - 1u;
+                    wd = row[w0 + w];
+                    base = (w0 + w) * 32;
+                }
+                flat[out++] = base + __ffs((int)wd) - 1;
+                wd &= wd - 1u;
+            }
+        }
+    }
 }
 
 // Split path, first and last step: one workgroup per kTrPart entries.
@@ -301,12 +427,29 @@ extern "C" int64_t llsa_work_list_len(int Mb, int Kb, int T, int chunk) {
     return 4 + 4 * (e / chunk + Kb) + 4 * (e / chunk + 1) + work_tail_len(Kb);
 }
 
-extern "C" int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, int32_t* work, int32_t* inv, int B, int H,
-                                      int Mb, int Kb, int T, int chunk, void* stream) {
+static int check_transpose_job(const int32_t* idx, const int32_t* offsets, const int32_t* flat, const int32_t* work, int B, int H, int Mb, int Kb,
+                               int T, int chunk) {
     LLSA_REQUIRE(idx && offsets && flat, "transpose_indices: null argument");
     LLSA_REQUIRE(B > 0 && H > 0 && Mb > 0 && Kb > 0 && T > 0, "transpose_indices: bad shape");
     LLSA_REQUIRE(work == nullptr || chunk >= 1, "transpose_indices: work list needs chunk >= 1");
-    if (chunk < 1) chunk = 1;
+    return 0;
+}
+
+// the jobs whose bitmaps fit LDS, all in one launch
+static int launch_bitmap_jobs(const TrJobs& jobs, int n_jobs, int B, int H, hipStream_t st) {
+    int64_t ints = 0;
+    for (int i = 0; i < n_jobs; i++) ints = std::max(ints, tr_bitmap_lds_ints(jobs.job[i].Mb, jobs.job[i].Kb));
+    const size_t lds = sizeof(int) * (size_t)ints;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void*)transpose_bitmap_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return fail(-101, "transpose_indices: cannot raise dynamic LDS to %zu bytes: %s", lds, hipGetErrorString(e));
+    }
+    hipLaunchKernelGGL(transpose_bitmap_kernel, dim3(B * H, n_jobs), dim3(kTrThreads), lds, st, jobs);
+    return launch_status("transpose_indices");
+}
+
+static int transpose_general(const int32_t* idx, int32_t* offsets, int32_t* flat, int32_t* work, int32_t* inv, int B, int H, int Mb, int Kb,
+                             int T, int chunk, void* stream) {
     const size_t lds = sizeof(int) * ((size_t)Kb + 128);
     static_assert(5 * kTrWaves <= 128, "wave totals must fit their LDS slot");
     LLSA_REQUIRE(lds <= 160 * 1024 || (work != nullptr && (int64_t)Mb * T >= 4 * kTrPart),
@@ -346,4 +489,35 @@ extern "C" int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int3
         hipLaunchKernelGGL(inverse_positions_kernel, dim3((unsigned)((E + 255) / 256), B * H), dim3(256), 0, (hipStream_t)stream, idx,
                            (const int*)offsets, (const int*)flat, inv, Mb, Kb, T);
     return launch_status("transpose_indices");
+}
+
+extern "C" int llsa_transpose_indices_multi(const llsa_transpose_job* jobs, int n_jobs, int B, int H, void* stream) {
+    LLSA_REQUIRE(jobs != nullptr && n_jobs >= 1 && n_jobs <= LLSA_MAX_LEVELS, "transpose_indices: 1..%d jobs, got %d", LLSA_MAX_LEVELS, n_jobs);
+    TrJobs small;
+    int n_small = 0;
+    for (int i = 0; i < n_jobs; i++) {
+        const llsa_transpose_job& j = jobs[i];
+        const int rc = check_transpose_job(j.idx, j.offsets, j.flat, j.work, B, H, j.Mb, j.Kb, j.T, j.chunk);
+        if (rc != 0) return rc;
+        const int chunk = j.chunk < 1 ? 1 : j.chunk;
+        if (tr_bitmap_lds_ints(j.Mb, j.Kb) <= kTrBitmapMaxInts) {
+            TrJob& t = small.job[n_small++];
+            t.idx = j.idx; t.offsets = j.offsets; t.flat = j.flat; t.work = j.work; t.inv = j.inv;
+            t.Mb = j.Mb; t.Kb = j.Kb; t.T = j.T; t.chunk = chunk;
+            t.work_stride = j.work ? (int)llsa_work_list_len(j.Mb, j.Kb, j.T, chunk) : 0;
+        } else {
+            const int rc2 = transpose_general(j.idx, j.offsets, j.flat, j.work, j.inv, B, H, j.Mb, j.Kb, j.T, chunk, stream);
+            if (rc2 != 0) return rc2;
+        }
+    }
+    if (n_small > 0) return launch_bitmap_jobs(small, n_small, B, H, (hipStream_t)stream);
+    return 0;
+}
+
+extern "C" int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, int32_t* work, int32_t* inv, int B, int H,
+                                      int Mb, int Kb, int T, int chunk, void* stream) {
+    llsa_transpose_job j;
+    j.idx = idx; j.offsets = offsets; j.flat = flat; j.work = work; j.inv = inv;
+    j.Mb = Mb; j.Kb = Kb; j.T = T; j.chunk = chunk;
+    return llsa_transpose_indices_multi(&j, 1, B, H, stream);
 }

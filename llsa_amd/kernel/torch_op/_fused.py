@@ -21,10 +21,11 @@ import ctypes as C
 import torch
 from torch.autograd import Function
 
-from ..._lib import CHUNK_FINE, MAX_LEVELS, AttnBwdArgs, AttnFwdArgs, PoolItem, current_lib
+from ..._lib import CHUNK_FINE, MAX_LEVELS, AttnBwdArgs, AttnFwdArgs, PoolItem, TransposeJob, current_lib
 
-_side = {}          # device -> (second stream, two events)
+_side = {}          # device -> second stream
 _SIDE_STREAM_MIN_TOKENS = 1 << 17
+_BITMAP_MAX_PAIRS = 1 << 20          # query blocks x key blocks up to which llsa_transpose_indices_multi is one small launch
 
 
 def _rows_ok(t):
@@ -213,18 +214,26 @@ class LlsaFused(Function):
             _check(lib, lib.topk_sparse(at(lay.pq, l), at(lay.pk, l), pi(lay.sel[l]), pi(lay.sel[l - 1]), B, H, n[l], topks[l - 1],
                                         topks[l], stream), "compute_topk_indices_sparse")
 
-        # The lists of the backward go to a second stream, beside the attention kernel.  The attention
-        # kernel is issued first (the GPU is waiting for it); an event recorded before it lets the
-        # second stream start as soon as the selection is done.
-        # (Below _SIDE_STREAM_MIN_TOKENS tokens over all heads the step is bound by the host, which the two
-        # event waits cost 30 us; the GPU then has the time to build the lists on the one stream.)
+        # The lists of the backward (the transposed selections of all levels).  Up to 2^14 tokens a (b,h)'s bitmap of
+        # (key block, query block) fits LDS and one launch of one workgroup per (b,h) and level does everything, sorted as
+        # it goes, behind the attention kernel on the same stream (on a second stream, beside the backward's dQ kernel, the
+        # two event edges cost more than the overlap saves: 0.373 against 0.358 ms a step at B=2, H=6, N=16384).  Beyond
+        # that the lists take several kernels per level, which run on a second stream beside the attention kernel: the
+        # attention kernel is issued first (the GPU is waiting for it), and an event recorded before it lets the second
+        # stream start as soon as the selection is done.  With few tokens over all heads the step is bound by the host,
+        # which the event calls cost more than the GPU saves: everything then goes to the one stream.
+        jobs = (TransposeJob * L)()
+        if grad:
+            jobs[0] = TransposeJob(pi(lay.sel[0]), pi(lay.off[0]), pi(lay.flat[0]), pi(lay.work), None, n[1], n[1], topks[0], CHUNK_FINE)
+            for l in range(1, L):
+                jobs[l] = TransposeJob(pi(lay.sel[l]), pi(lay.off[l]), pi(lay.flat[l]), None, pi(lay.inv[l]), n[l + 1], n[l + 1], topks[l], 1)
         cur = side = None
-        if grad and lib.device_library and B * H * N >= _SIDE_STREAM_MIN_TOKENS:
+        if grad and lib.device_library and n[1] * n[1] > _BITMAP_MAX_PAIRS and B * H * N >= _SIDE_STREAM_MIN_TOKENS:
             cur = torch.cuda.current_stream(dev)
-            pack = _side.get(dev)
-            if pack is None:
-                pack = _side[dev] = (torch.cuda.Stream(device=dev), torch.cuda.Event(), torch.cuda.Event())
-            side, ev_idx, ev_lists = pack
+            side = _side.get(dev)
+            if side is None:
+                side = _side[dev] = torch.cuda.Stream(device=dev)
+            ev_idx = torch.cuda.Event()
             ev_idx.record(cur)
 
         f = AttnFwdArgs()
@@ -244,14 +253,11 @@ class LlsaFused(Function):
             if side is not None:
                 side.wait_event(ev_idx)         # (the arena is older than the selection, so this covers it too)
                 s_lists = C.c_void_p(side.cuda_stream)
-            _check(lib, lib.transpose_indices(pi(lay.sel[0]), pi(lay.off[0]), pi(lay.flat[0]), pi(lay.work), None, B, H, n[1], n[1],
-                                              topks[0], CHUNK_FINE, s_lists), "transpose_indices")
-            for l in range(1, L):
-                _check(lib, lib.transpose_indices(pi(lay.sel[l]), pi(lay.off[l]), pi(lay.flat[l]), None, pi(lay.inv[l]), B, H,
-                                                  n[l + 1], n[l + 1], topks[l], 1, s_lists), "transpose_indices (pooled level)")
+            _check(lib, lib.transpose_indices_multi(jobs, L, B, H, s_lists), "transpose_indices")
             if side is not None:
+                ev_lists = torch.cuda.Event()
                 ev_lists.record(side)
-                cur.wait_event(ev_lists)
+                cur.wait_event(ev_lists)        # (and the arena is not handed out again before the second stream is done)
 
         if grad:
             # (q and k themselves are needed again only by the backward of the qk-norm)
