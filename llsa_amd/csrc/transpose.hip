@@ -28,10 +28,12 @@ constexpr int kTrPart = 16 * kTrThreads;       // entries per workgroup of the s
 // The middle step of every form of the transpose: counts per key block -> offsets, segment starts and the work list.
 // count_of(i): entries of key block i; set_start(i, start): where the caller wants the start of segment i (its cursor);
 // wave_tot: 5 * kTrWaves ints of LDS.  Called by all kTrThreads threads of the workgroup; `work` already points at the
-// (b,h)'s list (or is nullptr).  E: the sum of all counts.
+// (b,h)'s list (or is nullptr).  E: the sum of all counts.  write_out = false: only set_start is called, offsets and work list
+// stay untouched (a workgroup that shares the (b,h) with others and leaves these writes to one of them).
 template <typename CountFn, typename StartFn>
 __device__ __forceinline__ int offsets_and_work_list(CountFn count_of, StartFn set_start, int* wave_tot, int* __restrict__ offsets,
-                                                      int* __restrict__ work, int Kb, int E_items, int E_total, int chunk) {
+                                                      int* __restrict__ work, int Kb, int E_items, int E_total, int chunk,
+                                                      bool write_out = true) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     // exclusive scan over the counts: each thread owns `per` consecutive counters
     const int per = (Kb + kTrThreads - 1) / kTrThreads;
@@ -78,10 +80,10 @@ __device__ __forceinline__ int offsets_and_work_list(CountFn count_of, StartFn s
     const int max_items = E_items / chunk + Kb;
     for (int i = c0; i < c1; i++) {
         const int c = count_of(i);
-        offsets[i] = run;
+        if (write_out) offsets[i] = run;
         set_start(i, run);
         run += c;
-        if (work != nullptr) {
+        if (work != nullptr && write_out) {
             const int nch = max(1, (c + chunk - 1) / chunk);
             for (int ci = 0; ci < nch; ci++) {
                 const int n_ent = min(chunk, c - ci * chunk);
@@ -101,8 +103,8 @@ __device__ __forceinline__ int offsets_and_work_list(CountFn count_of, StartFn s
             run_s += (nch > 1) ? nch : 0;
         }
     }
-    if (tid == kTrThreads - 1) offsets[Kb] = run;             // (the last thread's running sum is the total)
-    if (work != nullptr && tid == kTrThreads - 1) {
+    if (write_out && tid == kTrThreads - 1) offsets[Kb] = run;        // (the last thread's running sum is the total)
+    if (write_out && work != nullptr && tid == kTrThreads - 1) {
         work[0] = run_i;                                      // (the last thread's short items end the list)
         work[1] = run_s;
         work[2] = run_m;
@@ -199,12 +201,17 @@ __global__ __launch_bounds__(kTrThreads) void transpose_indices_kernel(const int
 // atomic cursors and no sorting pass afterwards; the inverse position of an entry is its segment's start plus the
 // bits below its own.  Several jobs (the selections of all levels of one operator call) share a launch:
 // blockIdx.y picks the job.  A job fits when its bitmaps do (tr_bitmap_lds_ints); bigger ones take the kernels above.
+// Writing the segments is the long phase (4-byte stores, every lane into a line of its own, which one CU's memory
+// pipeline takes a lane at a time): a job with many key blocks is given `parts` workgroups per (b,h), each of which
+// builds the same bitmaps, counts and starts for itself (cheap, and no word has to pass between workgroups) and writes
+// the segments of its share of the key blocks; the first of them also writes offsets and work list.
 struct TrJob {
     const int* idx; int* offsets; int* flat; int* work; int* inv;
-    int Mb, Kb, T, chunk, work_stride;
+    int Mb, Kb, T, chunk, work_stride, parts;
 };
 struct TrJobs {
     TrJob job[LLSA_MAX_LEVELS];
+    int max_parts;                                            // workgroups per (b,h) in the grid; job i uses the first job[i].parts
 };
 __host__ __device__ inline int64_t tr_bitmap_lds_ints(int Mb, int Kb) { return (int64_t)Kb * ((Mb + 31) / 32 + 1) + 5 * kTrWaves; }
 constexpr int64_t kTrBitmapMaxInts = 36 * 1024;               // 144 KB
@@ -212,11 +219,13 @@ constexpr int64_t kTrBitmapMaxInts = 36 * 1024;               // 144 KB
 __global__ __launch_bounds__(kTrThreads) void transpose_bitmap_kernel(TrJobs jobs) {
     HIP_DYNAMIC_SHARED(int, smem)
     const TrJob& jb = jobs.job[blockIdx.y];
+    const int part = blockIdx.x % jobs.max_parts, bh = blockIdx.x / jobs.max_parts;
+    if (part >= jb.parts) return;
     const int Mb = jb.Mb, Kb = jb.Kb, T = jb.T;
     const int words = (Mb + 31) / 32, stride = words + 1;
     unsigned* bm = reinterpret_cast<unsigned*>(smem);         // [Kb][stride]
     int* wave_tot = smem + Kb * stride;                       // 5 * kTrWaves
-    const int tid = threadIdx.x, bh = blockIdx.x;
+    const int tid = threadIdx.x;
     const int E = Mb * T;
     const int* idx = jb.idx + (int64_t)bh * E;
     int* flat = jb.flat + (int64_t)bh * E;
@@ -252,13 +261,13 @@ __global__ __launch_bounds__(kTrThreads) void transpose_bitmap_kernel(TrJobs job
     __syncthreads();
     const int my_end = offsets_and_work_list([&](int i) { return (int)bm[i * stride + words]; },
                                              [&](int i, int st) { bm[i * stride + words] = (unsigned)st; },      // the count gives way to the start
-                                             wave_tot, offsets, work, Kb, E, E, jb.chunk);
+                                             wave_tot, offsets, work, Kb, E, E, jb.chunk, part == 0);
     __syncthreads();                                          // (everybody has read the wave totals)
     if (tid == kTrThreads - 1) wave_tot[0] = my_end;          // the end of the last segment
     __syncthreads();
-    if (jb.inv != nullptr) {                                  // (needs the bitmaps: before the rows are re-used below)
+    if (jb.inv != nullptr) {
         int* inv = jb.inv + (int64_t)bh * E;
-        for (int e = tid; e < E; e += kTrThreads) {
+        for (int e = part * kTrThreads + tid; e < E; e += jb.parts * kTrThreads) {
             const int q = e / T, n = clampi(idx[e], 0, Kb - 1);
             const unsigned* row = bm + n * stride;
             int pos = (int)row[words];
@@ -266,34 +275,31 @@ __global__ __launch_bounds__(kTrThreads) void transpose_bitmap_kernel(TrJobs job
             pos += __popc(row[q >> 5] & ((1u << (q & 31)) - 1u));
             inv[e] = pos;
         }
-        __syncthreads();
     }
-    // The segment of key block n, ascending: one loop over the row's set bits (a mask of its non-empty words says where the next
-    // one is), so a wave makes as many rounds as its longest segment has entries.  The phase is bound by its stores, 4 bytes per
-    // lane into a line of its own (11 of the kernel's 20 us at 1024 x 1024 blocks, topk 16); staging the segments in the rest
-    // of LDS for a linear copy was slower still (bank conflicts: the segments of a wave's rows start 16 words apart).
-    for (int n = tid; n < Kb; n += kTrThreads) {
-        const unsigned* row = bm + n * stride;
-        int out = (int)row[words];
-        for (int w0 = 0; w0 < words; w0 += 32) {
-            const int nw = min(32, words - w0);
-            unsigned full = 0u;
-            int bits = 0;
-            for (int w = 0; w < nw; w++) {
-                const unsigned wd = row[w0 + w];
-                full |= (wd != 0u ? 1u : 0u) << w;
-                bits += __popc(wd);
-            }
-            unsigned wd = 0u;
-            int base = 0;
-            for (int j = 0; j < bits; j++) {
-                if (wd == 0u) {
-                    const int w = __ffs((int)full) - 1;
-                    full &= full - 1u;
-                    wd = row[w0 + w];
-                    base = (w0 + w) * 32;
-                }
-                flat[out++] = base + __ffs((int)wd) - 1;
+    // The segments, ascending.  Eight neighbouring lanes share a key block's row, each with an eighth of its words: the lanes
+    // count their bits, a scan over the eight gives each its place in the segment, and each writes the query blocks of its
+    // own words.  (One lane per row made a wave walk as many rounds as its longest segment has entries, every round a 4-byte
+    // store per lane into a line of its own; this way a round writes eight segments, and a row of 16 entries takes 2 or 3.)
+    const int rows = (Kb + jb.parts - 1) / jb.parts, r1 = min(Kb, (part + 1) * rows);
+    const int sub = tid & 7, wps = (words + 7) / 8, w_lo = min(words, sub * wps), w_hi = min(words, w_lo + wps);
+    for (int n0 = part * rows; n0 < r1; n0 += kTrThreads / 8) {
+        const int n = n0 + (tid >> 3);
+        const unsigned* row = bm + min(n, Kb - 1) * stride;
+        int mine = 0;
+        if (n < r1)
+            for (int w = w_lo; w < w_hi; w++) mine += __popc(row[w]);
+        int incl = mine;                                      // (all lanes take part in the shuffles)
+#pragma unroll
+        for (int d = 1; d < 8; d <<= 1) {
+            const int o = __shfl_up(incl, d, 8);
+            if (sub >= d) incl += o;
+        }
+        if (n >= r1) continue;
+        int out = (int)row[words] + incl - mine;
+        for (int w = w_lo; w < w_hi; w++) {
+            unsigned wd = row[w];
+            while (wd) {
+                flat[out++] = w * 32 + __ffs((int)wd) - 1;
                 wd &= wd - 1u;
             }
         }
@@ -436,7 +442,7 @@ static int check_transpose_job(const int32_t* idx, const int32_t* offsets, const
 }
 
 // the jobs whose bitmaps fit LDS, all in one launch
-static int launch_bitmap_jobs(const TrJobs& jobs, int n_jobs, int B, int H, hipStream_t st) {
+static int launch_bitmap_jobs(TrJobs& jobs, int n_jobs, int B, int H, hipStream_t st) {
     int64_t ints = 0;
     for (int i = 0; i < n_jobs; i++) ints = std::max(ints, tr_bitmap_lds_ints(jobs.job[i].Mb, jobs.job[i].Kb));
     const size_t lds = sizeof(int) * (size_t)ints;
@@ -444,7 +450,9 @@ static int launch_bitmap_jobs(const TrJobs& jobs, int n_jobs, int B, int H, hipS
         hipError_t e = hipFuncSetAttribute((const void*)transpose_bitmap_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return fail(-101, "transpose_indices: cannot raise dynamic LDS to %zu bytes: %s", lds, hipGetErrorString(e));
     }
-    hipLaunchKernelGGL(transpose_bitmap_kernel, dim3(B * H, n_jobs), dim3(kTrThreads), lds, st, jobs);
+    jobs.max_parts = 1;
+    for (int i = 0; i < n_jobs; i++) jobs.max_parts = std::max(jobs.max_parts, jobs.job[i].parts);
+    hipLaunchKernelGGL(transpose_bitmap_kernel, dim3(B * H * jobs.max_parts, n_jobs), dim3(kTrThreads), lds, st, jobs);
     return launch_status("transpose_indices");
 }
 
@@ -505,6 +513,7 @@ extern "C" int llsa_transpose_indices_multi(const llsa_transpose_job* jobs, int 
             t.idx = j.idx; t.offsets = j.offsets; t.flat = j.flat; t.work = j.work; t.inv = j.inv;
             t.Mb = j.Mb; t.Kb = j.Kb; t.T = j.T; t.chunk = chunk;
             t.work_stride = j.work ? (int)llsa_work_list_len(j.Mb, j.Kb, j.T, chunk) : 0;
+            t.parts = std::min(8, std::max(1, j.Kb / 128));
         } else {
             const int rc2 = transpose_general(j.idx, j.offsets, j.flat, j.work, j.inv, B, H, j.Mb, j.Kb, j.T, chunk, stream);
             if (rc2 != 0) return rc2;
