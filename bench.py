@@ -114,7 +114,7 @@ def stage_profile(op, q, k, v, do, t1, t2, freq, iters, torch):
     fused operator makes, and times each stage with events on the launch stream."""
     from llsa_amd.kernel.hip import _attention as A
     from llsa_amd._lib import CHUNK_FINE
-    from llsa_amd.kernel.hip.indices_transpose import transpose_indices
+    from llsa_amd.kernel.hip.indices_transpose import transpose_indices_levels
     from llsa_amd.kernel.hip.mean_pool import PoolSpec, pool_pyramid
     from llsa_amd.kernel.hip.topk import compute_topk_indices_sparse, gen_sparse_indices
     B, H, N, D = q.shape
@@ -155,9 +155,9 @@ def stage_profile(op, q, k, v, do, t1, t2, freq, iters, torch):
     o, lse = A.attn_fwd(q, k, v, pk, pv, idx, 16.0, tiles=tiles, **kw)
     res["attn_fwd"] = timed(lambda: A.attn_fwd(q, k, v, pk, pv, idx, 16.0, tiles=tiles, **kw), iters, torch)
 
-    def transposes():
-        r = transpose_indices(idx, N // 16, CHUNK_FINE)
-        return r + transpose_indices(pidx, N // 256, inverse=True) if l2 else r
+    def transposes():          # all levels with one call, as the operator does it
+        r = transpose_indices_levels([idx, pidx] if l2 else [idx], CHUNK_FINE)
+        return r[0] + r[1] if l2 else r[0]
 
     csr = transposes()
     res["transpose_indices"] = timed(transposes, iters, torch)

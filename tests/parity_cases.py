@@ -270,6 +270,34 @@ def check_transpose(dev, B=2, H=2, Mb=64, T=8, Kb=None, chunk=0):
     assert ((inv.reshape(B, H, -1) >= lo) & (inv.reshape(B, H, -1) < hi)).all(), "inverse position outside its key block's segment"
 
 
+def check_transpose_levels(dev, B=2, H=3, sizes=((1024, 16), (64, 16)), chunk=64):
+    """All levels with one call of the library (one launch when the bitmaps fit) against the oracle and against
+    the work list the single-level call builds."""
+    from llsa_amd.kernel.hip.indices_transpose import transpose_indices, transpose_indices_levels
+    g = torch.Generator().manual_seed(14)
+    sels = [torch.stack([torch.randperm(Mb, generator=g)[:T] for _ in range(B * H * Mb)]).reshape(B, H, Mb, T).int() for Mb, T in sizes]
+    res = transpose_indices_levels([s.to(dev) for s in sels], chunk)
+    for l, (sel, (off, flat, extra)) in enumerate(zip(sels, res)):
+        Mb, T = sel.shape[2:]
+        ro, rf = O.transpose_indices(sel.long(), None)
+        assert torch.equal(off.cpu().long(), ro), f"level {l}: offsets differ"
+        assert torch.equal(flat.cpu().long(), rf), f"level {l}: flat list differs"
+        if l == 0:
+            work = transpose_indices(sel.to(dev), None, chunk)[2].cpu()
+            got, max_items = extra.cpu(), Mb * T // chunk + Mb
+            for b in range(B):              # header, items and multi-piece records (what lies beyond them is never read)
+                for h in range(H):
+                    a, w = got[b, h], work[b, h]
+                    assert torch.equal(a[:4], w[:4]), "work list header differs from the single call's"
+                    assert torch.equal(a[4:4 + 4 * int(w[0])], w[4:4 + 4 * int(w[0])]), "work items differ from the single call's"
+                    m0 = 4 + 4 * max_items
+                    assert torch.equal(a[m0:m0 + 4 * int(w[2])], w[m0:m0 + 4 * int(w[2])]), "multi-piece records differ"
+        else:
+            qid = torch.arange(Mb).view(1, 1, Mb, 1).expand(B, H, Mb, T)
+            inv = extra.cpu().long().reshape(B, H, -1)
+            assert torch.equal(torch.gather(rf, -1, inv).reshape(B, H, Mb, T), qid), f"level {l}: inverse positions do not hold their query block"
+
+
 def check_transpose_hot_block(dev):
     """Every query block selects key block 5 (a segment as long as the query axis) plus others."""
     from llsa_amd.kernel.hip.indices_transpose import transpose_indices
@@ -658,6 +686,73 @@ def check_op_l3(dev, B=1, H=1, N=262144, T=16, T2=16, T3=16, rope=True, qk_norm=
     _, own = O.llsa_l3_fwd(qr, kr, vc, T, T2, T3, 16)
     same = lambda a, b: (a.sort(-1).values == b.long().sort(-1).values).all(-1).float().mean().item()
     assert same(ppidx, own["pp_indices"]) > 0.9 and same(pidx, own["p_indices"]) > 0.9 and same(idx, own["indices"]) > 0.9
+
+
+
+def check_op_lk_sparse_dout(dev, N=4194304, topks=(16, 16, 16, 16), H=1, query_blocks=(0, 7777, -1), rope=True):
+    """dK and dV of llsa_lk, every element, at sizes the whole-tensor oracle cannot hold.  dO is zero outside a few
+    query blocks: a query with dO = 0 has dP = 0 and delta = 0, so it adds exact zeros to dK and dV, and the whole of
+    dK / dV follows from those few queries -- enumerated here in fp64 (torch.autograd over each query's key set, taken
+    from the device's own selection: its fine blocks, the pooled blocks of every level, the dense coarsest level) and
+    pushed down the chain of mean pools (a pooled token's gradient goes to its 16 children, divided by 16) and back
+    through the rotation.  This pins what the single-query checks of o and dq cannot: the group-major pass of every
+    level (its list owners 16, 256, ... groups wide), the partial sums placed by inverse positions, their reduction,
+    the dense coarsest level, and the fold of the whole chain into the fine dK / dV."""
+    import llsa_amd
+    from llsa_amd.kernel.torch_op._fused import selection
+    from llsa_amd.utils.rope_table import rope_table
+    L = len(topks)
+    assert L >= 2, "one level keeps the reference's weight-1 pooled gradient (sparse_attention_res_1.py:388-389): not enumerated here"
+    q, k, v, _ = smooth_inputs(1, H, N, 64, dev)
+    freq = rope_table(int(math.isqrt(N)), dtype=torch.bfloat16).to(dev) if rope else None
+    g = torch.Generator().manual_seed(31)
+    blocks = [b % (N // 16) for b in query_blocks]
+    do = torch.zeros(1, H, N, 64, dtype=torch.bfloat16)
+    for b in blocks:
+        do[0, :, b * 16:b * 16 + 16] = torch.randn(H, 16, 64, generator=g).bfloat16()
+    captured = {}
+
+    def run(q_, k_, v_):
+        out = llsa_amd.llsa_lk(q_, k_, v_, topks, 16, rope=freq)
+        captured["sel"] = [t.cpu().long() for t in selection(out)]
+        return out
+
+    _, _, dk, dv = _grads(run, q, k, v, do.to(dev))
+    sels = captured["sel"]
+    qc, kc, vc = (t.cpu() for t in (q, k, v))
+    fc = freq.cpu() if rope else None
+    qr, kr = (O.rope_apply(qc, fc), O.rope_apply(kc, fc)) if rope else (qc, kc)
+    ks, vs = [kr], [vc]                                       # level 0 .. L: what the attention multiplies (bf16 rows)
+    for _ in range(L):
+        ks.append(O.mean_pool(ks[-1], 16)), vs.append(O.mean_pool(vs[-1], 16))
+    for h in range(H):
+        gk = [torch.zeros(N // 16 ** l, 64, dtype=torch.float64) for l in range(L + 1)]
+        gv = [torch.zeros(N // 16 ** l, 64, dtype=torch.float64) for l in range(L + 1)]
+        for b in blocks:
+            rows, lvls = [], []                               # the key set of this query block: (level, token) lists
+            for l in range(L):
+                for blk in sels[l][0, h, b // 16 ** l].tolist():
+                    rows.append(torch.arange(blk * 16, blk * 16 + 16)), lvls.append(l)
+            rows.append(torch.arange(N // 16 ** L)), lvls.append(L)
+            kk = [ks[l][0, h, r].double().requires_grad_(True) for r, l in zip(rows, lvls)]
+            vv = [vs[l][0, h, r].double().requires_grad_(True) for r, l in zip(rows, lvls)]
+            logw = torch.cat([torch.full((len(r),), math.log(16.0 ** l), dtype=torch.float64) for r, l in zip(rows, lvls)])
+            qq = qr[0, h, b * 16:b * 16 + 16].double()
+            p = torch.softmax(qq @ torch.cat(kk).T / 8.0 + logw, -1)
+            loss = ((p @ torch.cat(vv)) * do[0, h, b * 16:b * 16 + 16].double()).sum()
+            grads = torch.autograd.grad(loss, kk + vv)
+            for i, (r, l) in enumerate(zip(rows, lvls)):
+                gk[l].index_add_(0, r, grads[i])
+                gv[l].index_add_(0, r, grads[len(rows) + i])
+        for l in range(L, 0, -1):                             # down the chain of mean pools
+            gk[l - 1] += gk[l].repeat_interleave(16, 0) / 16.0
+            gv[l - 1] += gv[l].repeat_interleave(16, 0) / 16.0
+        rk = gk[0].float().view(1, 1, N, 64)
+        if rope:
+            rk = O.rope_apply_bwd(rk.bfloat16(), fc).float()
+        tag = f"l{L} N={N} sparse dO"
+        close(f"dk[{h}]", dk[:, h:h + 1], rk, report=tag)
+        close(f"dv[{h}]", dv[:, h:h + 1], gv[0].float().view(1, 1, N, 64), report=tag)
 
 
 def check_op_lk_samples(dev, N=4194304, topks=(16, 16, 16, 16), H=1, queries=(0, 1234567, -1), rows=16384):

@@ -68,6 +68,7 @@ def test_transpose():
     P.check_transpose(DEV, B=1, H=1, Mb=64, T=4, Kb=16)
     P.check_transpose(DEV, B=1, H=2, Mb=4096, T=16, chunk=64)        # 65536 entries: the split form
     P.check_transpose_hot_block(DEV)
+    P.check_transpose_levels(DEV, B=1, H=2, sizes=((256, 8), (16, 4)))
 
 
 def test_attn_l1():
@@ -97,3 +98,9 @@ def test_attn_l2_hot_coarse_block():
 
 def test_op_l2_fused_rope():
     P.check_op_l2(DEV, B=1, H=1, N=16384, T=4, T2=4, fused=True, rope=True)
+
+
+def test_sparse_dout_enumeration_two_levels():
+    """The element-wise dK / dV check that the GPU suite runs at three and four levels, at two levels and N = 16384 here
+    (where the whole-tensor oracle agrees too: test_op_l2_fused_rope): the enumeration itself is what this pins."""
+    P.check_op_lk_sparse_dout(DEV, N=16384, topks=(8, 4), H=1, query_blocks=(0, 517, -1), rope=True)

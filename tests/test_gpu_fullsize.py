@@ -75,6 +75,13 @@ def test_four_levels_single_queries_against_enumeration(dev):
     P.check_op_lk_samples(dev, N=4194304, topks=(16, 16, 16, 16))
 
 
+@pytest.mark.parametrize("N,topks,H", [(4194304, (16, 16, 16, 16), 1), (262144, (8, 4, 8), 2), (16384, (16, 16), 2)])
+def test_dk_dv_elementwise_with_sparse_dout(dev, N, topks, H):
+    """Every element of dK and dV at two, three and four levels: dO is zero outside three query blocks, so the whole
+    gradient follows from 48 queries, enumerated on the CPU in fp64 from the device's selection."""
+    P.check_op_lk_sparse_dout(dev, N=N, topks=topks, H=H)
+
+
 def test_three_levels_single_queries_against_enumeration(dev):
     P.check_op_lk_samples(dev, N=262144, topks=(8, 4, 8), H=2)
 

@@ -85,6 +85,8 @@ def test_transpose(dev):
     P.check_transpose(dev, B=1, H=2, Mb=64, T=16)
     P.check_transpose(dev, B=1, H=1, Mb=64, T=4, Kb=16)
     P.check_transpose_hot_block(dev)
+    P.check_transpose_levels(dev)                                    # two levels, one launch
+    P.check_transpose_levels(dev, B=1, H=2, sizes=((256, 16),))
 
 
 def test_transpose_largest(dev):
