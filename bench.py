@@ -61,14 +61,14 @@ def measured_traffic(workload):
         parts = line.split()
         if len(parts) >= 7 and parts[0].startswith("llsa::"):
             try:
-                rows[parts[0]] = (float(parts[-3]) + float(parts[-2])) * 1e6       # read_MB + write_MB
+                rows.setdefault(parts[0], (float(parts[-3]) + float(parts[-2])) * 1e6)       # read_MB + write_MB; a kernel's first row is its largest dispatch shape
             except ValueError:
                 pass
     out = {}
     for stage, kern in TRAFFIC_KERNELS.items():
         for name, val in rows.items():
             if name.split("<")[0] == "llsa::" + kern or name.startswith("llsa::" + kern + "<"):
-                out.setdefault(stage, val)        # (the first row of a kernel is its largest dispatch shape)
+                out.setdefault(stage, val)
     return out, os.path.relpath(path, ROOT)
 
 

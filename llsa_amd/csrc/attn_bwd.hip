@@ -1220,11 +1220,12 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
     LLSA_REQUIRE(fold || a->freq_dk == nullptr, "attn_bwd: freq_dk needs fold_pooled");
 
     const int stages = a->stages ? a->stages : (0x7fffffff & ~LLSA_BWD_NO_REDUCE);
-    if (stages & LLSA_BWD_DQ)
+    if (stages & LLSA_BWD_DQ) {
         if (a->T <= kPairMaxTopk && N1 % 8 == 0)
             hipLaunchKernelGGL(attn_dq_pair_kernel, dim3(N1 / 8, BH), dim3(256), 0, s, *a, delta, dor);
         else
             hipLaunchKernelGGL(attn_dq_kernel, dim3((N1 + 3) / 4, BH), dim3(256), 0, s, *a, delta, dor);
+    }
 
     ReduceParams rp;
     rp.n_jobs = 0;

@@ -119,6 +119,10 @@ def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_wei
     else:
         off, flat, work = transpose_indices(idx, N // BLOCK, CHUNK_FINE)
         if levels == 2:
+            # A row that names a block twice would give both entries one inverse position and leave another slot of the
+            # segment unwritten (the kernels assume what a top-k guarantees): a caller's own p_indices are checked.
+            if T2 > 1 and bool((pidx.sort(-1).values.diff(dim=-1) == 0).any()):
+                raise ValueError("p_indices: a row names a block twice")
             poff, _, pinv = transpose_indices(pidx, N // (BLOCK * BLOCK), inverse=True)
     mk = lambda t: torch.empty_like(t) if rows_ok8(t) else torch.empty(t.shape, device=t.device, dtype=t.dtype)
     dq, dk, dv = mk(q), mk(k), mk(v)

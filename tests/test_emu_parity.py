@@ -104,3 +104,18 @@ def test_sparse_dout_enumeration_two_levels():
     """The element-wise dK / dV check that the GPU suite runs at three and four levels, at two levels and N = 16384 here
     (where the whole-tensor oracle agrees too: test_op_l2_fused_rope): the enumeration itself is what this pins."""
     P.check_op_lk_sparse_dout(DEV, N=16384, topks=(8, 4), H=1, query_blocks=(0, 517, -1), rope=True)
+
+
+def test_unfused_backward_rejects_a_repeated_parent():
+    """A caller's own p_indices that name a block twice in a row are an error, not a wrong gradient."""
+    from llsa_amd.kernel.hip import _attention as A
+    B, H, N = 1, 1, 16384
+    g = torch.Generator().manual_seed(3)
+    q, k, v, do, o = (torch.randn(B, H, N, 64, generator=g).bfloat16() for _ in range(5))
+    pk, pv = (torch.randn(B, H, N // 16, 64, generator=g).bfloat16() for _ in range(2))
+    pk2, pv2 = (torch.randn(B, H, N // 256, 64, generator=g).bfloat16() for _ in range(2))
+    lse = torch.zeros(B, H, N)
+    idx = torch.arange(8).expand(B, H, N // 16, 8).contiguous()
+    pidx = torch.tensor([0, 1, 2, 2]).expand(B, H, N // 256, 4).contiguous()
+    with pytest.raises(ValueError, match="names a block twice"):
+        A.attn_bwd(do, q, k, v, pk, pv, o, lse, idx, 16.0, 16.0, pk2=pk2, pv2=pv2, p_indices=pidx, token_weight_2=256.0)
