@@ -10,7 +10,8 @@ applied in-kernel, smooth-field inputs, dO ~ N(0,1).
 
 One JSON line is printed:
   value        effective TFLOP/s = 14*B*H*N*D*n_kv / step time (algorithmic FLOPs: forward 4, backward 10)
-  ms_per_step  forward + backward wall time per step (K steps between two synchronisations)
+  ms_per_step  forward + backward wall time per step (K steps between two synchronisations; before the W warm-up
+               steps the step runs untimed for a quarter of a second so that clocks and caches have settled)
   step_event_times  median and 20 % / 80 % quantiles of per-step HIP-event times (>= 50 steps), the statistics
                the reference's harness reports
   roofline     the slowest MFMA kernel of the step, timed with HIP events on the launch stream in a
@@ -22,6 +23,8 @@ One JSON line is printed:
   kernels      per-stage times of that second pass (ms), with the achieved rate of each (TFLOP/s on
                algorithmic FLOPs for the attention kernels, GB/s on algorithmic bytes for the others)
   dense_sdpa   F.scaled_dot_product_attention forward+backward on the same shapes, same GPU
+  other_workloads  (default workload only) the two other sizes the target names, three steps each: llsa_l2 against
+               dense SDPA at B=1, H=6, N=65536, and llsa_l2 at B=1, H=6, N=262144
 
 --workload c4 times something else, one training step of the operator's caller (a pixel DiT-S with
 llsa_l2 in its 12 attention layers, batch 8 of 3x128x128, bf16 autocast, AdamW), and prints a line
