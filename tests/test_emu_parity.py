@@ -69,6 +69,8 @@ def test_transpose():
     P.check_transpose(DEV, B=1, H=2, Mb=4096, T=16, chunk=64)        # 65536 entries: the split form
     P.check_transpose_hot_block(DEV)
     P.check_transpose_levels(DEV, B=1, H=2, sizes=((256, 8), (16, 4)))
+    P.check_transpose(DEV, B=1, H=1, Mb=40, T=4, Kb=2048, chunk=2)   # more key blocks than threads
+    P.check_transpose(DEV, B=1, H=1, Mb=200, T=12, Kb=200)           # a last word that is not full
 
 
 def test_attn_l1():

@@ -86,6 +86,8 @@ def test_transpose(dev):
     P.check_transpose(dev, B=1, H=1, Mb=64, T=4, Kb=16)
     P.check_transpose_hot_block(dev)
     P.check_transpose_levels(dev)                                    # two levels, one launch
+    P.check_transpose(dev, B=1, H=2, Mb=64, T=8, Kb=8192, chunk=4)   # more key blocks than threads, two words a row
+    P.check_transpose(dev, B=1, H=1, Mb=1000, T=12, Kb=1000)         # a last word that is not full, topk not a power of two
     P.check_transpose_levels(dev, B=1, H=2, sizes=((256, 16),))
 
 
