@@ -782,7 +782,8 @@ struct GroupSeg {
     const int* sel;                               // (BH, n_groups >> owner_shift, cnt) blocks selected by the group's ancestor;
                                                   // nullptr: blocks 0..cnt-1 (dense level)
     const int* inv;                               // (BH, n_groups >> owner_shift, cnt) position of each entry in the transposed selection
-    bf16x4* part;                                 // partial sums, in the accumulator layout of part_slot but rounded to bf16: the
+    bf16x8* part;                                 // partial sums, the accumulators of part_slot rounded to bf16, two registers (16 bytes)
+                                                  // per lane side by side: slot = [4 register pairs][64 lanes] bf16x8.  The
                                                   // group-major pass writes one per (group, key block), 8 KB each in fp32, which at
                                                   // 16384 tokens is more memory traffic than everything else the pass moves; a group's
                                                   // sum over its 256 queries is taken in fp32 and rounded once (2^-9 relative), and the
@@ -802,7 +803,7 @@ struct GroupStats { f32x4 l[2], d[2]; };
 
 // UPW key blocks against the group's 16 query blocks, two query blocks per step, operands out of LDS.
 template <int UPW>
-__device__ __forceinline__ void group_pass(const bf16x8 (&bk)[2][2], const bf16x8 (&bv)[2][2], const float (&w)[2], bf16x4* const (&dst)[2],
+__device__ __forceinline__ void group_pass(const bf16x8 (&bk)[2][2], const bf16x8 (&bv)[2][2], const float (&w)[2], bf16x8* const (&dst)[2],
                                            const bf16* shq, const bf16* shg, const float* lseb, const float* dlb, int lane) {
     const int quad = lane >> 4;
     f32x4 dk[UPW][4], dv[UPW][4];
@@ -880,9 +881,9 @@ __device__ __forceinline__ void group_pass(const bf16x8 (&bk)[2][2], const bf16x
 #pragma unroll
     for (int j = 0; j < UPW; j++)
 #pragma unroll
-        for (int dt = 0; dt < 4; dt++) {
-            dst[j][dt * kWave + lane] = cvt4(dk[j][dt] * w[j]);
-            dst[j][(4 + dt) * kWave + lane] = cvt4(dv[j][dt] * w[j]);
+        for (int pr = 0; pr < 2; pr++) {                      // registers 2 pr, 2 pr + 1 of dK, then of dV: 16 bytes a lane and store
+            dst[j][pr * kWave + lane] = cat(cvt4(dk[j][2 * pr] * w[j]), cvt4(dk[j][2 * pr + 1] * w[j]));
+            dst[j][(2 + pr) * kWave + lane] = cat(cvt4(dv[j][2 * pr] * w[j]), cvt4(dv[j][2 * pr + 1] * w[j]));
         }
 }
 
@@ -938,7 +939,7 @@ __global__ __launch_bounds__(64 * kGroupWaves, 2) void attn_kside_group_kernel(G
 
     bf16x8 bk[2][2], bv[2][2];
     float w[2];
-    bf16x4* dst[2];
+    bf16x8* dst[2];
     auto fetch = [&](int j, int u) __attribute__((always_inline)) {    // K, V tiles of key block j into register set u
         const int sgi = __builtin_amdgcn_readlane(my_seg, j);
         const int unit = __builtin_amdgcn_readlane(my_unit, j);
@@ -951,7 +952,7 @@ __global__ __launch_bounds__(64 * kGroupWaves, 2) void attn_kside_group_kernel(G
         bv[u][0] = ld16(vp);
         bv[u][1] = ld16(vp + 512);
         w[u] = sg.w;
-        dst[u] = sg.part + (((int64_t)(unsigned)slo) | ((int64_t)shi << 32)) * (8 * kWave);
+        dst[u] = sg.part + (((int64_t)(unsigned)slo) | ((int64_t)shi << 32)) * (4 * kWave);
     };
     if (lo < hi) fetch(lo, 0);
     if (lo + 1 < hi) fetch(lo + 1, 1);
@@ -1001,17 +1002,14 @@ __host__ __device__ inline int reduce_slots(int max_units) {
 }
 
 __global__ __launch_bounds__(256) void kside_reduce_kernel(ReduceParams rp) {
-    // Two workgroups per unit; every thread owns one f32x4 of the unit's 8 x 64 accumulator
-    // registers and streams that position of all partials, sixteen loads in flight.  Every job has
-    // its own range of workgroup pairs (reduce_slots of them), which walk the job's units with that
-    // stride: the number of units with several pieces is known only on the device and usually
-    // small, and a grid sized for the worst case would be mostly workgroups that start, look and leave.
+    // fp32 partial sums: two workgroups per unit; every thread owns one f32x4 of the unit's 8 x 64 accumulator
+    // registers and streams that position of all partials, sixteen loads in flight.  bf16 partial sums (the group-major
+    // pass): one workgroup per unit, every thread owns a pair of registers (16 bytes a partial, like the fp32 loads), and
+    // the two workgroups of a position take alternate units.  Every job has its own range of workgroup pairs
+    // (reduce_slots of them), which walk the job's units with that stride: the number of units with several pieces is
+    // known only on the device and usually small, and a grid sized for the worst case would be mostly workgroups that
+    // start, look and leave.
     const int bh = blockIdx.y, b = bh / rp.H, h = bh % rp.H;
-    const int pos = (blockIdx.x & 1) * 256 + threadIdx.x;
-    const int reg = pos >> 6, lane = pos & 63;
-    const int r = lane & 15, quad = lane >> 4;
-    const int dt = reg & 3;
-    const int which = reg >> 2;                               // 0: dK, 1: dV
     int u0 = blockIdx.x >> 1, j = 0;
     while (j < rp.n_jobs && u0 >= reduce_slots(rp.job[j].max_units)) {
         u0 -= reduce_slots(rp.job[j].max_units);
@@ -1019,7 +1017,14 @@ __global__ __launch_bounds__(256) void kside_reduce_kernel(ReduceParams rp) {
     }
     if (j >= rp.n_jobs) return;
     const ReduceJob& jb = rp.job[j];
-    const int step = reduce_slots(jb.max_units);
+    const int half = jb.half_part;
+    const int pos = half ? (int)threadIdx.x : (int)((blockIdx.x & 1) * 256 + threadIdx.x);
+    const int reg = half ? 2 * (pos >> 6) : (pos >> 6), lane = pos & 63;     // (half: registers reg, reg + 1)
+    const int r = lane & 15, quad = lane >> 4;
+    const int dt = reg & 3;
+    const int which = reg >> 2;                               // 0: dK, 1: dV
+    const int step = reduce_slots(jb.max_units) * (half ? 2 : 1);
+    if (half) u0 = 2 * u0 + (int)(blockIdx.x & 1);
     const int* work = jb.work ? jb.work + (int64_t)bh * jb.work_stride : nullptr;
     const int max_items = (int)(jb.work_stride - work_tail_len(jb.n_units) - 4 - 4 * jb.max_units) / 4;
     // the unit's record is fetched together with the count it is checked against (u0 is always
@@ -1058,20 +1063,22 @@ __global__ __launch_bounds__(256) void kside_reduce_kernel(ReduceParams rp) {
             first = (int64_t)bh * jb.n_units + unit;
             stride = (int64_t)gridDim.y * jb.n_units;
         }
-        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-        const int64_t at = first * (8 * kWave) + reg * kWave + lane;
-        if (jb.half_part) {
-            const bf16x4* ps = reinterpret_cast<const bf16x4*>(jb.part) + at;
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f}, acc2 = {0.f, 0.f, 0.f, 0.f};
+        if (half) {
+            const bf16x8* ps = reinterpret_cast<const bf16x8*>(jb.part) + first * (4 * kWave) + (reg >> 1) * kWave + lane;
             for (int c0 = 0; c0 < n; c0 += 16) {
-                bf16x4 v[16];
+                bf16x8 v[16];
 #pragma unroll
-                for (int k = 0; k < 16; k++) v[k] = ps[(int64_t)min(c0 + k, n - 1) * stride * (8 * kWave)];
+                for (int k = 0; k < 16; k++) v[k] = ps[(int64_t)min(c0 + k, n - 1) * stride * (4 * kWave)];
 #pragma unroll
                 for (int k = 0; k < 16; k++)
-                    if (c0 + k < n) acc += f32x4{(float)v[k][0], (float)v[k][1], (float)v[k][2], (float)v[k][3]};
+                    if (c0 + k < n) {
+                        acc += f32x4{(float)v[k][0], (float)v[k][1], (float)v[k][2], (float)v[k][3]};
+                        acc2 += f32x4{(float)v[k][4], (float)v[k][5], (float)v[k][6], (float)v[k][7]};
+                    }
             }
         } else {
-            const f32x4* ps = jb.part + at;
+            const f32x4* ps = jb.part + first * (8 * kWave) + reg * kWave + lane;
             for (int c0 = 0; c0 < n; c0 += 16) {
                 f32x4 v[16];
 #pragma unroll
@@ -1081,12 +1088,13 @@ __global__ __launch_bounds__(256) void kside_reduce_kernel(ReduceParams rp) {
                     if (c0 + k < n) acc += v[k];               // chunk order: the sum does not depend on scheduling
             }
         }
+        bf16* dst = which ? jb.dv + b * jb.sdvb + h * jb.sdvh + (int64_t)(unit * kBlk + r) * jb.sdvn
+                          : jb.dk + b * jb.sdkb + h * jb.sdkh + (int64_t)(unit * kBlk + r) * jb.sdkn;
         bf16x4 out = cvt4(which ? acc : acc * kScale);
         if (jb.fold.depth > 0)
             out = fold_pooled(out, jb.fold, which, bh, rp.N, unit * kBlk + r, dt * 16 + quad * 4);
-        bf16* dst = which ? jb.dv + b * jb.sdvb + h * jb.sdvh + (int64_t)(unit * kBlk + r) * jb.sdvn
-                          : jb.dk + b * jb.sdkb + h * jb.sdkh + (int64_t)(unit * kBlk + r) * jb.sdkn;
         st8(dst + quad * 4 + dt * 16, out);
+        if (half) st8(dst + quad * 4 + (dt + 1) * 16, cvt4(which ? acc2 : acc2 * kScale));      // (no fold on these jobs)
     }
 }
 
@@ -1296,7 +1304,7 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
                            int cnt, int64_t slots, float w) {
             GroupSeg& sgm = g.seg[g.n_segs++];
             sgm.kk = (const bf16*)kk; sgm.vv = (const bf16*)vv; sgm.sel = sel; sgm.inv = inv;
-            sgm.part = (bf16x4*)(ws + part_off); sgm.n_units = n_units; sgm.owner_shift = shift; sgm.cnt = cnt; sgm.slots = slots; sgm.w = w;
+            sgm.part = (bf16x8*)(ws + part_off); sgm.n_units = n_units; sgm.owner_shift = shift; sgm.cnt = cnt; sgm.slots = slots; sgm.w = w;
             g.n_blocks += cnt;
         };
         for (int l = 1; l < L; l++) {                         // level l: blocks N / 16^(l+1), one list per 16^(l-1) groups
