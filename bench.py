@@ -116,7 +116,7 @@ def stage_profile(op, q, k, v, do, t1, t2, freq, iters, torch):
     """Runs the kernels of one forward + backward one stage at a time, the same launches the
     fused operator makes, and times each stage with events on the launch stream."""
     from llsa_amd.kernel.hip import _attention as A
-    from llsa_amd._lib import CHUNK_FINE
+    from llsa_amd._lib import current_lib as _cur
     from llsa_amd.kernel.hip.indices_transpose import transpose_indices_levels
     from llsa_amd.kernel.hip.mean_pool import PoolSpec, pool_pyramid
     from llsa_amd.kernel.hip.topk import compute_topk_indices_sparse, gen_sparse_indices
@@ -159,7 +159,7 @@ def stage_profile(op, q, k, v, do, t1, t2, freq, iters, torch):
     res["attn_fwd"] = timed(lambda: A.attn_fwd(q, k, v, pk, pv, idx, 16.0, tiles=tiles, **kw), iters, torch)
 
     def transposes():          # all levels with one call, as the operator does it
-        r = transpose_indices_levels([idx, pidx] if l2 else [idx], CHUNK_FINE)
+        r = transpose_indices_levels([idx, pidx] if l2 else [idx], _cur().fine_chunk(N))
         return r[0] + r[1] if l2 else r[0]
 
     csr = transposes()

@@ -44,7 +44,7 @@ extern "C" {
 #define LLSA_DTYPE_BF16 0
 #define LLSA_DTYPE_F32 1
 
-#define LLSA_ABI_VERSION 202     /* changes with every change of a signature or argument structure below */
+#define LLSA_ABI_VERSION 203     /* changes with every change of a signature or argument structure below */
 int llsa_version(void);          /* LLSA_ABI_VERSION of the built library                                    */
 const char* llsa_last_error_string(void);
 
@@ -236,7 +236,7 @@ int llsa_transpose_indices_multi(const llsa_transpose_job* jobs, int n_jobs, int
  * per chunk, so that a key block selected by very many query blocks is spread over many waves
  * (the reference walks each segment serially, sparse_attention_res_1.py:300-322).  `work` is
  * (B,H,llsa_work_list_len(Mb,Kb,T,chunk)) int32, 16-byte aligned; llsa_attn_bwd needs the
- * work list of idx with chunk = LLSA_CHUNK_FINE (the pooled levels need none).  Per (b,h), in int32:
+ * work list of idx with chunk = llsa_fine_chunk(N) (the pooled levels need none).  Per (b,h), in int32:
  *   [0] items, [1] partial-sum slots, [2] key blocks with more than one chunk, [3] 0
  *   [4 + 4i ..]              item i = {key block, first entry in flat, entries, partial-sum slot or -1};
  *                            items with more than chunk/2 entries come first
@@ -244,7 +244,12 @@ int llsa_transpose_indices_multi(const llsa_transpose_job* jobs, int n_jobs, int
  *   then Kb ints (rounded up to a multiple of 4) that the transpose itself uses as scratch
  * with max_items = Mb*T/chunk + Kb; every key block has at least one item. */
 int64_t llsa_work_list_len(int Mb, int Kb, int T, int chunk);
-#define LLSA_CHUNK_FINE 64
+/* Entries per work item of the fine level for a sequence of N tokens: 64 up to N = 16384, where a step is short and a long
+ * item would end it alone, 256 beyond, where fewer items and fewer partial sums count for more (N = 65536: -2 %,
+ * N = 262144: -3 % of the step).  Never more than LLSA_CHUNK_FINE_MAX.  No counterpart in the reference, which walks a key
+ * block's whole list in one program (sparse_attention_res_1.py:300-322). */
+int llsa_fine_chunk(int N);
+#define LLSA_CHUNK_FINE_MAX 256
 
 /* ------------------------------------------------------------------------------------------
  * Backward.  Replaces sparse_indices_attn_res_scatter_bwd_v2 (sparse_attention_res_1.py:403-471)

@@ -94,13 +94,14 @@ _SIGNATURES = {
     "llsa_transpose_indices": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "llsa_transpose_indices_multi": (c_int, [C.POINTER(TransposeJob), c_int, c_int, c_int, c_void_p]),
     "llsa_work_list_len": (c_int64, [c_int, c_int, c_int, c_int]),
+    "llsa_fine_chunk": (c_int, [c_int]),
     "llsa_attn_bwd_workspace_bytes": (c_int64, [c_int, c_int, c_int, C.POINTER(c_int32), c_int]),
     "llsa_attn_bwd": (c_int, [C.POINTER(AttnBwdArgs), c_void_p]),
 }
 
 EXPORTS = tuple(_SIGNATURES)
-CHUNK_FINE = 64                                             # LLSA_CHUNK_FINE of include/llsa_hip.h
-ABI_VERSION = 202                                           # LLSA_ABI_VERSION
+CHUNK_FINE_MAX = 256                                        # LLSA_CHUNK_FINE_MAX of include/llsa_hip.h
+ABI_VERSION = 203                                           # LLSA_ABI_VERSION
 STATIC_PARTIALS_MAX = 262144                                # LLSA_STATIC_PARTIALS_MAX
 
 

@@ -451,7 +451,7 @@ __device__ __forceinline__ void kside_pair(f32x4 dk[4], f32x4 dv[4], const bf16x
 // accumulator layout: 8 f32x4 registers per lane (4 channel tiles of dK, then 4 of dV).
 __device__ __forceinline__ f32x4* part_slot(f32x4* part, int64_t slot) { return part + slot * (8 * kWave); }
 
-// One work item of the fine pass: a key block and a piece (at most LLSA_CHUNK_FINE entries) of its list.
+// One work item of the fine pass: a key block and a piece (at most fine_chunk(N) <= LLSA_CHUNK_FINE_MAX entries) of its list.
 // One wave = one workgroup per item (items differ a lot in length; a wave that shared its workgroup
 // with a longer one would keep its registers and LDS allocated while idle).
 __global__ __launch_bounds__(64) void attn_kside_kernel(KSideParams p) {
@@ -505,10 +505,21 @@ __global__ __launch_bounds__(64) void attn_kside_kernel(KSideParams p) {
             copy16_global_to_lds(fr + 512 + lane * 8, fold_buf + kFoldRows + 512);
         }
     }
-    // The item's list entries (at most 64 query blocks) are fetched once, entry i into lane i, and
-    // handed out with readlane: the walk below then has no load that depends on a load.
-    const int mine = (lane < cnt) ? fl[start + lane] : 0;
-    auto entry = [&](int i) -> int { return clampi(__builtin_amdgcn_readlane(mine, i), 0, N1 - 1); };   // i is wave-uniform
+    // The item's list entries (at most LLSA_CHUNK_FINE_MAX query blocks) are fetched once, entry i into lane i % 64 of
+    // register i / 64, and handed out with readlane: the walk below then has no load that depends on a load.
+    constexpr int kEntryRegs = LLSA_CHUNK_FINE_MAX / kWave;
+    int mine[kEntryRegs];
+#pragma unroll
+    for (int k = 0; k < kEntryRegs; k++) mine[k] = (k * kWave + lane < cnt) ? fl[start + k * kWave + lane] : 0;
+    auto entry = [&](int i) -> int {                          // i is wave-uniform
+        int v = __builtin_amdgcn_readlane(mine[0], i & (kWave - 1));
+#pragma unroll
+        for (int k = 1; k < kEntryRegs; k++) {
+            const int o = __builtin_amdgcn_readlane(mine[k], i & (kWave - 1));
+            v = ((i >> 6) == k) ? o : v;
+        }
+        return clampi(v, 0, N1 - 1);
+    };
 
     f32x4 dk[4], dv[4];
 #pragma unroll
@@ -1151,7 +1162,7 @@ static BwdWorkspace bwd_workspace(int B, int H, int N, const int32_t* topk, int 
     BwdWorkspace w;
     // a key block has several chunks only if it has more than `chunk` entries, so at most
     // E/chunk such blocks with at most E/chunk + E/chunk chunks in total
-    w.slots_fine = 2 * (N1 * topk[0] / LLSA_CHUNK_FINE) + 2;
+    w.slots_fine = 2 * (N1 * topk[0] / fine_chunk(N)) + 2;
     int64_t o = 0;
     w.delta = o;        o += align256(BH * N * 4);
     w.dor = o;          o += align256(BH * N * 64 * 2);
@@ -1277,7 +1288,8 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
         KSideParams p = base;
         p.kk = (const bf16*)a->kr; p.vv = (const bf16*)a->vr;
         p.off = a->off; p.flat = a->flat; p.flat_stride = (int64_t)N1 * a->T;
-        p.work = a->work; p.work_stride = llsa_work_list_len(N1, N1, a->T, LLSA_CHUNK_FINE);
+        const int chunk = fine_chunk(N);
+        p.work = a->work; p.work_stride = llsa_work_list_len(N1, N1, a->T, chunk);
         p.part = (f32x4*)(ws + wsp.part_fine); p.slot_stride = wsp.slots_fine;
         p.dk = (bf16*)a->dk; p.sdkb = a->sdkb; p.sdkh = a->sdkh; p.sdkn = a->sdkn;
         p.dv = (bf16*)a->dv; p.sdvb = a->sdvb; p.sdvh = a->sdvh; p.sdvn = a->sdvn;
@@ -1290,9 +1302,9 @@ extern "C" int llsa_attn_bwd(const llsa_attn_bwd_args* a, void* stream) {
             p.fold.freq = (const bf16*)a->freq_dk;
             p.fold.depth = L;
         }
-        const int max_items = N1 * a->T / LLSA_CHUNK_FINE + N1;
+        const int max_items = N1 * a->T / chunk + N1;
         hipLaunchKernelGGL(attn_kside_kernel, dim3(max_items, BH), dim3(64), 0, s, p);
-        add_job(p, LLSA_CHUNK_FINE, N1 * a->T / LLSA_CHUNK_FINE + 1, 0);
+        add_job(p, chunk, N1 * a->T / chunk + 1, 0);
     };
     // pooled levels under an ancestor's selection, group-major (one launch for all of them, plus the dense level when it is small)
     auto run_groups = [&]() {

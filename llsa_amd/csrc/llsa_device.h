@@ -144,6 +144,7 @@ __device__ __forceinline__ bf16x4 rope_bwd4(bf16x4 o, bf16x4 f) {
 // ints at the end of a (b,h)'s work list (see transpose.hip) that the transpose of many entries uses as
 // histogram, then as cursors
 __host__ __device__ inline int work_tail_len(int Kb) { return (Kb + 3) & ~3; }
+__host__ __device__ inline int fine_chunk(int N) { return N > 16384 ? 256 : 64; }      // llsa_fine_chunk
 
 constexpr int kGroup = 4;      // pooled blocks per LDS buffer in the query-side attention kernels (one per wave)
 

@@ -427,6 +427,8 @@ __global__ __launch_bounds__(256) void inverse_positions_kernel(const int* __res
 
 using namespace llsa;
 
+extern "C" int llsa_fine_chunk(int N) { return fine_chunk(N); }
+
 extern "C" int64_t llsa_work_list_len(int Mb, int Kb, int T, int chunk) {
     if (Mb <= 0 || Kb <= 0 || T <= 0 || chunk <= 0) return -1;
     const int64_t e = (int64_t)Mb * T;

@@ -6,7 +6,7 @@ from typing import Optional
 
 import torch
 
-from ..._lib import CHUNK_FINE, AttnBwdArgs, AttnFwdArgs
+from ..._lib import AttnBwdArgs, AttnFwdArgs
 from ._common import BLOCK, as_rows, lib_for, ptr, require_bf16, require_head_dim, s3, stream_of
 from .indices_transpose import transpose_indices
 
@@ -117,7 +117,7 @@ def attn_bwd(do, q, k, v, pk, pv, o, lse, indices, token_weight, coarse_grad_wei
         if levels == 2:
             poff, _, pinv = csr[3:6]
     else:
-        off, flat, work = transpose_indices(idx, N // BLOCK, CHUNK_FINE)
+        off, flat, work = transpose_indices(idx, N // BLOCK, lib.fine_chunk(N))
         if levels == 2:
             # A row that names a block twice would give both entries one inverse position and leave another slot of the
             # segment unwritten (the kernels assume what a top-k guarantees): a caller's own p_indices are checked.

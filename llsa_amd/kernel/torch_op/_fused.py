@@ -21,7 +21,7 @@ import ctypes as C
 import torch
 from torch.autograd import Function
 
-from ..._lib import CHUNK_FINE, MAX_LEVELS, AttnBwdArgs, AttnFwdArgs, PoolItem, TransposeJob, current_lib
+from ..._lib import MAX_LEVELS, AttnBwdArgs, AttnFwdArgs, PoolItem, TransposeJob, current_lib
 
 _side = {}          # device -> second stream
 _SIDE_STREAM_MIN_TOKENS = 1 << 17
@@ -76,7 +76,8 @@ class _Layout:
             o = _align(o + BH * per_bh, 64)
             return at
 
-        self.wl_f = lib.work_list_len(n[1], n[1], topks[0], CHUNK_FINE)
+        self.chunk = lib.fine_chunk(N)          # entries per work item of the fine level
+        self.wl_f = lib.work_list_len(n[1], n[1], topks[0], self.chunk)
         # sel[0] = idx (fine blocks per query block), sel[l] = blocks of level l per group of 16^(l+1) queries
         self.sel = [take_i(n[l + 1] * topks[l]) for l in range(L)]
         self.off = [take_i(n[l + 1] + 1, grad) for l in range(L)]
@@ -224,7 +225,7 @@ class LlsaFused(Function):
         # which the event calls cost more than the GPU saves: everything then goes to the one stream.
         jobs = (TransposeJob * L)()
         if grad:
-            jobs[0] = TransposeJob(pi(lay.sel[0]), pi(lay.off[0]), pi(lay.flat[0]), pi(lay.work), None, n[1], n[1], topks[0], CHUNK_FINE)
+            jobs[0] = TransposeJob(pi(lay.sel[0]), pi(lay.off[0]), pi(lay.flat[0]), pi(lay.work), None, n[1], n[1], topks[0], lay.chunk)
             for l in range(1, L):
                 jobs[l] = TransposeJob(pi(lay.sel[l]), pi(lay.off[l]), pi(lay.flat[l]), None, pi(lay.inv[l]), n[l + 1], n[l + 1], topks[l], 1)
         cur = side = None

@@ -87,6 +87,7 @@ def test_entry_points_reject_bad_arguments(lib):
     assert lib.attn_fwd(C.byref(a), None) != 0
     assert b"must not exceed 56" in lib.last_error_string()
     assert lib.work_list_len(1024, 1024, 16, 32) == 4 + 4 * (512 + 1024) + 4 * 513 + 1024
+    assert lib.fine_chunk(16384) == 64 and lib.fine_chunk(65536) == 256 and lib.fine_chunk(262144) <= 256      # <= LLSA_CHUNK_FINE_MAX
 
 
 def test_python_layer_rejects_unsupported_inputs():

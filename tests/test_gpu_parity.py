@@ -117,6 +117,7 @@ def test_attn_more_than_64_selected(dev):
 def test_attn_hot_blocks(dev):
     P.check_attn_l1(dev, B=1, H=2, N=4096, T=8, hot=5)
     P.check_attn_l2(dev, B=1, H=1, N=16384, T=8, T2=8, hot=3)
+    P.check_attn_l1(dev, B=1, H=1, N=32768, T=4, hot=5)          # beyond 16384 tokens a work item holds up to 256 entries: 8 full ones here
 
 
 def test_attn_special_cases(dev):
