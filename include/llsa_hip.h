@@ -221,9 +221,10 @@ int llsa_transpose_indices(const int32_t* idx, int32_t* offsets, int32_t* flat, 
                            int32_t* inv /* or NULL */, int B, int H, int Mb, int Kb, int T, int chunk, void* stream);
 
 /* The same for several index tensors of one operator call (the selections of all its levels) with as few launches as
- * possible: every job is what one llsa_transpose_indices call takes, all jobs share B and H.  Jobs small enough
- * for one workgroup per (b,h) to hold a bitmap of (key block, query block) in LDS -- roughly Mb * Kb <= 2^20 --
- * are done in ONE launch together, already sorted; the others go job by job.  It has no counterpart of its own in
+ * possible: every job is what one llsa_transpose_indices call takes, all jobs share B and H.  When every job is small
+ * enough for a workgroup to hold a bitmap of (key block, query block) in LDS -- roughly Mb * Kb <= 2^20 -- all of them
+ * are done in ONE launch, already sorted; otherwise the large ones go job by job, as llsa_transpose_indices does them,
+ * and so do the small ones whose bitmaps are more than 32 KB.  It has no counterpart of its own in
  * the reference, which calls transpose_indices once per index tensor (sparse_attention_res_2.py:593-594). */
 typedef struct llsa_transpose_job {
     const int32_t* idx; int32_t* offsets; int32_t* flat; int32_t* work /* or NULL */; int32_t* inv /* or NULL */;

@@ -503,22 +503,33 @@ static int transpose_general(const int32_t* idx, int32_t* offsets, int32_t* flat
 
 extern "C" int llsa_transpose_indices_multi(const llsa_transpose_job* jobs, int n_jobs, int B, int H, void* stream) {
     LLSA_REQUIRE(jobs != nullptr && n_jobs >= 1 && n_jobs <= LLSA_MAX_LEVELS, "transpose_indices: 1..%d jobs, got %d", LLSA_MAX_LEVELS, n_jobs);
-    TrJobs small;
-    int n_small = 0;
+    // One launch when the bitmaps of every job fit.  Beside a job that is too large for that, a small job shares the
+    // launch of the small ones only while its bitmaps are light (32 KB): a workgroup that wants most of a CU's LDS waits
+    // for a CU to drain when it runs next to the large job's kernels -- or next to an attention kernel on another
+    // stream, which is where a caller with large jobs runs this (0.6 ms instead of 16 us for the level-1 selection of
+    // 262144 tokens beside the forward kernel) -- so such a job takes the kernels for large jobs too.
+    bool all_fit = true;
     for (int i = 0; i < n_jobs; i++) {
         const llsa_transpose_job& j = jobs[i];
         const int rc = check_transpose_job(j.idx, j.offsets, j.flat, j.work, B, H, j.Mb, j.Kb, j.T, j.chunk);
         if (rc != 0) return rc;
+        all_fit = all_fit && tr_bitmap_lds_ints(j.Mb, j.Kb) <= kTrBitmapMaxInts;
+    }
+    constexpr int64_t kLightInts = 8 * 1024;
+    TrJobs small;
+    int n_small = 0;
+    for (int i = 0; i < n_jobs; i++) {
+        const llsa_transpose_job& j = jobs[i];
         const int chunk = j.chunk < 1 ? 1 : j.chunk;
-        if (tr_bitmap_lds_ints(j.Mb, j.Kb) <= kTrBitmapMaxInts) {
+        if (tr_bitmap_lds_ints(j.Mb, j.Kb) <= (all_fit ? kTrBitmapMaxInts : kLightInts)) {
             TrJob& t = small.job[n_small++];
             t.idx = j.idx; t.offsets = j.offsets; t.flat = j.flat; t.work = j.work; t.inv = j.inv;
             t.Mb = j.Mb; t.Kb = j.Kb; t.T = j.T; t.chunk = chunk;
             t.work_stride = j.work ? (int)llsa_work_list_len(j.Mb, j.Kb, j.T, chunk) : 0;
             t.parts = std::min(8, std::max(1, j.Kb / 128));
         } else {
-            const int rc2 = transpose_general(j.idx, j.offsets, j.flat, j.work, j.inv, B, H, j.Mb, j.Kb, j.T, chunk, stream);
-            if (rc2 != 0) return rc2;
+            const int rc = transpose_general(j.idx, j.offsets, j.flat, j.work, j.inv, B, H, j.Mb, j.Kb, j.T, chunk, stream);
+            if (rc != 0) return rc;
         }
     }
     if (n_small > 0) return launch_bitmap_jobs(small, n_small, B, H, (hipStream_t)stream);
