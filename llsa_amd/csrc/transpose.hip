@@ -259,12 +259,10 @@ __global__ __launch_bounds__(kTrThreads) void transpose_bitmap_kernel(TrJobs job
         bm[n * stride + words] = (unsigned)c;
     }
     __syncthreads();
-    const int my_end = offsets_and_work_list([&](int i) { return (int)bm[i * stride + words]; },
-                                             [&](int i, int st) { bm[i * stride + words] = (unsigned)st; },      // the count gives way to the start
-                                             wave_tot, offsets, work, Kb, E, E, jb.chunk, part == 0);
-    __syncthreads();                                          // (everybody has read the wave totals)
-    if (tid == kTrThreads - 1) wave_tot[0] = my_end;          // the end of the last segment
-    __syncthreads();
+    offsets_and_work_list([&](int i) { return (int)bm[i * stride + words]; },
+                          [&](int i, int st) { bm[i * stride + words] = (unsigned)st; },      // the count gives way to the start
+                          wave_tot, offsets, work, Kb, E, E, jb.chunk, part == 0);
+    __syncthreads();                                          // (every row's start is in place)
     if (jb.inv != nullptr) {
         int* inv = jb.inv + (int64_t)bh * E;
         for (int e = part * kTrThreads + tid; e < E; e += jb.parts * kTrThreads) {
