@@ -23,7 +23,7 @@ One JSON line is printed:
   kernels      per-stage times of that second pass (ms), with the achieved rate of each (TFLOP/s on
                algorithmic FLOPs for the attention kernels, GB/s on algorithmic bytes for the others)
   dense_sdpa   F.scaled_dot_product_attention forward+backward on the same shapes, same GPU
-  other_workloads  (default workload only) the two other sizes the target names, three steps each: llsa_l2 against
+  other_workloads  (default workload only) the two other sizes the target names, 20 steps each: llsa_l2 against
                dense SDPA at B=1, H=6, N=65536, and llsa_l2 at B=1, H=6, N=262144
 
 --workload c4 times something else, one training step of the operator's caller (a pixel DiT-S with
@@ -187,7 +187,8 @@ def stage_profile(op, q, k, v, do, t1, t2, freq, iters, torch):
 
 
 def other_workloads(dev):
-    """The two other sizes the target names, three steps each after two untimed ones (HIP events on the launch stream):
+    """The two other sizes the target names, 20 steps each after 10 untimed ones (HIP events on the launch stream; three
+    after one for the dense comparison, whose step is 54 ms):
     llsa_l2 forward + backward against dense F.scaled_dot_product_attention at B=1, H=6, N=65536 (the sparse-vs-dense
     comparison), and llsa_l2 at the largest configuration, B=1, H=6, N=262144.  Same generator, seeds and in-kernel
     RoPE as the headline workload; the reference's harness sweeps the same three sizes (test_kernel.py:27-53)."""
@@ -210,11 +211,12 @@ def other_workloads(dev):
             q.grad = k.grad = v.grad = None
             F.scaled_dot_product_attention(q, k, v).backward(do)
 
-        for _ in range(2):
+        n_warm, n_timed = 10, 20           # (the first steps at a new shape are slower: allocator, clocks)
+        for _ in range(n_warm):
             step()
-        ms = timed(step, 3, torch)
+        ms = timed(step, n_timed, torch)
         flops = 14.0 * B * H * N * 64 * n_kv(op, N, t1, t2)
-        e = {"workload": f"llsa_l2 fwd+bwd B={B} H={H} N={N} D=64 topk={t1}/{t2} rope=in-kernel", "steps": 3, "ms_per_step": ms,
+        e = {"workload": f"llsa_l2 fwd+bwd B={B} H={H} N={N} D=64 topk={t1}/{t2} rope=in-kernel", "steps": n_timed, "ms_per_step": ms,
              "tflops": flops / (ms * 1e-3) / 1e12}
         if name == "n65536":
             try:
