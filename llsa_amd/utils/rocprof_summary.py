@@ -44,7 +44,7 @@ tot = sum(r[5] for r in rows)
 steps = [r[1] for r in rows if 'attn_kside_kernel' in r[0]][0]      # one fine K-side launch per step
 with open(f'{out}/step_kernels_{wl}_kernel_trace.txt', 'w') as f:
     f.write(f"Kernel trace of one bench run, workload {wl}: {desc}\n")
-    f.write(f"command (from the repository root, on the MI355X box):\n  rocprofv3 --kernel-trace --stats -d gpurun_out/kt -o t -- {bench} --steps 20 --warmup 5\n")
+    f.write(f"command (from the repository root, on the MI355X box):\n  rocprofv3 --kernel-trace --stats -d prof/kt -o t -- {bench} --steps 20 --warmup 5\n")
     f.write(f"bench line of that run: ms_per_step={j['ms_per_step']:.4f} (under the profiler), value={j['value']:.1f} {j['unit']}\n")
     f.write(f"{steps} steps in the run (a quarter of a second untimed, 5 warm-up, 20 timed, 50 timed one by one with events); per-kernel statistics over all dispatches, durations in microseconds\n\n")
     f.write(f"{'kernel':62s} {'calls':>6s} {'avg_us':>9s} {'min_us':>9s} {'max_us':>9s} {'us/step':>9s} {'pct':>6s}\n")
@@ -68,8 +68,8 @@ w_fac = 262144.0 / wd[copyk]['WRITE_SIZE']
 with open(f'{out}/step_kernels_{wl}_hbm_traffic.txt', 'w') as f:
     f.write(f"HBM-side traffic per dispatch (L2 <-> fabric), workload {wl}: {desc}\n")
     f.write("commands (from the repository root, on the MI355X box), one counter per run:\n")
-    f.write(f"  rocprofv3 --pmc FETCH_SIZE --kernel-trace -d gpurun_out/fetch -o p -- {bench} --steps 5 --warmup 2 --calibrate\n")
-    f.write(f"  rocprofv3 --pmc WRITE_SIZE --kernel-trace -d gpurun_out/write -o p -- {bench} --steps 5 --warmup 2 --calibrate\n")
+    f.write(f"  rocprofv3 --pmc FETCH_SIZE --kernel-trace -d prof/fetch -o p -- {bench} --steps 5 --warmup 2 --calibrate\n")
+    f.write(f"  rocprofv3 --pmc WRITE_SIZE --kernel-trace -d prof/write -o p -- {bench} --steps 5 --warmup 2 --calibrate\n")
     f.write("--calibrate adds a plain elementwise copy of 256 MiB (torch.mul(src, 1.0, out=dst), fp32: reads 262144 KiB, writes 262144 KiB).\n")
     f.write(f"That copy reads FETCH_SIZE={fd[copyk]['FETCH_SIZE']:.0f} KiB and WRITE_SIZE={wd[copyk]['WRITE_SIZE']:.0f} KiB per dispatch, so\n")
     f.write(f"scale factors: fetch x{f_fac:.3f}, write x{w_fac:.3f}.  Values below are averages per dispatch over all dispatches of the kernel.\n\n")
@@ -92,8 +92,8 @@ cd, cdur = counters(f'{raw}/cache/p_results.db')
 with open(f'{out}/step_kernels_{wl}_sq_cache_counters.txt', 'w') as f:
     f.write(f"Wave-scheduler and cache counters per dispatch, workload {wl}: {desc}\n")
     f.write("commands (from the repository root, on the MI355X box):\n")
-    f.write(f"  rocprofv3 --pmc SQ_WAVE_CYCLES SQ_BUSY_CU_CYCLES SQ_ACTIVE_INST_VALU SQ_ACTIVE_INST_SCA SQ_ACTIVE_INST_LDS SQ_WAIT_INST_ANY SQ_VALU_MFMA_BUSY_CYCLES SQ_INSTS_VALU --kernel-trace -d gpurun_out/sq -o p -- {bench} --steps 5 --warmup 2\n")
-    f.write(f"  rocprofv3 --pmc TCC_HIT_sum TCC_MISS_sum TCP_TOTAL_CACHE_ACCESSES_sum TCP_TCC_READ_REQ_sum --kernel-trace -d gpurun_out/cache -o p -- {bench} --steps 5 --warmup 2\n")
+    f.write(f"  rocprofv3 --pmc SQ_WAVE_CYCLES SQ_BUSY_CU_CYCLES SQ_ACTIVE_INST_VALU SQ_ACTIVE_INST_SCA SQ_ACTIVE_INST_LDS SQ_WAIT_INST_ANY SQ_VALU_MFMA_BUSY_CYCLES SQ_INSTS_VALU --kernel-trace -d prof/sq -o p -- {bench} --steps 5 --warmup 2\n")
+    f.write(f"  rocprofv3 --pmc TCC_HIT_sum TCC_MISS_sum TCP_TOTAL_CACHE_ACCESSES_sum TCP_TCC_READ_REQ_sum --kernel-trace -d prof/cache -o p -- {bench} --steps 5 --warmup 2\n")
     f.write("averages per dispatch, summed over the chip.  WAVE_CYCLES, ACTIVE_INST_*, WAIT_INST_ANY are in units of 4 cycles per wave;\n")
     f.write("BUSY_CU_CYCLES and VALU_MFMA_BUSY_CYCLES in cycles.  mfma% = VALU_MFMA_BUSY_CYCLES / (duration x 2.4 GHz x 1024 SIMDs);\n")
     f.write("valu% = 4 x ACTIVE_INST_VALU / (same); wait% = WAIT_INST_ANY / WAVE_CYCLES; waves/CU = 4 x WAVE_CYCLES / (duration x 2.4 GHz x 256).\n\n")
