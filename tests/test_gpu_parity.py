@@ -266,3 +266,12 @@ def test_graphed_step_matches_eager(dev):
         for name, a, b in zip(("o", "dq", "dk", "dv"), [out] + grads, ref):
             assert torch.equal(a, b), f"replay {rep}: {name} differs from the eager step"
         eager()                                       # the program's own eager work between replays
+
+
+def test_op_l2_largest_topk_and_odd_shapes(dev):
+    """The largest top-k the selection kernels take (64 fine blocks: 65536 list entries per (b,h) through the one-launch
+    transposes, key blocks with several work items) and a batch x heads that is no power of two with top-k values that
+    are none either."""
+    P.check_op_l2(dev, B=1, H=1, N=16384, T=64, T2=32, fused=True, rope=True)
+    P.check_op_l2(dev, B=3, H=5, N=16384, T=12, T2=20, fused=True, rope=True, smooth=True, slices=[(0, 0), (2, 4)])
+    P.check_op_l1(dev, B=2, H=2, N=4096, T=64, fused=True, rope=True)
